@@ -1,0 +1,154 @@
+/*
+ * sp_aurora_hip.h — C ABI of libsp_aurora_hip.so (gfx950 / MI355X).
+ *
+ * The library holds the attention hot path of sp_aurora as hand-written HIP
+ * kernels: the single-block flash-attention forward that every ring step
+ * calls, the update_out_and_lse merge, the Ulysses head-scatter /
+ * sequence-gather re-layout, and the block-wise backward.  It is the native
+ * plugin that stands where the reference's pybind11/SYCL module
+ * `sp_aurora.sycl_flash_attn` stands (sp_aurora/sycl_bindings/bindings.cpp:316-369),
+ * but speaks plain C: pointers, sizes, strides, a stream handle.
+ *
+ * Conventions shared by every entry point
+ *   - All pointers are DEVICE pointers owned by the caller.  The library
+ *     allocates nothing, frees nothing, and never synchronises: each call
+ *     enqueues kernels on `stream` (a hipStream_t passed as void*; NULL is
+ *     the default stream) and returns.
+ *   - Return value: 0 on success, a negative SPA_E* code on failure; the
+ *     message is available from spa_last_error() (thread-local).  Nothing
+ *     throws.  On failure no kernel has been launched.
+ *   - Strides are in ELEMENTS, given as int64_t[3] = {batch, head, seq}; the
+ *     head-dim stride is always 1.  This one convention covers both the
+ *     reference's public layout [B,S,H,D] (stride = {S*H*D, D, H*D}) and its
+ *     operator layout [B,H,S,D] (stride = {H*S*D, S*D, D}), and the strided
+ *     views qkv[:, :, i] of packed tensors.
+ *   - Data pointers and row starts must be 16-byte aligned (every stride a
+ *     multiple of 8 elements for 16-bit types, 4 for fp32).
+ *   - LSE tensors are fp32, contiguous [B, H, Sq], natural log.
+ *   - `dtype`: SPA_F32 / SPA_BF16 / SPA_F16 = element type of q,k,v,out.
+ *   - Re-entrant; calls on distinct streams may run concurrently.
+ */
+#ifndef SP_AURORA_HIP_H
+#define SP_AURORA_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SPA_ABI_VERSION 1
+
+enum { SPA_F32 = 0, SPA_BF16 = 1, SPA_F16 = 2 };
+
+/* mask_mode of the block operator.  SPA_MASK_CAUSAL is the reference's
+ * top-left aligned `triu(diagonal=1)` mask (sp_aurora/intel_flash_attn.py:79-84):
+ * query row i sees keys j <= i.  A ring step uses it on the diagonal block
+ * pair only (sp_aurora/intel_ring_flash_attn.py:88). */
+enum { SPA_MASK_NONE = 0, SPA_MASK_CAUSAL = 1 };
+
+enum {
+  SPA_OK = 0,
+  SPA_EINVAL = -1,      /* bad argument (null pointer, non-positive size, bad enum) */
+  SPA_EUNSUPPORTED = -2,/* head dim / dtype combination without a kernel */
+  SPA_EALIGN = -3,      /* pointer or stride not 16-byte aligned */
+  SPA_ELAUNCH = -4      /* HIP runtime refused the launch */
+};
+
+/* Library identity.  Replaces `is_available()` / `get_device_info()` of the
+ * reference plugin (sp_aurora/sycl_bindings/bindings.cpp:298-313,357-368). */
+int spa_abi_version(void);
+const char* spa_last_error(void);
+/* Writes a NUL-terminated "name=..;arch=..;cus=..;lds=..;clock_khz=.." line
+ * for the current device into buf (at most n bytes). */
+int spa_device_info(char* buf, int n);
+
+/*
+ * Block attention forward: out = softmax(q k^T * scale + mask) v,
+ * lse = logsumexp(q k^T * scale + mask) over keys, fp32.
+ * Replaces intel_flash_attn_forward / _flash_attn_forward
+ * (sp_aurora/intel_flash_attn.py:18-126,161-163;
+ *  sp_aurora/intel_flash_attn_optimized.py:95-225) and the native
+ * `forward(...)` of the reference plugin (sp_aurora/sycl_bindings/bindings.cpp:50-272).
+ * q: [B,H,Sq,D] by strides, k,v: [B,H,Sk,D] by strides, out: like q.
+ * D in {32, 64, 128}.  scale must be > 0.  Any Sq, Sk >= 1.
+ */
+int spa_flash_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                  int B, int H, int Sq, int Sk, int D,
+                  const int64_t q_strides[3], const int64_t k_strides[3],
+                  const int64_t v_strides[3], const int64_t o_strides[3],
+                  float scale, int mask_mode, int dtype, void* stream);
+
+/*
+ * Merge of one block result into the running (out_acc, lse_acc):
+ *   lse' = logaddexp(lse, lse_b);  out' = out - sigmoid(lse_b - lse) * (out - out_b)
+ * Replaces update_out_and_lse / _update_out_and_lse (sp_aurora/utils.py:47-147).
+ * init != 0 is the first call of a ring (utils.py:116-122): out_acc = float(blk_out),
+ * lse_acc = blk_lse.  out_acc is fp32 [B,H,Sq,D] by acc_strides; lse_acc and
+ * blk_lse are fp32 contiguous [B,H,Sq]; blk_out has element type blk_dtype.
+ * D must be a multiple of 8 (16-bit blocks) or 4 (fp32 blocks).
+ */
+int spa_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* blk_lse,
+              int B, int H, int Sq, int D,
+              const int64_t acc_strides[3], const int64_t blk_strides[3],
+              int blk_dtype, int init, void* stream);
+
+/* out = cast(out_acc) — the `out.to(q.dtype)` that closes a ring forward
+ * (sp_aurora/intel_ring_flash_attn.py:141-143). */
+int spa_finalize(void* out, const float* out_acc,
+                 int B, int H, int Sq, int D,
+                 const int64_t o_strides[3], const int64_t acc_strides[3],
+                 int dtype, void* stream);
+
+/*
+ * Ulysses re-layout, all P ranks' shards stacked on a leading axis of one
+ * device buffer.  `pack` = 1 for a 4-D tensor, 2 / 3 for kv- / qkv-packed
+ * 5-D tensors (the packed axis sits between sequence and heads).
+ *   s2h (scatter heads, gather sequence):
+ *     x [P][B, s, pack, H, D]  ->  y [P][B, P*s, pack, H/P, D]
+ *     y[r][b, q*s+t, c, j, :] = x[q][b, t, c, r*(H/P)+j, :]
+ *   h2s (scatter sequence, gather heads) is its inverse.
+ * Replaces the reshape/transpose/contiguous + all_to_all_single chains of
+ * intel_all_to_all_4d (sp_aurora/intel_ulysses_attn.py:60-143),
+ * all_to_all_4D and all_to_all_5D (sp_aurora/comm/all_to_all.py:17-180,228-335).
+ * elem_bytes in {1,2,4,8}; H must be divisible by P.  Pure byte movement.
+ */
+int spa_relayout_s2h(const void* x, void* y, int P, int B, int s, int H, int D,
+                     int pack, int elem_bytes, void* stream);
+int spa_relayout_h2s(const void* y, void* x, int P, int B, int s, int H, int D,
+                     int pack, int elem_bytes, void* stream);
+
+/*
+ * delta[b,h,i] = sum_d dout[b,h,i,d] * out[b,h,i,d]   (fp32, [B,H,Sq] contiguous)
+ * First pass of the block-wise backward; the reference obtains the same term
+ * implicitly through autograd (sp_aurora/intel_ring_flash_attn.py:229-244).
+ */
+int spa_bwd_delta(const void* out, const void* dout, float* delta,
+                  int B, int H, int Sq, int D,
+                  const int64_t o_strides[3], const int64_t do_strides[3],
+                  int dtype, void* stream);
+
+/*
+ * Block-wise backward of one (q chunk, kv chunk) pair with the GLOBAL lse
+ * and delta of the q chunk's rows:
+ *   P = exp(q k^T * scale + mask - lse);  dV += P^T dO;  dP = dO V^T;
+ *   dS = P * (dP - delta);  dQ += dS K * scale;  dK += dS^T Q * scale.
+ * dq_acc [B,H,Sq,D], dk_acc / dv_acc [B,H,Sk,D]: fp32, ACCUMULATED into (the
+ * caller zeroes them before the first block pair of a chunk); strides as given.
+ * Replaces the per-step body of intel_ring_flash_attn_backward
+ * (sp_aurora/intel_ring_flash_attn.py:192-258).
+ */
+int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout,
+                  const float* lse, const float* delta,
+                  float* dq_acc, float* dk_acc, float* dv_acc,
+                  int B, int H, int Sq, int Sk, int D,
+                  const int64_t q_strides[3], const int64_t k_strides[3],
+                  const int64_t v_strides[3], const int64_t do_strides[3],
+                  const int64_t dq_strides[3], const int64_t dk_strides[3],
+                  const int64_t dv_strides[3],
+                  float scale, int mask_mode, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SP_AURORA_HIP_H */

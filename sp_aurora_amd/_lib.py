@@ -1,0 +1,79 @@
+"""ctypes binding of libsp_aurora_hip.so — the only way this package reaches the GPU kernels.
+
+The library must have been built (``python -m sp_aurora_amd.build``); there is no
+fallback path: a missing library raises, it never degrades to torch ops.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libsp_aurora_hip.so")
+
+SPA_F32, SPA_BF16, SPA_F16 = 0, 1, 2
+SPA_MASK_NONE, SPA_MASK_CAUSAL = 0, 1
+
+_I64x3 = ctypes.c_int64 * 3
+_vp = ctypes.c_void_p
+_i = ctypes.c_int
+_f = ctypes.c_float
+_s3 = ctypes.POINTER(ctypes.c_int64)
+
+# name -> (restype, argtypes); mirrors include/sp_aurora_hip.h declaration by declaration
+SIGNATURES = {
+    "spa_abi_version": (_i, []),
+    "spa_last_error": (ctypes.c_char_p, []),
+    "spa_device_info": (_i, [ctypes.c_char_p, _i]),
+    "spa_flash_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _vp]),
+    "spa_merge": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _s3, _s3, _i, _i, _vp]),
+    "spa_finalize": (_i, [_vp, _vp, _i, _i, _i, _i, _s3, _s3, _i, _vp]),
+    "spa_relayout_s2h": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "spa_relayout_h2s": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "spa_bwd_delta": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _s3, _s3, _i, _vp]),
+    "spa_flash_bwd": (_i, [_vp] * 9 + [_i] * 5 + [_s3] * 7 + [_f, _i, _i, _vp]),
+}
+
+_lib = None
+
+
+class SpaError(RuntimeError):
+    """A negative return code from the C ABI; .code holds it."""
+
+    def __init__(self, code, msg):
+        super().__init__(f"[spa {code}] {msg}")
+        self.code = code
+
+
+def load():
+    """Load the shared library once and attach the prototypes.  Raises if it was not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} not found: build it with `python -m sp_aurora_amd.build` "
+            "(sp_aurora_amd has no non-HIP path)"
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    if lib.spa_abi_version() != 1:
+        raise ImportError(f"{LIB_PATH}: ABI version {lib.spa_abi_version()} != 1")
+    _lib = lib
+    return lib
+
+
+def strides3(vals):
+    return _I64x3(*[int(v) for v in vals])
+
+
+def check(code):
+    if code != 0:
+        raise SpaError(code, load().spa_last_error().decode("utf-8", "replace"))
+
+
+def device_info():
+    buf = ctypes.create_string_buffer(512)
+    check(load().spa_device_info(buf, 512))
+    return dict(kv.split("=", 1) for kv in buf.value.decode().split(";"))

@@ -1,0 +1,44 @@
+"""Builds libsp_aurora_hip.so (the C-ABI library with the gfx950 kernels) in-tree with hipcc.
+
+Usage:  python -m sp_aurora_amd.build        (cross-compiles; no GPU needed)
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_NAME = "libsp_aurora_hip.so"
+LIB_PATH = os.path.join(HERE, LIB_NAME)
+SOURCES = ["spa_abi.hip", "flash_fwd.hip", "flash_bwd.hip", "merge.hip", "relayout.hip"]
+FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    # packed fp32 VALU ops are kept off on purpose (scalar fp32 code only)
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def build(verbose: bool = True) -> str:
+    """Compile every HIP source into sp_aurora_amd/libsp_aurora_hip.so and return its path."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    if not os.path.exists(hipcc):
+        hipcc = "hipcc"
+    cmd = [hipcc] + FLAGS + ["-o", LIB_PATH] + [os.path.join(CSRC, s) for s in SOURCES]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l and l.strip())
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + out)
+    if verbose and out:
+        print(out)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()
+    sys.exit(0)

@@ -1,0 +1,210 @@
+// extern "C" boundary of libsp_aurora_hip.so: argument checks, then a launch.
+// No allocation, no synchronisation, no torch types; errors are codes plus a
+// thread-local message.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/sp_aurora_hip.h"
+#include "spa_common.h"
+
+hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream);
+hipError_t spa_launch_flash_bwd(BwdParams p, int D, int dtype, hipStream_t stream);
+hipError_t spa_launch_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* blk_lse, int B,
+                            int H, int Sq, int D, Strides3 as, Strides3 bs, int dtype, int init,
+                            hipStream_t stream);
+hipError_t spa_launch_finalize(void* out, const float* out_acc, int B, int H, int Sq, int D, Strides3 os,
+                               Strides3 as, int dtype, hipStream_t stream);
+hipError_t spa_launch_delta(const void* out, const void* dout, float* delta, int B, int H, int Sq, int D,
+                            Strides3 os, Strides3 ds, int dtype, hipStream_t stream);
+hipError_t spa_launch_relayout(const void* src, void* dst, int P, int B, int s, int H, int D, int pack,
+                               int elem_bytes, bool s2h, hipStream_t stream);
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int elem_size(int dtype) { return dtype == SPA_F32 ? 4 : 2; }
+
+bool dtype_ok(int dtype) { return dtype == SPA_F32 || dtype == SPA_BF16 || dtype == SPA_F16; }
+
+Strides3 S3(const int64_t* s) {
+  Strides3 r;
+  r.b = s[0]; r.h = s[1]; r.s = s[2];
+  return r;
+}
+
+// 16-byte alignment of the base pointer and of every row start.
+bool aligned16(const void* p, const int64_t* s, int esz) {
+  if (((uintptr_t)p & 15) != 0) return false;
+  for (int i = 0; i < 3; ++i)
+    if ((s[i] * esz) % 16 != 0) return false;
+  return true;
+}
+
+// The largest element offset a (B,H,S,D) view touches must fit what the kernels index.
+bool dims_ok(int B, int H, int S, int D) { return B > 0 && H > 0 && S > 0 && D > 0; }
+
+bool pow2_8_512(int D) { return D >= 8 && D <= 512 && (D & (D - 1)) == 0; }
+
+int launch_result(hipError_t e, const char* what) {
+  if (e == hipSuccess) return SPA_OK;
+  if (e == hipErrorInvalidValue) return fail(SPA_EUNSUPPORTED, "%s: no kernel for this head dim / dtype", what);
+  return fail(SPA_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+}
+
+}  // namespace
+
+extern "C" {
+
+int spa_abi_version(void) { return SPA_ABI_VERSION; }
+
+const char* spa_last_error(void) { return g_err; }
+
+int spa_device_info(char* buf, int n) {
+  if (!buf || n <= 0) return fail(SPA_EINVAL, "spa_device_info: null buffer");
+  int dev = 0;
+  hipDeviceProp_t prop;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess) e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) return fail(SPA_ELAUNCH, "spa_device_info: %s", hipGetErrorString(e));
+  snprintf(buf, n, "name=%s;arch=%s;cus=%d;lds=%zu;clock_khz=%d;mem_clock_khz=%d;bus_bits=%d;hbm=%zu", prop.name,
+           prop.gcnArchName, prop.multiProcessorCount, prop.maxSharedMemoryPerMultiProcessor, prop.clockRate,
+           prop.memoryClockRate, prop.memoryBusWidth, prop.totalGlobalMem);
+  return SPA_OK;
+}
+
+int spa_flash_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int B, int H, int Sq,
+                  int Sk, int D, const int64_t q_strides[3], const int64_t k_strides[3],
+                  const int64_t v_strides[3], const int64_t o_strides[3], float scale, int mask_mode,
+                  int dtype, void* stream) {
+  if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "spa_flash_fwd: null pointer");
+  if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(SPA_EINVAL, "spa_flash_fwd: null strides");
+  if (!dims_ok(B, H, Sq, D) || Sk <= 0) return fail(SPA_EINVAL, "spa_flash_fwd: sizes must be positive (B=%d H=%d Sq=%d Sk=%d D=%d)", B, H, Sq, Sk, D);
+  if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "spa_flash_fwd: bad dtype %d", dtype);
+  if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "spa_flash_fwd: bad mask_mode %d", mask_mode);
+  if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "spa_flash_fwd: softmax scale must be positive and finite");
+  if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "spa_flash_fwd: head dim %d not in {32,64,128}", D);
+  const int esz = elem_size(dtype);
+  if (!aligned16(q, q_strides, esz) || !aligned16(k, k_strides, esz) || !aligned16(v, v_strides, esz) ||
+      !aligned16(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0)
+    return fail(SPA_EALIGN, "spa_flash_fwd: pointers and row strides must be 16-byte aligned");
+  if ((int64_t)B * H * ((Sq + 127) / 128) > 0x7fffffffLL) return fail(SPA_EINVAL, "spa_flash_fwd: grid too large");
+  FwdParams p;
+  p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
+  p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
+  p.qs = S3(q_strides); p.ks = S3(k_strides); p.vs = S3(v_strides); p.os = S3(o_strides);
+  p.scale = scale;
+  p.scale_log2 = scale * 1.4426950408889634f;
+  p.causal = mask_mode == SPA_MASK_CAUSAL;
+  p.nqt = 0;
+  return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), "spa_flash_fwd");
+}
+
+int spa_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* blk_lse, int B, int H, int Sq,
+              int D, const int64_t acc_strides[3], const int64_t blk_strides[3], int blk_dtype, int init,
+              void* stream) {
+  if (!out_acc || !lse_acc || !blk_out || !blk_lse || !acc_strides || !blk_strides)
+    return fail(SPA_EINVAL, "spa_merge: null pointer");
+  if (!dims_ok(B, H, Sq, D)) return fail(SPA_EINVAL, "spa_merge: sizes must be positive");
+  if (!dtype_ok(blk_dtype)) return fail(SPA_EINVAL, "spa_merge: bad dtype %d", blk_dtype);
+  if (!pow2_8_512(D)) return fail(SPA_EUNSUPPORTED, "spa_merge: head dim %d must be a power of two in [8,512]", D);
+  if (!aligned16(out_acc, acc_strides, 4) || !aligned16(blk_out, blk_strides, elem_size(blk_dtype)))
+    return fail(SPA_EALIGN, "spa_merge: pointers and row strides must be 16-byte aligned");
+  if ((int64_t)B * H * Sq * (D / 8) / 256 > 0x7ffffff0LL) return fail(SPA_EINVAL, "spa_merge: grid too large");
+  return launch_result(spa_launch_merge(out_acc, lse_acc, blk_out, blk_lse, B, H, Sq, D, S3(acc_strides),
+                                        S3(blk_strides), blk_dtype, init, (hipStream_t)stream),
+                       "spa_merge");
+}
+
+int spa_finalize(void* out, const float* out_acc, int B, int H, int Sq, int D, const int64_t o_strides[3],
+                 const int64_t acc_strides[3], int dtype, void* stream) {
+  if (!out || !out_acc || !o_strides || !acc_strides) return fail(SPA_EINVAL, "spa_finalize: null pointer");
+  if (!dims_ok(B, H, Sq, D)) return fail(SPA_EINVAL, "spa_finalize: sizes must be positive");
+  if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "spa_finalize: bad dtype %d", dtype);
+  if (!pow2_8_512(D)) return fail(SPA_EUNSUPPORTED, "spa_finalize: head dim %d must be a power of two in [8,512]", D);
+  if (!aligned16(out_acc, acc_strides, 4) || !aligned16(out, o_strides, elem_size(dtype)))
+    return fail(SPA_EALIGN, "spa_finalize: pointers and row strides must be 16-byte aligned");
+  if ((int64_t)B * H * Sq * (D / 8) / 256 > 0x7ffffff0LL) return fail(SPA_EINVAL, "spa_finalize: grid too large");
+  return launch_result(spa_launch_finalize(out, out_acc, B, H, Sq, D, S3(o_strides), S3(acc_strides), dtype,
+                                           (hipStream_t)stream),
+                       "spa_finalize");
+}
+
+static int relayout(const void* src, void* dst, int P, int B, int s, int H, int D, int pack, int elem_bytes,
+                    bool s2h, void* stream, const char* what) {
+  if (!src || !dst) return fail(SPA_EINVAL, "%s: null pointer", what);
+  if (P <= 0 || B <= 0 || s <= 0 || H <= 0 || D <= 0) return fail(SPA_EINVAL, "%s: sizes must be positive", what);
+  if (pack < 1 || pack > 3) return fail(SPA_EINVAL, "%s: pack must be 1, 2 or 3", what);
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)
+    return fail(SPA_EINVAL, "%s: elem_bytes must be 1, 2, 4 or 8", what);
+  if (H % P != 0) return fail(SPA_EINVAL, "%s: heads (%d) not divisible by ranks (%d)", what, H, P);
+  if (src == dst) return fail(SPA_EINVAL, "%s: in-place re-layout is not supported", what);
+  return launch_result(spa_launch_relayout(src, dst, P, B, s, H, D, pack, elem_bytes, s2h, (hipStream_t)stream), what);
+}
+
+int spa_relayout_s2h(const void* x, void* y, int P, int B, int s, int H, int D, int pack, int elem_bytes,
+                     void* stream) {
+  return relayout(x, y, P, B, s, H, D, pack, elem_bytes, true, stream, "spa_relayout_s2h");
+}
+
+int spa_relayout_h2s(const void* y, void* x, int P, int B, int s, int H, int D, int pack, int elem_bytes,
+                     void* stream) {
+  return relayout(y, x, P, B, s, H, D, pack, elem_bytes, false, stream, "spa_relayout_h2s");
+}
+
+int spa_bwd_delta(const void* out, const void* dout, float* delta, int B, int H, int Sq, int D,
+                  const int64_t o_strides[3], const int64_t do_strides[3], int dtype, void* stream) {
+  if (!out || !dout || !delta || !o_strides || !do_strides) return fail(SPA_EINVAL, "spa_bwd_delta: null pointer");
+  if (!dims_ok(B, H, Sq, D)) return fail(SPA_EINVAL, "spa_bwd_delta: sizes must be positive");
+  if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "spa_bwd_delta: bad dtype %d", dtype);
+  if (!pow2_8_512(D)) return fail(SPA_EUNSUPPORTED, "spa_bwd_delta: head dim %d must be a power of two in [8,512]", D);
+  const int esz = elem_size(dtype);
+  if (!aligned16(out, o_strides, esz) || !aligned16(dout, do_strides, esz))
+    return fail(SPA_EALIGN, "spa_bwd_delta: pointers and row strides must be 16-byte aligned");
+  return launch_result(spa_launch_delta(out, dout, delta, B, H, Sq, D, S3(o_strides), S3(do_strides), dtype,
+                                        (hipStream_t)stream),
+                       "spa_bwd_delta");
+}
+
+int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                  const float* delta, float* dq_acc, float* dk_acc, float* dv_acc, int B, int H, int Sq, int Sk,
+                  int D, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                  const int64_t do_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                  const int64_t dv_strides[3], float scale, int mask_mode, int dtype, void* stream) {
+  if (!q || !k || !v || !dout || !lse || !delta || !dq_acc || !dk_acc || !dv_acc)
+    return fail(SPA_EINVAL, "spa_flash_bwd: null pointer");
+  if (!q_strides || !k_strides || !v_strides || !do_strides || !dq_strides || !dk_strides || !dv_strides)
+    return fail(SPA_EINVAL, "spa_flash_bwd: null strides");
+  if (!dims_ok(B, H, Sq, D) || Sk <= 0) return fail(SPA_EINVAL, "spa_flash_bwd: sizes must be positive");
+  if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "spa_flash_bwd: bad dtype %d", dtype);
+  if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "spa_flash_bwd: bad mask_mode %d", mask_mode);
+  if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "spa_flash_bwd: softmax scale must be positive and finite");
+  if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "spa_flash_bwd: head dim %d not in {32,64,128}", D);
+  const int esz = elem_size(dtype);
+  if (!aligned16(q, q_strides, esz) || !aligned16(k, k_strides, esz) || !aligned16(v, v_strides, esz) ||
+      !aligned16(dout, do_strides, esz) || !aligned16(dq_acc, dq_strides, 4) || !aligned16(dk_acc, dk_strides, 4) ||
+      !aligned16(dv_acc, dv_strides, 4))
+    return fail(SPA_EALIGN, "spa_flash_bwd: pointers and row strides must be 16-byte aligned");
+  BwdParams p;
+  p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta;
+  p.dq = dq_acc; p.dk = dk_acc; p.dv = dv_acc;
+  p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
+  p.qs = S3(q_strides); p.ks = S3(k_strides); p.vs = S3(v_strides); p.dos = S3(do_strides);
+  p.dqs = S3(dq_strides); p.dks = S3(dk_strides); p.dvs = S3(dv_strides);
+  p.scale = scale;
+  p.scale_log2 = scale * 1.4426950408889634f;
+  p.causal = mask_mode == SPA_MASK_CAUSAL;
+  p.nkt = 0;
+  return launch_result(spa_launch_flash_bwd(p, D, dtype, (hipStream_t)stream), "spa_flash_bwd");
+}
+
+}  // extern "C"

@@ -1,0 +1,106 @@
+// Shared device-side types and helpers for the sp_aurora HIP kernels (gfx950).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+struct Strides3 {
+  int64_t b, h, s;  // element strides of (batch, head, seq); head-dim stride is 1
+};
+
+struct FwdParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  float* lse;
+  int B, H, Sq, Sk;
+  Strides3 qs, ks, vs, os;
+  float scale;       // softmax scale
+  float scale_log2;  // scale * log2(e)
+  int causal;        // 1: query row i sees keys j <= i (top-left aligned)
+  int nqt;           // number of query tiles per (batch, head)
+};
+
+struct BwdParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* dout;
+  const float* lse;
+  const float* delta;
+  float* dq;
+  float* dk;
+  float* dv;
+  int B, H, Sq, Sk;
+  Strides3 qs, ks, vs, dos, dqs, dks, dvs;
+  float scale;
+  float scale_log2;
+  int causal;
+  int nkt;  // number of key tiles per (batch, head)
+};
+
+// 16-bit element traits: MFMA 32x32x16 with 8 elements per lane per operand.
+template <typename T>
+struct Mma16;
+
+template <>
+struct Mma16<__bf16> {
+  typedef bf16x8 frag;
+  static __device__ __forceinline__ f32x16 run(frag a, frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ frag pack(float x0, float x1, float x2, float x3,
+                                              float x4, float x5, float x6, float x7) {
+    frag r;
+    r[0] = (__bf16)x0; r[1] = (__bf16)x1; r[2] = (__bf16)x2; r[3] = (__bf16)x3;
+    r[4] = (__bf16)x4; r[5] = (__bf16)x5; r[6] = (__bf16)x6; r[7] = (__bf16)x7;
+    return r;
+  }
+  static __device__ __forceinline__ unsigned pack2(float lo, float hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    bf16x2 r;
+    r[0] = (__bf16)lo; r[1] = (__bf16)hi;
+    return __builtin_bit_cast(unsigned, r);
+  }
+};
+
+template <>
+struct Mma16<_Float16> {
+  typedef f16x8 frag;
+  static __device__ __forceinline__ f32x16 run(frag a, frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ frag pack(float x0, float x1, float x2, float x3,
+                                              float x4, float x5, float x6, float x7) {
+    frag r;
+    r[0] = (_Float16)x0; r[1] = (_Float16)x1; r[2] = (_Float16)x2; r[3] = (_Float16)x3;
+    r[4] = (_Float16)x4; r[5] = (_Float16)x5; r[6] = (_Float16)x6; r[7] = (_Float16)x7;
+    return r;
+  }
+  static __device__ __forceinline__ unsigned pack2(float lo, float hi) {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    f16x2 r;
+    r[0] = (_Float16)lo; r[1] = (_Float16)hi;
+    return __builtin_bit_cast(unsigned, r);
+  }
+};
+
+template <typename F>
+static __device__ __forceinline__ F as_frag(u32x4 x) {
+  return __builtin_bit_cast(F, x);
+}
+
+// Exchange with the lane 32 away (the other half of the wavefront).
+static __device__ __forceinline__ float xhalf(float x) {
+  return __shfl_xor(x, 32, 64);
+}
+
+static __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+static __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }

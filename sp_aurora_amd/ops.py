@@ -1,0 +1,195 @@
+"""Tensor-level wrappers over the C ABI: torch is used for device memory and streams only.
+
+Every function takes tensors in either the reference's public layout ``"bshd"``
+([B,S,H,D], sp_aurora/intel_ring_flash_attn.py:399-435) or its operator layout
+``"bhsd"`` ([B,H,S,D], sp_aurora/intel_flash_attn.py:56); both reach the same
+kernels through (batch, head, seq) strides, so no transposes or copies are made.
+"""
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: _lib.SPA_F32, torch.bfloat16: _lib.SPA_BF16, torch.float16: _lib.SPA_F16}
+
+
+def _dtype_code(t):
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}; expected float32, bfloat16 or float16") from None
+
+
+def _bhs(t, layout):
+    """(B, H, S, D) sizes and (batch, head, seq) element strides of a 4-D view."""
+    if t.dim() != 4:
+        raise ValueError(f"expected a 4-D tensor, got {tuple(t.shape)}")
+    st = t.stride()
+    if layout == "bshd":
+        B, S, H, D = t.shape
+        return (B, H, S, D), (st[0], st[2], st[1])
+    if layout == "bhsd":
+        B, H, S, D = t.shape
+        return (B, H, S, D), (st[0], st[1], st[2])
+    raise ValueError(f"layout must be 'bshd' or 'bhsd', got {layout!r}")
+
+
+def _rows_ok(t, esz):
+    return t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all((s * esz) % 16 == 0 for s in t.stride()[:-1])
+
+
+def _prep(t):
+    """A view the kernels can read as is, else a compact copy (inner stride 1, 16-byte rows)."""
+    if not t.is_cuda:
+        raise ValueError("sp_aurora_amd kernels need tensors on a HIP device (got a CPU tensor)")
+    return t if _rows_ok(t, t.element_size()) else t.contiguous()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None, lse=None):
+    """Block attention forward -> (out like q, lse fp32 [B,H,Sq]).  Calls spa_flash_fwd."""
+    lib = _lib.load()
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise TypeError("q, k, v must share a dtype")
+    (B, H, Sq, D), qs = _bhs(q, layout)
+    (Bk, Hk, Sk, Dk), ks = _bhs(k, layout)
+    (Bv, Hv, Sv, Dv), vs = _bhs(v, layout)
+    if (Bk, Hk, Dk) != (B, H, D) or (Bv, Hv, Sv, Dv) != (Bk, Hk, Sk, Dk):
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    if softmax_scale is None:
+        softmax_scale = D ** (-0.5)
+    if out is None:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    if lse is None:
+        lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    _, os_ = _bhs(out, layout)
+    with torch.cuda.device(q.device):
+        _lib.check(lib.spa_flash_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            B, H, Sq, Sk, D,
+            _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
+            float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE,
+            _dtype_code(q), _stream()))
+    return out, lse
+
+
+def merge(out_acc, lse_acc, blk_out, blk_lse, layout="bshd", init=False):
+    """In-place merge of (blk_out, blk_lse) into fp32 (out_acc, lse_acc).  Calls spa_merge."""
+    lib = _lib.load()
+    blk_out = _prep(blk_out)
+    (B, H, Sq, D), as_ = _bhs(out_acc, layout)
+    shp, bs = _bhs(blk_out, layout)
+    if shp != (B, H, Sq, D) or tuple(lse_acc.shape) != (B, H, Sq) or tuple(blk_lse.shape) != (B, H, Sq):
+        raise ValueError("merge: shape mismatch")
+    if out_acc.dtype != torch.float32 or lse_acc.dtype != torch.float32 or blk_lse.dtype != torch.float32:
+        raise TypeError("merge: accumulators and lse must be float32")
+    if not (lse_acc.is_contiguous() and blk_lse.is_contiguous() and _rows_ok(out_acc, 4)):
+        raise ValueError("merge: lse tensors must be contiguous and out_acc 16-byte aligned")
+    with torch.cuda.device(out_acc.device):
+        _lib.check(lib.spa_merge(
+            out_acc.data_ptr(), lse_acc.data_ptr(), blk_out.data_ptr(), blk_lse.data_ptr(),
+            B, H, Sq, D, _lib.strides3(as_), _lib.strides3(bs), _dtype_code(blk_out),
+            1 if init else 0, _stream()))
+    return out_acc, lse_acc
+
+
+def finalize(out_acc, dtype, layout="bshd", out=None):
+    """out = out_acc.to(dtype) through spa_finalize."""
+    lib = _lib.load()
+    (B, H, Sq, D), as_ = _bhs(out_acc, layout)
+    if out is None:
+        out = torch.empty(out_acc.shape, dtype=dtype, device=out_acc.device)
+    _, os_ = _bhs(out, layout)
+    with torch.cuda.device(out_acc.device):
+        _lib.check(lib.spa_finalize(out.data_ptr(), out_acc.data_ptr(), B, H, Sq, D,
+                                    _lib.strides3(os_), _lib.strides3(as_), _dtype_code(out), _stream()))
+    return out
+
+
+def _relayout(x, P, s2h, out=None):
+    """x: [P, B, s, (pack,) H, D] (s2h) or [P, B, P*s, (pack,) H/P, D] (h2s), contiguous."""
+    lib = _lib.load()
+    if x.dim() not in (5, 6):
+        raise ValueError(f"expected [P,B,S,H,D] or [P,B,S,pack,H,D], got {tuple(x.shape)}")
+    if not x.is_cuda:
+        raise ValueError("sp_aurora_amd kernels need tensors on a HIP device (got a CPU tensor)")
+    x = x.contiguous()
+    pack = x.shape[3] if x.dim() == 6 else 1
+    if x.shape[0] != P:
+        raise ValueError(f"leading axis {x.shape[0]} != P={P}")
+    B, S_in, H_in, D = x.shape[1], x.shape[2], x.shape[-2], x.shape[-1]
+    if s2h:
+        if H_in % P:
+            raise ValueError(f"heads ({H_in}) not divisible by P={P}")
+        s, H = S_in, H_in
+        oshape = (P, B, P * s) + ((pack,) if x.dim() == 6 else ()) + (H // P, D)
+    else:
+        if S_in % P:
+            raise ValueError(f"sequence ({S_in}) not divisible by P={P}")
+        s, H = S_in // P, H_in * P
+        oshape = (P, B, s) + ((pack,) if x.dim() == 6 else ()) + (H, D)
+    if out is None:
+        out = torch.empty(oshape, dtype=x.dtype, device=x.device)
+    fn = lib.spa_relayout_s2h if s2h else lib.spa_relayout_h2s
+    with torch.cuda.device(x.device):
+        _lib.check(fn(x.data_ptr(), out.data_ptr(), P, B, s, H, D, pack, x.element_size(), _stream()))
+    return out
+
+
+def relayout_s2h(x, P, out=None):
+    """Sequence-sharded [P][B,s,(pack,)H,D] -> head-sharded [P][B,P*s,(pack,)H/P,D]."""
+    return _relayout(x, P, True, out)
+
+
+def relayout_h2s(y, P, out=None):
+    """Head-sharded [P][B,P*s,(pack,)H/P,D] -> sequence-sharded [P][B,s,(pack,)H,D]."""
+    return _relayout(y, P, False, out)
+
+
+def bwd_delta(out, dout, layout="bshd"):
+    """delta = rowsum(dout * out), fp32 [B,H,Sq].  Calls spa_bwd_delta."""
+    lib = _lib.load()
+    out, dout = _prep(out), _prep(dout)
+    (B, H, Sq, D), os_ = _bhs(out, layout)
+    shp, ds = _bhs(dout, layout)
+    if shp != (B, H, Sq, D) or out.dtype != dout.dtype:
+        raise ValueError("bwd_delta: out and dout must match in shape and dtype")
+    delta = torch.empty((B, H, Sq), dtype=torch.float32, device=out.device)
+    with torch.cuda.device(out.device):
+        _lib.check(lib.spa_bwd_delta(out.data_ptr(), dout.data_ptr(), delta.data_ptr(), B, H, Sq, D,
+                                     _lib.strides3(os_), _lib.strides3(ds), _dtype_code(out), _stream()))
+    return delta
+
+
+def flash_bwd(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, softmax_scale=None, causal=False,
+              layout="bshd"):
+    """Block-wise backward of one (q chunk, kv chunk) pair; adds into fp32 dq/dk/dv accumulators."""
+    lib = _lib.load()
+    q, k, v, dout = _prep(q), _prep(k), _prep(v), _prep(dout)
+    (B, H, Sq, D), qs = _bhs(q, layout)
+    (_, _, Sk, _), ks = _bhs(k, layout)
+    _, vs = _bhs(v, layout)
+    _, dos = _bhs(dout, layout)
+    _, dqs = _bhs(dq_acc, layout)
+    _, dks = _bhs(dk_acc, layout)
+    _, dvs = _bhs(dv_acc, layout)
+    if softmax_scale is None:
+        softmax_scale = D ** (-0.5)
+    for t in (dq_acc, dk_acc, dv_acc, lse, delta):
+        if t.dtype != torch.float32:
+            raise TypeError("flash_bwd: accumulators, lse and delta must be float32")
+    if not (lse.is_contiguous() and delta.is_contiguous()):
+        raise ValueError("flash_bwd: lse and delta must be contiguous [B,H,Sq]")
+    with torch.cuda.device(q.device):
+        _lib.check(lib.spa_flash_bwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            dq_acc.data_ptr(), dk_acc.data_ptr(), dv_acc.data_ptr(),
+            B, H, Sq, Sk, D,
+            _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(dos),
+            _lib.strides3(dqs), _lib.strides3(dks), _lib.strides3(dvs),
+            float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE,
+            _dtype_code(q), _stream()))
+    return dq_acc, dk_acc, dv_acc
