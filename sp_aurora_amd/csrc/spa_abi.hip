@@ -203,6 +203,7 @@ int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout,
   p.scale = scale;
   p.scale_log2 = scale * 1.4426950408889634f;
   p.causal = mask_mode == SPA_MASK_CAUSAL;
+  p.nqt = 0;
   p.nkt = 0;
   return launch_result(spa_launch_flash_bwd(p, D, dtype, (hipStream_t)stream), "spa_flash_bwd");
 }

@@ -43,6 +43,7 @@ struct BwdParams {
   float scale;
   float scale_log2;
   int causal;
+  int nqt;  // number of query tiles per (batch, head)
   int nkt;  // number of key tiles per (batch, head)
 };
 

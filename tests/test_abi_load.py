@@ -1,0 +1,117 @@
+"""CPU-side checks of the drop-in boundary: the library loads without a GPU, exports exactly
+what include/sp_aurora_hip.h declares, and its argument checks answer with codes, not crashes."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from sp_aurora_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "sp_aurora_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(spa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    assert declared_symbols() == sorted(_lib.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+
+
+def test_abi_version_and_error_string():
+    lib = _lib.load()
+    assert lib.spa_abi_version() == 1
+    assert isinstance(lib.spa_last_error(), bytes)
+
+
+def _s3(*v):
+    return _lib.strides3(v)
+
+
+def test_bad_arguments_return_codes_without_touching_a_device():
+    lib = _lib.load()
+    st = _s3(64, 64, 64)
+    # null pointers
+    assert lib.spa_flash_fwd(None, None, None, None, None, 1, 1, 8, 8, 64, st, st, st, st, 1.0, 0, 1, None) == -1
+    assert b"null" in lib.spa_last_error()
+    p = ctypes.c_void_p(4096)  # aligned, never dereferenced: every check below fails before a launch
+    # unsupported head dim
+    assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 8, 8, 48, st, st, st, st, 1.0, 0, 1, None) == -2
+    # non-positive scale
+    assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 8, 8, 64, st, st, st, st, 0.0, 0, 1, None) == -1
+    # bad dtype / mask
+    assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 8, 8, 64, st, st, st, st, 1.0, 0, 7, None) == -1
+    assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 8, 8, 64, st, st, st, st, 1.0, 5, 1, None) == -1
+    # misaligned pointer / stride
+    assert lib.spa_flash_fwd(ctypes.c_void_p(4098), p, p, p, p, 1, 1, 8, 8, 64, st, st, st, st, 1.0, 0, 1, None) == -3
+    assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 8, 8, 64, _s3(63, 63, 63), st, st, st, 1.0, 0, 1, None) == -3
+    # sizes
+    assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 0, 8, 64, st, st, st, st, 1.0, 0, 1, None) == -1
+    # merge: head dim must be a power of two
+    assert lib.spa_merge(p, p, p, p, 1, 1, 8, 24, st, st, 1, 0, None) == -2
+    # relayout: heads not divisible, in place, bad pack
+    assert lib.spa_relayout_s2h(p, ctypes.c_void_p(8192), 3, 1, 4, 8, 16, 1, 2, None) == -1
+    assert lib.spa_relayout_s2h(p, p, 2, 1, 4, 8, 16, 1, 2, None) == -1
+    assert lib.spa_relayout_h2s(p, ctypes.c_void_p(8192), 2, 1, 4, 8, 16, 4, 2, None) == -1
+    # backward: fp32 has no kernel
+    f = ctypes.c_void_p(4096)
+    args = [f] * 9 + [1, 1, 8, 8, 64] + [st] * 7
+    assert lib.spa_flash_bwd(*args, 1.0, 0, 9, None) == -1
+
+
+def test_python_wrappers_refuse_cpu_tensors():
+    import torch
+    from sp_aurora_amd import ops
+    q = torch.zeros(1, 8, 1, 64)
+    with pytest.raises(ValueError, match="HIP device"):
+        ops.flash_fwd(q, q, q)
+
+
+def test_public_signatures_match_the_reference():
+    """Argument names and defaults of sp_aurora/intel_ring_flash_attn.py:344-411 and
+    sp_aurora/intel_ulysses_attn.py:501-513, plus the keyword-only ring_size extension."""
+    import inspect
+    import sp_aurora_amd as spa
+    base = ["dropout_p", "softmax_scale", "causal", "window_size", "alibi_slopes", "deterministic",
+            "return_attn_probs", "group"]
+    for fn, head in ((spa.ring_flash_attn_func, ["q", "k", "v"]), (spa.ring_flash_attn_kvpacked_func, ["q", "kv"]),
+                     (spa.ring_flash_attn_qkvpacked_func, ["qkv"])):
+        sig = inspect.signature(fn)
+        names = list(sig.parameters)
+        assert names == head + base + ["ring_size"]
+        assert sig.parameters["ring_size"].kind is inspect.Parameter.KEYWORD_ONLY
+        assert sig.parameters["dropout_p"].default == 0.0
+        assert sig.parameters["causal"].default is False
+        assert sig.parameters["window_size"].default == (-1, -1)
+    assert spa.sp_aurora_func is spa.ring_flash_attn_func is spa.intel_ring_flash_attn_func
+    assert spa.sp_aurora_kvpacked_func is spa.ring_flash_attn_kvpacked_func
+    assert spa.sp_aurora_qkvpacked_func is spa.ring_flash_attn_qkvpacked_func
+    assert list(inspect.signature(spa.ulysses_flash_attn_func).parameters) == ["q", "k", "v"] + base
+    assert list(inspect.signature(spa.intel_all_to_all_4d).parameters) == ["input", "scatter_idx", "gather_idx", "group"]
+    assert list(inspect.signature(spa.update_out_and_lse).parameters) == ["out", "lse", "block_out", "block_lse", "slice_"]
+    fwd = list(inspect.signature(spa._flash_attn_forward).parameters)
+    assert fwd[:9] == ["q", "k", "v", "dropout_p", "softmax_scale", "causal", "window_size", "alibi_slopes", "return_softmax"]
+
+
+def test_unsupported_features_raise_before_any_launch():
+    import torch
+    import sp_aurora_amd as spa
+    q = torch.zeros(1, 8, 1, 64)
+    with pytest.raises(NotImplementedError):
+        spa.ring_flash_attn_func(q, q, q, dropout_p=0.1)
+    with pytest.raises(NotImplementedError):
+        spa.ring_flash_attn_func(q, q, q, window_size=(4, 0))
+    with pytest.raises(AssertionError):
+        spa.ring_flash_attn_func(q, q, q, alibi_slopes=torch.zeros(1))
+    with pytest.raises(NotImplementedError):
+        spa.ring_flash_attn_func(q, q, q, group=object())

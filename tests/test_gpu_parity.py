@@ -1,0 +1,374 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on the same seeded inputs.
+
+Tolerances (BASELINE north_star): fp32 out atol 1e-5; bf16 out atol 2e-2 / rtol 1.6e-2;
+lse atol 1e-3; re-layout bit-exact.  fp16 uses the bf16 bound (it is tighter in practice).
+The oracle computes in float64 from the inputs at their storage precision.
+"""
+import hashlib
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import rand, rand_qkv
+from oracle import attn_oracle as O
+import sp_aurora_amd as spa
+from sp_aurora_amd import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+OUT_TOL = {torch.float32: dict(atol=1e-5, rtol=1e-3), torch.bfloat16: dict(atol=2e-2, rtol=1.6e-2),
+           torch.float16: dict(atol=2e-2, rtol=1.6e-2)}
+LSE_ATOL = 1e-3
+
+
+def check_out(got, want, dtype, what="out"):
+    got = got.detach().cpu().to(torch.float64)
+    want = want.to(torch.float64)
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    tol = OUT_TOL[dtype]
+    bad = (got - want).abs() > tol["atol"] + tol["rtol"] * want.abs()
+    assert not bad.any(), f"{what}: {int(bad.sum())} elements out of tolerance, max abs err {(got - want).abs().max():.3e}"
+
+
+def check_lse(got, want):
+    got = got.detach().cpu().to(torch.float64)
+    assert got.dtype == torch.float64 and got.shape == want.shape
+    err = (got - want.to(torch.float64)).abs().max().item()
+    assert err <= LSE_ATOL, f"lse max abs err {err:.3e}"
+
+
+# ------------------------------------------------------------------ block operator
+BLOCK_CASES = [
+    # B, H, Sq, Sk, D, causal
+    (1, 2, 64, 64, 32, True),     # test/flash_attention/test_flash_attention_simple.py:74-137
+    (1, 4, 64, 64, 32, True),     # test_flash_attention_validation.py:76-134, config 1
+    (2, 8, 128, 128, 64, False),  # config 2
+    (1, 12, 256, 256, 64, True),  # config 3
+    (2, 16, 512, 512, 128, False),  # config 4 (batch halved to keep the CPU oracle quick)
+    (1, 3, 1, 1, 64, False),      # a single query, a single key
+    (1, 2, 1, 200, 128, False),   # decode-like
+    (2, 3, 77, 133, 32, False),   # ragged, Sq != Sk
+    (1, 2, 200, 200, 64, True),   # ragged causal
+    (1, 2, 130, 67, 128, True),   # causal with fewer keys than queries
+    (1, 2, 67, 130, 128, True),   # causal with more keys than queries
+    (1, 1, 384, 320, 128, False),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,Sq,Sk,D,causal", BLOCK_CASES)
+def test_block_forward_matches_oracle(B, H, Sq, Sk, D, causal, dtype):
+    q, = rand_qkv((B, H, Sq, D), 42, dtype, n=1)
+    k, v = rand_qkv((B, H, Sk, D), 43, dtype, n=2)
+    want_out, want_lse = O.attn_block(q, k, v, None, causal)
+    out, lse = spa._flash_attn_forward(q.to(DEV), k.to(DEV), v.to(DEV), causal=causal)
+    assert out.dtype == dtype and lse.dtype == torch.float32
+    assert out.shape == (B, H, Sq, D) and lse.shape == (B, H, Sq)
+    check_out(out, want_out, dtype)
+    check_lse(lse, want_lse)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_forward_scale_and_layouts(dtype):
+    """softmax_scale is honoured, and [B,S,H,D] / [B,H,S,D] / packed strided views give one answer."""
+    B, S, H, D = 2, 96, 3, 64
+    qkv = rand((B, S, 3, H, D), 44, dtype)
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+    want_out, want_lse = O.full_attention(q, k, v, 0.2, True)
+    dq = qkv.to(DEV)
+    o1, l1 = ops.flash_fwd(dq[:, :, 0], dq[:, :, 1], dq[:, :, 2], 0.2, True, layout="bshd")  # strided views
+    o2, l2 = ops.flash_fwd(q.to(DEV), k.to(DEV), v.to(DEV), 0.2, True, layout="bshd")
+    o3, l3 = spa.intel_flash_attn_forward(q.transpose(1, 2).to(DEV), k.transpose(1, 2).to(DEV),
+                                          v.transpose(1, 2).to(DEV), softmax_scale=0.2, causal=True)
+    check_out(o1, want_out, dtype)
+    check_lse(l1, want_lse)
+    assert torch.equal(o1, o2) and torch.equal(l1, l2)
+    assert torch.equal(o1, o3.transpose(1, 2)) and torch.equal(l1, l3)
+
+
+def test_block_forward_special_cases():
+    """Closed forms on the device: uniform keys -> mean(V); constant V -> V; causal row 0 -> v[0]."""
+    B, H, S, D = 1, 2, 160, 64
+    q, k, v = rand_qkv((B, H, S, D), 45, torch.float32)
+    k_same = k[:, :, :1].expand(B, H, S, D).contiguous()
+    out, lse = spa._flash_attn_forward(q.to(DEV), k_same.to(DEV), v.to(DEV), softmax_scale=0.5)
+    assert torch.allclose(out.cpu(), v.mean(2, keepdim=True).expand_as(v), atol=1e-5)
+    assert torch.allclose(lse.cpu(), np.log(S) + 0.5 * (q * k[:, :, :1]).sum(-1), atol=1e-4)
+    vc = torch.full_like(v, 2.5)
+    out, _ = spa._flash_attn_forward(q.to(DEV), k.to(DEV), vc.to(DEV), causal=True)
+    assert torch.allclose(out.cpu(), vc, atol=1e-5)
+    out, lse = spa._flash_attn_forward(q.to(DEV), k.to(DEV), v.to(DEV), softmax_scale=0.5, causal=True)
+    assert torch.allclose(out[:, :, 0].cpu(), v[:, :, 0], atol=1e-6)
+    assert torch.allclose(lse[:, :, 0].cpu(), 0.5 * (q[:, :, 0] * k[:, :, 0]).sum(-1), atol=1e-5)
+
+
+def test_block_forward_is_deterministic():
+    """test/flash_attention/test_lse_computation.py:110-112."""
+    q, k, v = [t.to(DEV) for t in rand_qkv((1, 4, 300, 128), 46, torch.bfloat16)]
+    a = spa._flash_attn_forward(q, k, v, causal=True)
+    b = spa._flash_attn_forward(q, k, v, causal=True)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_large_scores_do_not_overflow():
+    q, k, v = rand_qkv((1, 2, 128, 64), 47, torch.bfloat16, scale=30.0)
+    want_out, want_lse = O.attn_block(q, k, v, None, False)
+    out, lse = spa._flash_attn_forward(q.to(DEV), k.to(DEV), v.to(DEV))
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    check_out(out, want_out, torch.bfloat16)
+    assert torch.allclose(lse.cpu().double(), want_lse, rtol=1e-5, atol=1e-3)
+
+
+# ------------------------------------------------------------------ golden fixtures
+def _digest(*tensors):
+    h = hashlib.sha256()
+    for t in tensors:
+        h.update(t.contiguous().view(torch.uint8).numpy().tobytes())
+    return h.hexdigest()
+
+
+GOLDEN_CASES = {
+    "cfg1_fp32_b1_s512_h8_d64": (0, torch.float32, (1, 512, 8, 64), False, 1, 1.0 / 8.0),
+    "simple_fp32_b1_s64_h2_d32_causal": (42, torch.float32, (1, 64, 2, 32), True, 1, None),
+    "ring4_bf16_b1_s256_h4_d64_causal": (7, torch.bfloat16, (1, 256, 4, 64), True, 4, None),
+    "ring2_fp16_b2_s128_h2_d128": (8, torch.float16, (2, 128, 2, 128), False, 2, None),
+    "ring4_fp32_b1_s96_h2_d32_causal": (9, torch.float32, (1, 96, 2, 32), True, 4, None),
+}
+
+
+@pytest.mark.parametrize("name", sorted(GOLDEN_CASES))
+def test_golden_fixture(name):
+    """Committed vectors (tests/golden/make_golden.py); cfg1_* is BASELINE config 1."""
+    seed, dtype, shape, causal, P, scale = GOLDEN_CASES[name]
+    fx = np.load(os.path.join(GOLDEN, name + ".npz"))
+    q, k, v = rand_qkv(shape, seed, dtype)
+    assert _digest(q, k, v) == str(fx["input_sha256"]), "seeded inputs differ from the ones the fixture was made from"
+    res = spa.ring_flash_attn_func(q.to(DEV), k.to(DEV), v.to(DEV), softmax_scale=scale, causal=causal,
+                                   return_attn_probs=True, ring_size=P)
+    out, lse, none = res
+    assert none is None
+    check_out(out, torch.from_numpy(fx["out"]), dtype)
+    check_lse(lse, torch.from_numpy(fx["lse"]))
+
+
+# ------------------------------------------------------------------ merge
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_merge_kernel_matches_oracle(dtype):
+    B, H, S, D = 2, 3, 50, 64
+    g = torch.Generator().manual_seed(60)
+    acc = torch.randn(B, S, H, D, generator=g)
+    lse = torch.randn(B, H, S, generator=g) * 3
+    blk = torch.randn(B, S, H, D, generator=g).to(dtype)
+    blk_lse = torch.randn(B, H, S, generator=g) * 3
+    blk_lse[0, 0, :5] = float("-inf")   # a block that saw nothing leaves the row alone
+    want_out, want_lse = O.merge(acc.double().transpose(1, 2), lse.double().unsqueeze(-1),
+                                 blk.double().transpose(1, 2), blk_lse.double().unsqueeze(-1))
+    d_acc, d_lse = acc.to(DEV), lse.to(DEV)
+    ops.merge(d_acc, d_lse, blk.to(DEV), blk_lse.to(DEV), layout="bshd")
+    assert torch.allclose(d_acc.cpu().double(), want_out.transpose(1, 2), atol=2e-6, rtol=1e-6)
+    assert torch.allclose(d_lse.cpu().double(), want_lse.squeeze(-1), atol=2e-6, rtol=1e-6)
+    assert torch.equal(d_acc[0, :5, 0].cpu(), acc[0, :5, 0])
+    # init = cast/copy; finalize = cast
+    ops.merge(d_acc, d_lse, blk.to(DEV), blk_lse.to(DEV), layout="bshd", init=True)
+    assert torch.equal(d_acc.cpu(), blk.float()) and torch.equal(d_lse.cpu(), blk_lse)
+    fin = ops.finalize(acc.to(DEV), dtype, layout="bshd")
+    assert torch.equal(fin.cpu(), acc.to(dtype))
+
+
+def test_update_out_and_lse_follows_the_reference_contract():
+    """Shapes of sp_aurora/utils.py:116-122 and the split-KV == unsplit invariant."""
+    B, H, S, D = 1, 4, 96, 64
+    q, = rand_qkv((B, H, S, D), 61, torch.bfloat16, n=1)
+    parts = [rand_qkv((B, H, n, D), 62 + i, torch.bfloat16, n=2) for i, n in enumerate((64, 40, 128))]
+    out = lse = None
+    for k, v in parts:
+        b_out, b_lse = spa._flash_attn_forward(q.to(DEV), k.to(DEV), v.to(DEV))
+        out, lse = spa.update_out_and_lse(out, lse, b_out, b_lse)
+        assert out.shape == (B, S, H, D) and out.dtype == torch.float32
+        assert lse.shape == (B, S, H, 1) and lse.dtype == torch.float32
+    k_all = torch.cat([p[0] for p in parts], 2)
+    v_all = torch.cat([p[1] for p in parts], 2)
+    want_out, want_lse = O.attn_block(q, k_all, v_all)
+    check_out(out.transpose(1, 2), want_out, torch.bfloat16)
+    check_lse(lse.squeeze(-1).transpose(1, 2), want_lse)
+    with pytest.raises(RuntimeError):
+        spa.update_out_and_lse(None, None, b_out, b_lse, slice_=(slice(None),))
+    # slice_ updates only the addressed rows
+    before = out.clone()
+    sl = (slice(None), slice(0, 32))
+    b_out, b_lse = spa._flash_attn_forward(q[:, :, :32].to(DEV), parts[0][0].to(DEV), parts[0][1].to(DEV))
+    out2, lse2 = spa.update_out_and_lse(out, lse, b_out, b_lse, slice_=sl)
+    assert torch.equal(out2[:, 32:], before[:, 32:]) and not torch.equal(out2[:, :32], before[:, :32])
+
+
+# ------------------------------------------------------------------ ring
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("P", [1, 2, 4])
+def test_ring_equals_full_attention(P, causal, dtype):
+    """test/test_ring_attention_full_accuracy.py:29-171 (B2, s128, H8, D64, gather and compare)."""
+    B, s, H, D = 2, 128, 8, 64
+    q, k, v = rand_qkv((B, P * s, H, D), 70, dtype)
+    want_out, want_lse = O.full_attention(q, k, v, None, causal)
+    out, lse, _ = spa.ring_flash_attn_func(q.to(DEV), k.to(DEV), v.to(DEV), causal=causal,
+                                           return_attn_probs=True, ring_size=P)
+    check_out(out, want_out, dtype)
+    check_lse(lse, want_lse)
+    only_out = spa.sp_aurora_func(q.to(DEV), k.to(DEV), v.to(DEV), causal=causal, ring_size=P)
+    assert torch.equal(only_out, out)
+
+
+def test_ring_rank_follows_the_oracle_schedule():
+    """One rank's chunk against its KV chunks in ring order, as BASELINE config 2 (scaled down)."""
+    P, B, s, H, D, rank = 4, 2, 96, 4, 64, 2
+    q, k, v = rand_qkv((B, P * s, H, D), 71, torch.bfloat16)
+    ks, vs = list(k.chunk(P, 1)), list(v.chunk(P, 1))
+    q_r = q[:, rank * s:(rank + 1) * s]
+    for causal in (True, False):
+        want_out, want_lse = O.ring_forward_rank(q_r, ks, vs, rank, None, causal, out_dtype=torch.float64)
+        out, lse = spa.ring_flash_attn_forward_rank(q_r.to(DEV), [t.to(DEV) for t in ks], [t.to(DEV) for t in vs],
+                                                    rank, None, causal)
+        check_out(out, want_out, torch.bfloat16)
+        check_lse(lse, want_lse)
+
+
+def test_packed_equals_unpacked():
+    """test/test_ring_attention_comprehensive.py:205-218."""
+    B, S, H, D = 1, 256, 4, 64
+    qkv = rand((B, S, 3, H, D), 72, torch.bfloat16).to(DEV)
+    q, k, v = [qkv[:, :, i].contiguous() for i in range(3)]
+    a = spa.ring_flash_attn_func(q, k, v, causal=True, ring_size=2)
+    b = spa.ring_flash_attn_qkvpacked_func(qkv, causal=True, ring_size=2)
+    c = spa.ring_flash_attn_kvpacked_func(q, qkv[:, :, 1:], causal=True, ring_size=2)
+    assert torch.equal(a, b) and torch.equal(a, c)
+
+
+# ------------------------------------------------------------------ re-layout
+def _tagged(shape, dtype):
+    n = int(np.prod(shape))
+    if dtype in (torch.int16, torch.uint8):
+        info = torch.iinfo(dtype)
+        return (torch.arange(n, dtype=torch.int64) % (info.max + 1)).to(dtype).view(shape)
+    return torch.arange(n, dtype=torch.int64).to(dtype).view(shape)
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int32, torch.int64])
+@pytest.mark.parametrize("P,B,s,H,D,pack", [(4, 1, 4, 8, 8, None), (2, 2, 3, 4, 16, None), (8, 1, 5, 16, 32, None),
+                                            (4, 2, 4, 8, 8, 3), (2, 1, 6, 2, 64, 2), (3, 2, 2, 3, 5, None)])
+def test_relayout_is_bit_exact(P, B, s, H, D, pack, dtype):
+    """Tagged integers land where the reference's op chain puts them
+    (archived_fallbacks/test_all_to_all_alternatives.py:126-161 uses tagged aranges the same way)."""
+    shape = (P, B, s) + ((pack,) if pack else ()) + (H, D)
+    x = _tagged(shape, dtype)
+    if pack == 3:
+        want = torch.stack(O.all_to_all_5d_s2h(list(x)))
+    elif pack is None:
+        want = torch.stack(O.all_to_all_4d_s2h(list(x)))
+    else:
+        want = O.relayout_s2h_formula(x)
+    y = ops.relayout_s2h(x.to(DEV), P)
+    assert y.shape == want.shape and torch.equal(y.cpu(), want)
+    back = ops.relayout_h2s(y, P)
+    assert torch.equal(back.cpu(), x)  # inverse o forward = identity
+    if pack == 3:
+        assert torch.equal(back.cpu(), torch.stack(O.all_to_all_5d_h2s(list(want))))
+    elif pack is None:
+        assert torch.equal(back.cpu(), torch.stack(O.all_to_all_4d_h2s(list(want))))
+
+
+def test_relayout_api_names():
+    P, B, s, H, D = 4, 2, 8, 8, 32
+    x = rand((P, B, s, H, D), 80, torch.bfloat16).to(DEV)
+    y = spa.intel_all_to_all_4d(x, 2, 1)
+    assert y.shape == (P, B, P * s, H // P, D)   # test/ulysses/test_intel_alltoall_4d.py:93-100
+    assert torch.equal(y.cpu(), O.relayout_s2h_formula(x.cpu()))
+    assert torch.equal(spa.intel_all_to_all_4d(y, 1, 2), x)   # :140-147 and round trip
+    assert torch.equal(spa.all_to_all_4D(x, 2, 1), y)
+    x5 = rand((P, B, s, 3, H, D), 81, torch.bfloat16).to(DEV)
+    y5 = spa.all_to_all_5D(x5, 3, 1)
+    assert torch.equal(y5.cpu(), O.relayout_s2h_formula(x5.cpu()))
+    assert torch.equal(spa.all_to_all_5D(y5, 1, 3), x5)
+    assert spa.intel_all_to_all_4d(x[0]) is x[0] or torch.equal(spa.intel_all_to_all_4d(x[0]), x[0])  # world size 1
+    with pytest.raises(ValueError):
+        spa.intel_all_to_all_4d(x, 0, 3)
+    # autograd: backward of the re-layout is the inverse re-layout
+    xr = x.float().requires_grad_(True)
+    yr = spa.SeqAllToAll4D.apply(None, xr, 2, 1)
+    g = torch.randn_like(yr)
+    yr.backward(g)
+    assert torch.equal(xr.grad, ops.relayout_h2s(g, P))
+
+
+# ------------------------------------------------------------------ Ulysses
+@pytest.mark.parametrize("causal", [False, True])
+def test_ulysses_equals_full_attention(causal):
+    """test/verification/test_ulysses_fixed.py:165-344 (fp16, B2, s64, H4, D64) — here with strict bounds."""
+    P, B, s, H, D = 4, 2, 64, 4, 64
+    q, k, v = rand_qkv((B, P * s, H, D), 90, torch.float16)
+    want_out, want_lse = O.full_attention(q, k, v, None, causal)
+    stack = lambda t: torch.stack(t.chunk(P, 1)).contiguous().to(DEV)
+    out = spa.ulysses_flash_attn_func(stack(q), stack(k), stack(v), causal=causal)
+    assert out.shape == (P, B, s, H, D)
+    check_out(torch.cat(list(out), 1), want_out, torch.float16)
+    out2, lse = spa.intel_ulysses_flash_attn_forward(None, stack(q), stack(k), stack(v), D ** -0.5, causal=causal)
+    assert torch.equal(out, out2) and lse.shape == (P, B, H // P, P * s)
+    check_lse(torch.cat(list(lse), 1), want_lse)
+    qkv = torch.stack([stack(q), stack(k), stack(v)], dim=3)
+    assert torch.equal(spa.ulysses_flash_attn_qkvpacked_func(qkv, causal=causal), out)
+
+
+# ------------------------------------------------------------------ backward
+GRAD_TOL = {torch.bfloat16: dict(atol=3e-2, rtol=3e-2), torch.float16: dict(atol=4e-3, rtol=1e-2)}
+
+
+def check_grad(got, want, dtype, what):
+    got = got.detach().cpu().double()
+    tol = GRAD_TOL[dtype]
+    bad = (got - want).abs() > tol["atol"] * want.abs().max() + tol["rtol"] * want.abs()
+    assert not bad.any(), f"{what}: {int(bad.sum())} out of tolerance, max abs err {(got - want).abs().max():.3e} (scale {want.abs().max():.3e})"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,S,H,D,causal,P", [(1, 128, 2, 64, False, 1), (2, 256, 3, 128, True, 1), (1, 256, 2, 32, True, 4),
+                                              (1, 192, 2, 128, False, 3), (1, 200, 2, 64, True, 1), (1, 77, 1, 128, False, 1),
+                                              (1, 512, 2, 128, True, 4)])
+def test_backward_matches_autograd_of_full_attention(B, S, H, D, causal, P, dtype):
+    """Gradients against the oracle's autograd through full attention, relative to each gradient's scale."""
+    q, k, v, dout = rand_qkv((B, S, H, D), 100, dtype, n=4)
+    want = O.attn_backward_autograd(q, k, v, dout, None, causal)
+    dq_, dk_, dv_ = [t.to(DEV).requires_grad_(True) for t in (q, k, v)]
+    out = spa.ring_flash_attn_func(dq_, dk_, dv_, causal=causal, ring_size=P)
+    out.backward(dout.to(DEV))
+    for got, w, name in zip((dq_.grad, dk_.grad, dv_.grad), want, "qkv"):
+        assert got.dtype == dtype
+        check_grad(got, w, dtype, "d" + name)
+
+
+def test_backward_packed_and_operator_entry():
+    B, S, H, D = 1, 256, 2, 128
+    qkv = rand((B, S, 3, H, D), 101, torch.bfloat16)
+    dout = rand((B, S, H, D), 102, torch.bfloat16)
+    want = O.attn_backward_autograd(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], dout, None, True)
+    dqkv = qkv.to(DEV).requires_grad_(True)
+    out, lse, _ = spa.ring_flash_attn_qkvpacked_func(dqkv, causal=True, return_attn_probs=True, ring_size=2)
+    out.backward(dout.to(DEV))
+    for i, name in enumerate("qkv"):
+        check_grad(dqkv.grad[:, :, i], want[i], torch.bfloat16, "packed d" + name)
+    # operator-level backward ([B,H,S,D], saved out and lse)
+    t = lambda x: x.transpose(1, 2).contiguous().to(DEV)
+    q, k, v = t(qkv[:, :, 0]), t(qkv[:, :, 1]), t(qkv[:, :, 2])
+    o, l = spa._flash_attn_forward(q, k, v, causal=True)
+    dq, dk, dv = spa._flash_attn_backward(t(dout), q, k, v, o, l, causal=True)
+    for got, w, name in zip((dq, dk, dv), want, "qkv"):
+        check_grad(got.transpose(1, 2), w, torch.bfloat16, "operator d" + name)
+
+
+def test_delta_kernel():
+    o, do = rand_qkv((2, 40, 3, 64), 103, torch.bfloat16, n=2)
+    got = ops.bwd_delta(o.to(DEV), do.to(DEV))
+    want = (o.double() * do.double()).sum(-1).transpose(1, 2)
+    assert torch.allclose(got.cpu().double(), want, atol=1e-4, rtol=1e-5)
