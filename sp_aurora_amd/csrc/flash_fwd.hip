@@ -19,38 +19,49 @@
 //   B agree; V^T is stored in LDS with keys permuted (bits 2 and 3 of the key
 //   index within a 32-key block swapped) so that the 8 keys a lane needs for
 //   one P^T operand are one 16-byte LDS read.
+#include <stdlib.h>
+
 #include "spa_common.h"
 
 namespace {
 
 constexpr int FWD_BM = 128;  // query rows per workgroup
-constexpr int FWD_BN = 64;   // keys per LDS tile
-constexpr int FWD_THREADS = 256;
+constexpr int FWD_BN = 64;   // keys per LDS sub-tile (one per wave group)
+constexpr int FWD_THREADS = 256;  // threads of one wave group (4 waves x 32 query rows)
 
-template <int D>
+// NG wave groups share the 128 query rows and split the keys: in every step group g works on
+// the g-th 64-key sub-tile of a 64*NG-key tile, so 4*NG waves sit on the CU's 4 SIMDs and the
+// MFMA phase of one wave overlaps the softmax (VALU) phase of its SIMD neighbour.  The groups'
+// partial (O, m, l) are combined through LDS after the key loop.
+template <int D, int NG>
 struct Fwd16Cfg {
+  static constexpr int THREADS = FWD_THREADS * NG;
   static constexpr int KP = D * 2 + 16;       // K tile row pitch in bytes (+16: bank spread)
   static constexpr int VP = FWD_BN * 2 + 16;  // V^T tile row pitch in bytes
   static constexpr int KBYTES = FWD_BN * KP;
   static constexpr int VBYTES = D * VP;
-  static constexpr int STAGE = KBYTES + VBYTES;
-  static constexpr int SMEM = 2 * STAGE;
+  static constexpr int SUB = KBYTES + VBYTES;  // one 64-key sub-tile: K rows, then V^T
+  static constexpr int STAGE = NG * SUB;
+  static constexpr int XCH = NG > 1 ? 4 * (D / 2 + 2) * 64 * 4 : 0;  // group exchange area
+  static constexpr int SMEM = 2 * STAGE > XCH ? 2 * STAGE : XCH;
   static constexpr int CPR = D / 8;              // 16-byte chunks per row
-  static constexpr int RPP = FWD_THREADS / CPR;  // K rows fetched per pass
-  static constexpr int KPASS = FWD_BN / RPP;     // passes per K tile
-  static constexpr int VUNITS = 16 * CPR;        // (4 keys x 8 dims) units per V tile
+  static constexpr int RPP = THREADS / CPR;      // K rows fetched per pass
+  static constexpr int KPASS = FWD_BN * NG / RPP;  // passes per K tile
+  static constexpr int VUNITS = 16 * NG * CPR;   // (4 keys x 8 dims) units per V tile
 };
 
-template <typename T, int D>
-__global__ void __launch_bounds__(FWD_THREADS, 2) flash_fwd16_kernel(const FwdParams p) {
-  typedef Fwd16Cfg<D> C;
+template <typename T, int D, int NG>
+__global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams p) {
+  typedef Fwd16Cfg<D, NG> C;
   typedef Mma16<T> M;
   typedef typename M::frag frag;
   extern __shared__ __align__(16) unsigned char smem[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int w = tid >> 6;
+  const int wave = tid >> 6;
+  const int w = wave & 3;    // which 32 query rows
+  const int grp = wave >> 2;  // which key sub-tile
   const int ln = lane & 31;
   const int hh = lane >> 5;
 
@@ -76,23 +87,25 @@ __global__ void __launch_bounds__(FWD_THREADS, 2) flash_fwd16_kernel(const FwdPa
   for (int ks = 0; ks < D / 16; ++ks)
     qf[ks] = as_frag<frag>(*(const u32x4*)(qp + (int64_t)qrow_c * p.qs.s + ks * 16 + hh * 8));
 
+  constexpr int TILE = FWD_BN * NG;
   const int kv_end = p.causal ? (q0 + FWD_BM < p.Sk ? q0 + FWD_BM : p.Sk) : p.Sk;
-  const int nt = (kv_end + FWD_BN - 1) / FWD_BN;
+  const int nt = (kv_end + TILE - 1) / TILE;
 
   // ---- global -> register staging of one K / V tile ----
   const int kc = tid % C::CPR;
   const int kr = tid / C::CPR;
-  const int vkg = tid & 15;  // group of 4 consecutive keys
-  const int vdc = tid >> 4;  // chunk of 8 head dims
+  const int vkg = tid & (16 * NG - 1);  // group of 4 consecutive keys
+  const int vdc = tid / (16 * NG);      // chunk of 8 head dims
   const bool vact = tid < C::VUNITS;
-  // position of this key group inside the permuted 64-key row of V^T
-  const int vpos = (vkg >> 3) * 32 + ((vkg >> 2) & 1) * 16 + (vkg & 1) * 8 + ((vkg >> 1) & 1) * 4;
+  // position of this key group inside the permuted 64-key row of its sub-tile's V^T
+  const int vsub = vkg >> 4;
+  const int vpos = ((vkg >> 3) & 1) * 32 + ((vkg >> 2) & 1) * 16 + (vkg & 1) * 8 + ((vkg >> 1) & 1) * 4;
 
   u32x4 kreg[C::KPASS];
   u32x4 vreg[4];
 
   auto gload = [&](int it) {
-    const int key0 = it * FWD_BN;
+    const int key0 = it * TILE;
 #pragma unroll
     for (int i = 0; i < C::KPASS; ++i) {
       int r = key0 + kr + i * C::RPP;
@@ -110,12 +123,14 @@ __global__ void __launch_bounds__(FWD_THREADS, 2) flash_fwd16_kernel(const FwdPa
   };
 
   auto lstore = [&](int stage) {
-    unsigned char* kb = smem + stage * C::STAGE;
-    unsigned char* vb = kb + C::KBYTES;
+    unsigned char* sb = smem + stage * C::STAGE;
 #pragma unroll
-    for (int i = 0; i < C::KPASS; ++i)
-      *(u32x4*)(kb + (kr + i * C::RPP) * C::KP + kc * 16) = kreg[i];
+    for (int i = 0; i < C::KPASS; ++i) {
+      const int r = kr + i * C::RPP;
+      *(u32x4*)(sb + (r >> 6) * C::SUB + (r & 63) * C::KP + kc * 16) = kreg[i];
+    }
     if (vact) {
+      unsigned char* vb = sb + vsub * C::SUB + C::KBYTES;
       // 4 keys x 8 dims in registers -> 8 rows (dims) of 4 consecutive keys
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
@@ -136,7 +151,7 @@ __global__ void __launch_bounds__(FWD_THREADS, 2) flash_fwd16_kernel(const FwdPa
   for (int i = 0; i < D / 32; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[i][v] = 0.f;
-  float m_run = -INFINITY;  // running row max of the raw scores
+  float m_run = -INFINITY;  // reference row max of the raw scores (may lag the true max, see below)
   float l_run = 0.f;        // this lane's share of the running row sum
 
   gload(0);
@@ -147,14 +162,14 @@ __global__ void __launch_bounds__(FWD_THREADS, 2) flash_fwd16_kernel(const FwdPa
 
   for (int it = 0; it < nt; ++it) {
     const int cur = it & 1;
-    const int key0 = it * FWD_BN;
+    const int key0 = it * TILE + grp * FWD_BN;
     const bool more = it + 1 < nt;
     if (more) gload(it + 1);
 
-    // a wave whose rows all precede this tile has nothing to do in it
-    const bool active = !(p.causal && key0 > qw0 + 31);
+    // a wave whose rows all precede its sub-tile, or whose sub-tile lies past the keys, idles
+    const bool active = key0 < kv_end && !(p.causal && key0 > qw0 + 31);
     if (active) {
-      const unsigned char* kb = smem + cur * C::STAGE;
+      const unsigned char* kb = smem + cur * C::STAGE + grp * C::SUB;
       const unsigned char* vb = kb + C::KBYTES;
 
       f32x16 s[2];
@@ -187,10 +202,19 @@ __global__ void __launch_bounds__(FWD_THREADS, 2) flash_fwd16_kernel(const FwdPa
 #pragma unroll
       for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[1][v]);
       mx = fmaxf(mx, xhalf(mx));
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = fast_exp2((m_run - m_new) * c);
-      const float mc = m_new * c;
-      m_run = m_new;
+      // Lazy rescale: the reference max only moves when some row's max grew by more than
+      // 2^8 in the exp2 domain; until then P <= 256, harmless in fp32 sums and bf16 operands.
+      if (__builtin_amdgcn_ballot_w64((mx - m_run) * c > 8.f) != 0) {
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = fast_exp2((m_run - m_new) * c);
+        m_run = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
+      }
+      const float mc = m_run * c;
 
       float ps = 0.f;
 #pragma unroll
@@ -201,12 +225,7 @@ __global__ void __launch_bounds__(FWD_THREADS, 2) flash_fwd16_kernel(const FwdPa
           s[t][v] = e;
           ps += e;
         }
-      l_run = l_run * alpha + ps;
-
-#pragma unroll
-      for (int i = 0; i < D / 32; ++i)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
+      l_run += ps;
 
       frag pf[2][2];
 #pragma unroll
@@ -232,22 +251,54 @@ __global__ void __launch_bounds__(FWD_THREADS, 2) flash_fwd16_kernel(const FwdPa
     __syncthreads();
   }
 
+  // ---- combine the wave groups: groups 1.. hand (O, m, l) to group 0 through LDS ----
+  if (NG > 1) {
+    float* xch = (float*)smem;  // [w][slot][lane], slot = D/2 accumulators, then m, then l
+    constexpr int SLOTS = D / 2 + 2;
+    if (grp == 1) {
+      float* dst = xch + (w * SLOTS) * 64 + lane;
+#pragma unroll
+      for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dst[(i * 16 + v) * 64] = o[i][v];
+      dst[(D / 2) * 64] = m_run;
+      dst[(D / 2 + 1) * 64] = l_run;
+    }
+    __syncthreads();
+    if (grp == 0) {
+      const float* src = xch + (w * SLOTS) * 64 + lane;
+      const float m1 = src[(D / 2) * 64];
+      const float l1 = src[(D / 2 + 1) * 64];
+      const float m_new = fmaxf(m_run, m1);  // finite: group 0 always sees key 0
+      const float a0 = fast_exp2((m_run - m_new) * c);
+      const float a1 = fast_exp2((m1 - m_new) * c);
+      m_run = m_new;
+      l_run = l_run * a0 + l1 * a1;
+#pragma unroll
+      for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[i][v] = o[i][v] * a0 + src[(i * 16 + v) * 64] * a1;
+    }
+  }
+
   // ---- epilogue: normalise, store out and lse ----
-  const float l_tot = l_run + xhalf(l_run);
-  const float inv = 1.f / l_tot;
-  if (qrow < p.Sq) {
-    T* op = (T*)p.out + b * p.os.b + h * p.os.h + (int64_t)qrow * p.os.s;
+  if (grp == 0) {
+    const float l_tot = l_run + xhalf(l_run);
+    const float inv = 1.f / l_tot;
+    if (qrow < p.Sq) {
+      T* op = (T*)p.out + b * p.os.b + h * p.os.h + (int64_t)qrow * p.os.s;
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db)
+      for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 st;
-        st[0] = M::pack2(o[db][4 * g + 0] * inv, o[db][4 * g + 1] * inv);
-        st[1] = M::pack2(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
-        *(u32x2*)(op + db * 32 + 8 * g + 4 * hh) = st;
-      }
-    if (hh == 0)
-      p.lse[((int64_t)b * p.H + h) * p.Sq + qrow] = (m_run * c + fast_log2(l_tot)) * 0.6931471805599453f;
+        for (int g = 0; g < 4; ++g) {
+          u32x2 st;
+          st[0] = M::pack2(o[db][4 * g + 0] * inv, o[db][4 * g + 1] * inv);
+          st[1] = M::pack2(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
+          *(u32x2*)(op + db * 32 + 8 * g + 4 * hh) = st;
+        }
+      if (hh == 0)
+        p.lse[((int64_t)b * p.H + h) * p.Sq + qrow] = (m_run * c + fast_log2(l_tot)) * 0.6931471805599453f;
+    }
   }
 }
 
@@ -442,12 +493,24 @@ __global__ void __launch_bounds__(FWD_THREADS, 1) flash_fwd32_kernel(const FwdPa
 }
 
 template <typename K>
-hipError_t launch(K kernel, int smem, const FwdParams& p, hipStream_t stream) {
+hipError_t launch(K kernel, int threads, int smem, const FwdParams& p, hipStream_t stream) {
   hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return e;
   const dim3 grid((unsigned)((int64_t)p.B * p.H * p.nqt));
-  hipLaunchKernelGGL(kernel, grid, dim3(FWD_THREADS), smem, stream, p);
+  hipLaunchKernelGGL(kernel, grid, dim3(threads), smem, stream, p);
   return hipGetLastError();
+}
+
+// Two wave groups once there are at least two 64-key sub-tiles to split.
+template <typename T, int D>
+hipError_t launch16(const FwdParams& p, hipStream_t stream) {
+  static const int force = []() {
+    const char* e = getenv("SPA_FWD_GROUPS");
+    return e ? atoi(e) : 0;
+  }();
+  const bool two = force ? force == 2 : p.Sk > FWD_BN;
+  if (two) return launch(flash_fwd16_kernel<T, D, 2>, 2 * FWD_THREADS, Fwd16Cfg<D, 2>::SMEM, p, stream);
+  return launch(flash_fwd16_kernel<T, D, 1>, FWD_THREADS, Fwd16Cfg<D, 1>::SMEM, p, stream);
 }
 
 }  // namespace
@@ -456,17 +519,17 @@ hipError_t launch(K kernel, int smem, const FwdParams& p, hipStream_t stream) {
 hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream) {
   p.nqt = (p.Sq + FWD_BM - 1) / FWD_BM;
   if (dtype == 1) {
-    if (D == 128) return launch(flash_fwd16_kernel<__bf16, 128>, Fwd16Cfg<128>::SMEM, p, stream);
-    if (D == 64) return launch(flash_fwd16_kernel<__bf16, 64>, Fwd16Cfg<64>::SMEM, p, stream);
-    if (D == 32) return launch(flash_fwd16_kernel<__bf16, 32>, Fwd16Cfg<32>::SMEM, p, stream);
+    if (D == 128) return launch16<__bf16, 128>(p, stream);
+    if (D == 64) return launch16<__bf16, 64>(p, stream);
+    if (D == 32) return launch16<__bf16, 32>(p, stream);
   } else if (dtype == 2) {
-    if (D == 128) return launch(flash_fwd16_kernel<_Float16, 128>, Fwd16Cfg<128>::SMEM, p, stream);
-    if (D == 64) return launch(flash_fwd16_kernel<_Float16, 64>, Fwd16Cfg<64>::SMEM, p, stream);
-    if (D == 32) return launch(flash_fwd16_kernel<_Float16, 32>, Fwd16Cfg<32>::SMEM, p, stream);
+    if (D == 128) return launch16<_Float16, 128>(p, stream);
+    if (D == 64) return launch16<_Float16, 64>(p, stream);
+    if (D == 32) return launch16<_Float16, 32>(p, stream);
   } else if (dtype == 0) {
-    if (D == 128) return launch(flash_fwd32_kernel<128>, Fwd32Cfg<128>::SMEM, p, stream);
-    if (D == 64) return launch(flash_fwd32_kernel<64>, Fwd32Cfg<64>::SMEM, p, stream);
-    if (D == 32) return launch(flash_fwd32_kernel<32>, Fwd32Cfg<32>::SMEM, p, stream);
+    if (D == 128) return launch(flash_fwd32_kernel<128>, FWD_THREADS, Fwd32Cfg<128>::SMEM, p, stream);
+    if (D == 64) return launch(flash_fwd32_kernel<64>, FWD_THREADS, Fwd32Cfg<64>::SMEM, p, stream);
+    if (D == 32) return launch(flash_fwd32_kernel<32>, FWD_THREADS, Fwd32Cfg<32>::SMEM, p, stream);
   }
   return hipErrorInvalidValue;
 }

@@ -22,7 +22,7 @@ from . import ops
 from .flash_attn import _check_unsupported
 
 __all__ = [
-    "ring_flash_attn_forward_rank", "ring_flash_attn_forward", "ring_flash_attn_backward",
+    "ring_flash_attn_forward_rank", "ring_flash_attn_forward", "ring_flash_attn_backward", "make_ring_forward_step",
     "RingFlashAttnFunc", "IntelRingFlashAttnFunc",
     "ring_flash_attn_func", "ring_flash_attn_kvpacked_func", "ring_flash_attn_qkvpacked_func",
     "intel_ring_flash_attn_func", "intel_ring_flash_attn_kvpacked_func", "intel_ring_flash_attn_qkvpacked_func",
@@ -44,6 +44,7 @@ class _RingWorkspace:
         self.blk_out = torch.empty((B, s, H, D), dtype=dtype, device=device)
         self.blk_lse = torch.empty((B, H, s), dtype=torch.float32, device=device)
         self.acc = torch.empty((B, s, H, D), dtype=torch.float32, device=device)
+        self.lse_r = torch.empty((B, H, s), dtype=torch.float32, device=device)
 
 
 def ring_flash_attn_forward_rank(q_local, k_chunks, v_chunks, rank, softmax_scale=None, causal=False,
@@ -79,25 +80,44 @@ def ring_flash_attn_forward_rank(q_local, k_chunks, v_chunks, rank, softmax_scal
     return out, lse
 
 
-def ring_flash_attn_forward(q, k, v, softmax_scale=None, causal=False, ring_size=1):
-    """All ranks of a simulated ring over contiguous shards of q,k,v [B,S,H,D]."""
+def ring_flash_attn_forward(q, k, v, softmax_scale=None, causal=False, ring_size=1, out=None, lse=None,
+                            workspace=None):
+    """All ranks of a simulated ring over contiguous shards of q,k,v [B,S,H,D].
+    Returns out [B,S,H,D] (q dtype) and lse fp32 [B,H,S]; `out`, `lse`, `workspace` may be
+    passed in to run without allocating."""
     B, S, H, D = q.shape
     P = int(ring_size)
-    if P < 1 or S % P or k.shape[1] != S and P > 1:
+    if P < 1 or S % P or (P > 1 and k.shape[1] != S):
         raise ValueError(f"ring_size={P} must divide the sequence length {S} (and k/v must match q)")
     if P == 1:
-        return ops.flash_fwd(q, k, v, softmax_scale, causal, layout="bshd")
+        return ops.flash_fwd(q, k, v, softmax_scale, causal, layout="bshd", out=out, lse=lse)
     s = S // P
-    out = torch.empty((B, S, H, D), dtype=q.dtype, device=q.device)
-    lse_all = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
+    if out is None:
+        out = torch.empty((B, S, H, D), dtype=q.dtype, device=q.device)
+    if lse is None:
+        lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
     ks, vs = list(k.split(s, dim=1)), list(v.split(s, dim=1))
-    ws = _RingWorkspace(B, s, H, D, q.dtype, q.device)
-    lse_r = torch.empty((B, H, s), dtype=torch.float32, device=q.device)
+    ws = workspace or _RingWorkspace(B, s, H, D, q.dtype, q.device)
     for r in range(P):
         ring_flash_attn_forward_rank(q[:, r * s:(r + 1) * s], ks, vs, r, softmax_scale, causal,
-                                     out=out[:, r * s:(r + 1) * s], lse=lse_r, workspace=ws)
-        lse_all[:, :, r * s:(r + 1) * s] = lse_r
-    return out, lse_all
+                                     out=out[:, r * s:(r + 1) * s], lse=ws.lse_r, workspace=ws)
+        lse[:, :, r * s:(r + 1) * s] = ws.lse_r
+    return out, lse
+
+
+def make_ring_forward_step(q, k, v, softmax_scale=None, causal=False, ring_size=1):
+    """Preallocates every buffer ring_flash_attn_forward needs and returns a zero-argument
+    callable that runs the whole ring forward into them and returns (out, lse)."""
+    B, S, H, D = q.shape
+    P = int(ring_size)
+    out = torch.empty((B, S, H, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
+    ws = _RingWorkspace(B, S // P, H, D, q.dtype, q.device) if P > 1 else None
+
+    def step():
+        return ring_flash_attn_forward(q, k, v, softmax_scale, causal, P, out=out, lse=lse, workspace=ws)
+
+    return step
 
 
 def ring_flash_attn_backward(dout, q, k, v, out, softmax_lse, softmax_scale=None, causal=False, ring_size=1):
