@@ -5,8 +5,7 @@
 // one Q.K^T instead of the reference's two, scores never leave the CU.
 //
 // Work decomposition (16-bit kernel)
-//   workgroup = 128 query rows of one (batch, head), 4 wavefronts x 32 rows;
-//   KV is walked in tiles of 64 keys, double-buffered in LDS.
+//   workgroup = 128 query rows of one (batch, head); a wave owns 32 of them.
 //   Both contractions are computed TRANSPOSED on v_mfma_f32_32x32x16:
 //     S^T[key][qrow] = K[key][:] . Q[qrow][:]      A = K tile (LDS), B = Q (registers)
 //     O^T[d][qrow]  += V^T[d][key] . P^T[key][qrow] A = V^T tile (LDS), B = P^T (registers)
@@ -19,35 +18,40 @@
 //   B agree; V^T is stored in LDS with keys permuted (bits 2 and 3 of the key
 //   index within a 32-key block swapped) so that the 8 keys a lane needs for
 //   one P^T operand are one 16-byte LDS read.
+//
+//   Two wave groups (8 waves, two per SIMD) share the query rows and take alternate
+//   64-key sub-tiles; each group streams its own sub-tiles through its own
+//   double-buffered LDS.  A wave's loop is software-pipelined into two phases,
+//       VALU phase:  softmax of S(i) -> P(i);  stage K(i+2), V(i+1) into LDS
+//       MFMA phase:  issue the next global loads;  O += V(i)^T P(i);  S(i+1) = K(i+1) Q^T
+//   separated by workgroup barriers, and group 1 runs one barrier behind group 0, so at
+//   any time one wave of a SIMD is in its MFMA phase while its neighbour is in its VALU
+//   phase (ping-pong).  The groups' partial (O, m, l) are combined through LDS at the end.
 #include <stdlib.h>
+
+#include <type_traits>
 
 #include "spa_common.h"
 
 namespace {
 
 constexpr int FWD_BM = 128;  // query rows per workgroup
-constexpr int FWD_BN = 64;   // keys per LDS sub-tile (one per wave group)
+constexpr int FWD_BN = 64;   // keys per LDS sub-tile
 constexpr int FWD_THREADS = 256;  // threads of one wave group (4 waves x 32 query rows)
 
-// NG wave groups share the 128 query rows and split the keys: in every step group g works on
-// the g-th 64-key sub-tile of a 64*NG-key tile, so 4*NG waves sit on the CU's 4 SIMDs and the
-// MFMA phase of one wave overlaps the softmax (VALU) phase of its SIMD neighbour.  The groups'
-// partial (O, m, l) are combined through LDS after the key loop.
 template <int D, int NG>
 struct Fwd16Cfg {
-  static constexpr int THREADS = FWD_THREADS * NG;
   static constexpr int KP = D * 2 + 16;       // K tile row pitch in bytes (+16: bank spread)
   static constexpr int VP = FWD_BN * 2 + 16;  // V^T tile row pitch in bytes
   static constexpr int KBYTES = FWD_BN * KP;
   static constexpr int VBYTES = D * VP;
-  static constexpr int SUB = KBYTES + VBYTES;  // one 64-key sub-tile: K rows, then V^T
-  static constexpr int STAGE = NG * SUB;
-  static constexpr int XCH = NG > 1 ? 4 * (D / 2 + 2) * 64 * 4 : 0;  // group exchange area
-  static constexpr int SMEM = 2 * STAGE > XCH ? 2 * STAGE : XCH;
+  static constexpr int GROUP = 2 * KBYTES + 2 * VBYTES;  // one group's K[2] and V^T[2] buffers
+  static constexpr int EPI = (NG * FWD_BM * (D + 4) + NG * FWD_BM * 2 + FWD_BM) * 4;  // epilogue staging
+  static constexpr int SMEM = NG * GROUP > EPI ? NG * GROUP : EPI;
   static constexpr int CPR = D / 8;              // 16-byte chunks per row
-  static constexpr int RPP = THREADS / CPR;      // K rows fetched per pass
-  static constexpr int KPASS = FWD_BN * NG / RPP;  // passes per K tile
-  static constexpr int VUNITS = 16 * NG * CPR;   // (4 keys x 8 dims) units per V tile
+  static constexpr int RPP = FWD_THREADS / CPR;  // K rows fetched per pass
+  static constexpr int KPASS = FWD_BN / RPP;     // passes per K sub-tile
+  static constexpr int VUNITS = 16 * CPR;        // (4 keys x 8 dims) units per V sub-tile
 };
 
 template <typename T, int D, int NG>
@@ -59,9 +63,10 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int w = wave & 3;    // which 32 query rows
-  const int grp = wave >> 2;  // which key sub-tile
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int w = wave & 3;     // which 32 query rows
+  const int grp = wave >> 2;  // which key sub-tiles
+  const int tg = tid & (FWD_THREADS - 1);  // thread index inside the group
   const int ln = lane & 31;
   const int hh = lane >> 5;
 
@@ -87,61 +92,95 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   for (int ks = 0; ks < D / 16; ++ks)
     qf[ks] = as_frag<frag>(*(const u32x4*)(qp + (int64_t)qrow_c * p.qs.s + ks * 16 + hh * 8));
 
-  constexpr int TILE = FWD_BN * NG;
   const int kv_end = p.causal ? (q0 + FWD_BM < p.Sk ? q0 + FWD_BM : p.Sk) : p.Sk;
-  const int nt = (kv_end + TILE - 1) / TILE;
+  const int n = (kv_end + FWD_BN * NG - 1) / (FWD_BN * NG);  // sub-tiles per group
+  // first key of this group's i-th sub-tile
+  auto key_of = [&](int i) { return (i * NG + grp) * FWD_BN; };
+  unsigned char* gbase = smem + grp * C::GROUP;
+  auto kbuf = [&](int i) { return gbase + (i & 1) * C::KBYTES; };
+  auto vbuf = [&](int i) { return gbase + 2 * C::KBYTES + (i & 1) * C::VBYTES; };
 
-  // ---- global -> register staging of one K / V tile ----
-  const int kc = tid % C::CPR;
-  const int kr = tid / C::CPR;
-  const int vkg = tid & (16 * NG - 1);  // group of 4 consecutive keys
-  const int vdc = tid / (16 * NG);      // chunk of 8 head dims
-  const bool vact = tid < C::VUNITS;
-  // position of this key group inside the permuted 64-key row of its sub-tile's V^T
-  const int vsub = vkg >> 4;
-  const int vpos = ((vkg >> 3) & 1) * 32 + ((vkg >> 2) & 1) * 16 + (vkg & 1) * 8 + ((vkg >> 1) & 1) * 4;
+  // ---- global -> register -> LDS staging of one K / V sub-tile by the group's 256 threads ----
+  const int kc = tg % C::CPR;
+  const int kr = tg / C::CPR;
+  const int vkg = tg & 15;  // group of 4 consecutive keys
+  const int vdc = tg >> 4;  // chunk of 8 head dims
+  const bool vact = tg < C::VUNITS;
+  // position of this key group inside the permuted 64-key row of V^T
+  const int vpos = (vkg >> 3) * 32 + ((vkg >> 2) & 1) * 16 + (vkg & 1) * 8 + ((vkg >> 1) & 1) * 4;
+  // Loads are formed as (wave-uniform 64-bit base) + (per-lane 32-bit byte offset): the base
+  // moves with the sub-tile, the lane offset never changes.
+  const unsigned kvoff = (unsigned)((kr * p.ks.s + kc * 8) * (int64_t)sizeof(T));
+  const unsigned vvoff = (unsigned)((vkg * 4 * p.vs.s + vdc * 8) * (int64_t)sizeof(T));
+  const int64_t kpass = (int64_t)C::RPP * p.ks.s * (int64_t)sizeof(T);
+  const int64_t vrow = p.vs.s * (int64_t)sizeof(T);
 
-  u32x4 kreg[C::KPASS];
-  u32x4 vreg[4];
-
-  auto gload = [&](int it) {
-    const int key0 = it * TILE;
+  auto gload_k = [&](int i, u32x4 (&kreg)[C::KPASS]) {
+    if (i >= n) return;
+    const int k0 = key_of(i);
+    if (k0 + FWD_BN <= p.Sk) {
+      const char* base = (const char*)kp + (int64_t)k0 * p.ks.s * (int64_t)sizeof(T);
 #pragma unroll
-    for (int i = 0; i < C::KPASS; ++i) {
-      int r = key0 + kr + i * C::RPP;
-      r = r < p.Sk ? r : p.Sk - 1;
-      kreg[i] = *(const u32x4*)(kp + (int64_t)r * p.ks.s + kc * 8);
+      for (int j = 0; j < C::KPASS; ++j) kreg[j] = *(const u32x4*)(base + j * kpass + kvoff);
+    } else {  // ragged tail: rows past the last key re-read the last key (masked later)
+#pragma unroll
+      for (int j = 0; j < C::KPASS; ++j) {
+        int r = k0 + kr + j * C::RPP;
+        r = r < p.Sk ? r : p.Sk - 1;
+        kreg[j] = *(const u32x4*)(kp + (int64_t)r * p.ks.s + kc * 8);
+      }
     }
-    if (vact) {
+  };
+  auto gload_v = [&](int i, u32x4 (&vreg)[4]) {
+    if (i >= n || !vact) return;
+    const int k0 = key_of(i);
+    if (k0 + FWD_BN <= p.Sk) {
+      const char* base = (const char*)vp + (int64_t)k0 * p.vs.s * (int64_t)sizeof(T);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) vreg[j] = *(const u32x4*)(base + j * vrow + vvoff);
+    } else {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        int r = key0 + vkg * 4 + j;
+        int r = k0 + vkg * 4 + j;
         r = r < p.Sk ? r : p.Sk - 1;
         vreg[j] = *(const u32x4*)(vp + (int64_t)r * p.vs.s + vdc * 8);
       }
     }
   };
-
-  auto lstore = [&](int stage) {
-    unsigned char* sb = smem + stage * C::STAGE;
+  auto lstore_k = [&](int i, const u32x4 (&kreg)[C::KPASS]) {
+    if (i >= n) return;
+    unsigned char* kb = kbuf(i);
 #pragma unroll
-    for (int i = 0; i < C::KPASS; ++i) {
-      const int r = kr + i * C::RPP;
-      *(u32x4*)(sb + (r >> 6) * C::SUB + (r & 63) * C::KP + kc * 16) = kreg[i];
+    for (int j = 0; j < C::KPASS; ++j) *(u32x4*)(kb + (kr + j * C::RPP) * C::KP + kc * 16) = kreg[j];
+  };
+  auto lstore_v = [&](int i, const u32x4 (&vreg)[4]) {
+    if (i >= n || !vact) return;
+    unsigned char* vb = vbuf(i);
+    // 4 keys x 8 dims in registers -> 8 rows (dims) of 4 consecutive keys
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const unsigned a0 = vreg[0][m], a1 = vreg[1][m], a2 = vreg[2][m], a3 = vreg[3][m];
+      u32x2 even, odd;
+      even[0] = __builtin_amdgcn_perm(a1, a0, 0x05040100u);  // lo16(a0) | lo16(a1) << 16
+      even[1] = __builtin_amdgcn_perm(a3, a2, 0x05040100u);
+      odd[0] = __builtin_amdgcn_perm(a1, a0, 0x07060302u);   // hi16(a0) | hi16(a1) << 16
+      odd[1] = __builtin_amdgcn_perm(a3, a2, 0x07060302u);
+      *(u32x2*)(vb + (vdc * 8 + 2 * m) * C::VP + vpos * 2) = even;
+      *(u32x2*)(vb + (vdc * 8 + 2 * m + 1) * C::VP + vpos * 2) = odd;
     }
-    if (vact) {
-      unsigned char* vb = sb + vsub * C::SUB + C::KBYTES;
-      // 4 keys x 8 dims in registers -> 8 rows (dims) of 4 consecutive keys
+  };
+
+  f32x16 s[2];
+  auto mma_s = [&](int i) {  // S(i)^T = K(i) Q^T
+    const unsigned char* kb = kbuf(i);
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        const unsigned a0 = vreg[0][m], a1 = vreg[1][m], a2 = vreg[2][m], a3 = vreg[3][m];
-        u32x2 even, odd;
-        even[0] = (a0 & 0xffffu) | (a1 << 16);
-        even[1] = (a2 & 0xffffu) | (a3 << 16);
-        odd[0] = (a0 >> 16) | (a1 & 0xffff0000u);
-        odd[1] = (a2 >> 16) | (a3 & 0xffff0000u);
-        *(u32x2*)(vb + (vdc * 8 + 2 * m) * C::VP + vpos * 2) = even;
-        *(u32x2*)(vb + (vdc * 8 + 2 * m + 1) * C::VP + vpos * 2) = odd;
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s[t][v] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks) {
+        const frag a = as_frag<frag>(*(const u32x4*)(kb + (t * 32 + ln) * C::KP + (ks * 16 + hh * 8) * 2));
+        s[t] = M::run(a, qf[ks], s[t]);
       }
     }
   };
@@ -153,151 +192,292 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     for (int v = 0; v < 16; ++v) o[i][v] = 0.f;
   float m_run = -INFINITY;  // reference row max of the raw scores (may lag the true max, see below)
   float l_run = 0.f;        // this lane's share of the running row sum
-
-  gload(0);
-  lstore(0);
-  __syncthreads();
-
   const float c = p.scale_log2;
 
-  for (int it = 0; it < nt; ++it) {
-    const int cur = it & 1;
-    const int key0 = it * TILE + grp * FWD_BN;
-    const bool more = it + 1 < nt;
-    if (more) gload(it + 1);
-
-    // a wave whose rows all precede its sub-tile, or whose sub-tile lies past the keys, idles
-    const bool active = key0 < kv_end && !(p.causal && key0 > qw0 + 31);
-    if (active) {
-      const unsigned char* kb = smem + cur * C::STAGE + grp * C::SUB;
-      const unsigned char* vb = kb + C::KBYTES;
-
-      f32x16 s[2];
+  // MFMA phase of step i: O += V(i)^T P(i) (if PV) followed by S(i+1) = K(i+1) Q^T (if NS).
+  // The LDS operand of MFMA number j is fetched LOOK MFMAs ahead of its use, so the whole
+  // phase runs off a rolling window of LOOK fragments instead of stalling on every read.
+  auto mfma_phase = [&](auto do_pv, auto do_s, int i, frag (&pfr)[2][2]) {
+    constexpr bool PV = decltype(do_pv)::value, NS = decltype(do_s)::value;
+    constexpr int NPV = PV ? (D / 32) * 4 : 0;
+    constexpr int NSS = NS ? (D / 16) * 2 : 0;
+    constexpr int TOTAL = NPV + NSS;
+    constexpr int LOOK = 8;
+    const unsigned char* vb = vbuf(i) + ln * C::VP + hh * 16;
+    const unsigned char* kb = kbuf(i + 1) + ln * C::KP + hh * 16;
+    auto fetch = [&](int j) -> frag {
+      if (j < NPV) {  // j = (t*2+u)*(D/32) + db : consecutive MFMAs hit different accumulators
+        const int db = j % (D / 32), tu = j / (D / 32);
+        return as_frag<frag>(*(const u32x4*)(vb + db * 32 * C::VP + tu * 32));
+      }
+      const int jj = j - NPV;  // jj = ks*2 + t
+      const int t = jj & 1, ks = jj >> 1;
+      return as_frag<frag>(*(const u32x4*)(kb + t * 32 * C::KP + ks * 32));
+    };
+    frag win[LOOK];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+    for (int j = 0; j < LOOK && j < TOTAL; ++j) win[j] = fetch(j);
+    // scheduling fences keep the compiler from sinking each read back next to its use
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) s[t][v] = 0.f;
+    for (int j = 0; j < TOTAL; ++j) {
+      const frag a = win[j % LOOK];
+      if (j + LOOK < TOTAL) win[j % LOOK] = fetch(j + LOOK);
+      __builtin_amdgcn_sched_barrier(0);
+      if (j < NPV) {
+        const int db = j % (D / 32), tu = j / (D / 32);
+        o[db] = M::run(a, pfr[tu >> 1][tu & 1], o[db]);
+      } else {
+        const int jj = j - NPV;
+        const int t = jj & 1, ks = jj >> 1;
+        if (ks == 0) {
+          f32x16 z;
 #pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) {
-          const frag a = as_frag<frag>(*(const u32x4*)(kb + (t * 32 + ln) * C::KP + (ks * 16 + hh * 8) * 2));
+          for (int v = 0; v < 16; ++v) z[v] = 0.f;
+          s[t] = M::run(a, qf[0], z);
+        } else {
           s[t] = M::run(a, qf[ks], s[t]);
         }
       }
+    }
+  };
 
-      const bool need_mask = (p.causal && key0 + FWD_BN - 1 > qw0) || (key0 + FWD_BN > p.Sk);
-      if (need_mask) {
-        const int lim = p.causal ? (qrow < p.Sk - 1 ? qrow : p.Sk - 1) : p.Sk - 1;  // last visible key
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int key = key0 + t * 32 + 8 * (v >> 2) + 4 * hh + (v & 3);
-            if (key > lim) s[t][v] = -INFINITY;
-          }
-      }
-
-      float mx = s[0][0];
-#pragma unroll
-      for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[0][v]);
-#pragma unroll
-      for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[1][v]);
-      mx = fmaxf(mx, xhalf(mx));
-      // Lazy rescale: the reference max only moves when some row's max grew by more than
-      // 2^8 in the exp2 domain; until then P <= 256, harmless in fp32 sums and bf16 operands.
-      if (__builtin_amdgcn_ballot_w64((mx - m_run) * c > 8.f) != 0) {
-        const float m_new = fmaxf(m_run, mx);
-        const float alpha = fast_exp2((m_run - m_new) * c);
-        m_run = m_new;
-        l_run *= alpha;
-#pragma unroll
-        for (int i = 0; i < D / 32; ++i)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
-      }
-      const float mc = m_run * c;
-
-      float ps = 0.f;
+  // VALU phase of step i: softmax of S(i) -> P(i) as MFMA operands, O rescaled if needed.
+  auto softmax_phase = [&](int i, frag (&pfr)[2][2]) {
+    const int key0 = key_of(i);
+    const bool need_mask = (p.causal && key0 + FWD_BN - 1 > qw0) || (key0 + FWD_BN > p.Sk);
+    if (need_mask) {
+      const int lim = p.causal ? (qrow < p.Sk - 1 ? qrow : p.Sk - 1) : p.Sk - 1;  // last visible key
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const float e = fast_exp2(__builtin_fmaf(s[t][v], c, -mc));
-          s[t][v] = e;
-          ps += e;
+          const int key = key0 + t * 32 + 8 * (v >> 2) + 4 * hh + (v & 3);
+          if (key > lim) s[t][v] = -INFINITY;
         }
-      l_run += ps;
-
-      frag pf[2][2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-          pf[t][u] = M::pack(s[t][8 * u + 0], s[t][8 * u + 1], s[t][8 * u + 2], s[t][8 * u + 3],
-                             s[t][8 * u + 4], s[t][8 * u + 5], s[t][8 * u + 6], s[t][8 * u + 7]);
-
-#pragma unroll
-      for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int u = 0; u < 2; ++u) {
-            const frag a = as_frag<frag>(
-                *(const u32x4*)(vb + (db * 32 + ln) * C::VP + (t * 32 + u * 16 + hh * 8) * 2));
-            o[db] = M::run(a, pf[t][u], o[db]);
-          }
     }
 
-    if (more) lstore(cur ^ 1);
-    __syncthreads();
-  }
-
-  // ---- combine the wave groups: groups 1.. hand (O, m, l) to group 0 through LDS ----
-  if (NG > 1) {
-    float* xch = (float*)smem;  // [w][slot][lane], slot = D/2 accumulators, then m, then l
-    constexpr int SLOTS = D / 2 + 2;
-    if (grp == 1) {
-      float* dst = xch + (w * SLOTS) * 64 + lane;
+    float mx = s[0][0];
 #pragma unroll
-      for (int i = 0; i < D / 32; ++i)
+    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[0][v]);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) dst[(i * 16 + v) * 64] = o[i][v];
-      dst[(D / 2) * 64] = m_run;
-      dst[(D / 2 + 1) * 64] = l_run;
-    }
-    __syncthreads();
-    if (grp == 0) {
-      const float* src = xch + (w * SLOTS) * 64 + lane;
-      const float m1 = src[(D / 2) * 64];
-      const float l1 = src[(D / 2 + 1) * 64];
-      const float m_new = fmaxf(m_run, m1);  // finite: group 0 always sees key 0
-      const float a0 = fast_exp2((m_run - m_new) * c);
-      const float a1 = fast_exp2((m1 - m_new) * c);
+    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[1][v]);
+    mx = fmaxf(mx, xhalf(mx));
+    // Lazy rescale: the reference max only moves when some row's max grew by more than
+    // 2^8 in the exp2 domain; until then P <= 256, harmless in fp32 sums and bf16 operands.
+    if (__builtin_amdgcn_ballot_w64((mx - m_run) * c > 8.f) != 0) {
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = fast_exp2((m_run - m_new) * c);
       m_run = m_new;
-      l_run = l_run * a0 + l1 * a1;
+      l_run *= alpha;
 #pragma unroll
-      for (int i = 0; i < D / 32; ++i)
+      for (int d = 0; d < D / 32; ++d)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) o[i][v] = o[i][v] * a0 + src[(i * 16 + v) * 64] * a1;
+        for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
     }
+    const float mc = m_run * c;
+
+    float ps = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const float e = fast_exp2(__builtin_fmaf(s[t][v], c, -mc));
+        s[t][v] = e;
+        ps += e;
+      }
+    l_run += ps;
+    asm volatile("" : "+v"(l_run));  // keep the row sum in this phase as well (see below)
+
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+        pfr[t][u] = M::pack(s[t][8 * u + 0], s[t][8 * u + 1], s[t][8 * u + 2], s[t][8 * u + 3],
+                            s[t][8 * u + 4], s[t][8 * u + 5], s[t][8 * u + 6], s[t][8 * u + 7]);
+    // P must exist in registers when the phase ends: without this the compiler sinks the
+    // exponentials past the barrier into the MFMA phase they are meant to overlap with.
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        u32x4 x = __builtin_bit_cast(u32x4, pfr[t][u]);
+        asm volatile("" : "+v"(x));
+        pfr[t][u] = __builtin_bit_cast(frag, x);
+      }
+  };
+
+  // Sub-tiles in which this wave has work form a prefix 0..n_act-1 of the group's n sub-tiles:
+  // a sub-tile is idle for the wave when it lies past the keys or after all of the wave's rows.
+  int n_act;
+  {
+    int last_key = kv_end - 1;
+    if (p.causal && qw0 + 31 < last_key) last_key = qw0 + 31;
+    const int last_sub = last_key / FWD_BN;
+    n_act = last_sub >= grp ? (last_sub - grp) / NG + 1 : 0;
+    n_act = n_act < n ? n_act : n;
   }
 
-  // ---- epilogue: normalise, store out and lse ----
-  if (grp == 0) {
-    const float l_tot = l_run + xhalf(l_run);
-    const float inv = 1.f / l_tot;
-    if (qrow < p.Sq) {
-      T* op = (T*)p.out + b * p.os.b + h * p.os.h + (int64_t)qrow * p.os.s;
+  // ---- prologue: one round trip for Q, K(0), V(0), K(1); then K(2) / V(1) on their way ----
+  u32x4 kreg[C::KPASS];
+  u32x4 vreg[4];
+  {
+    u32x4 k1[C::KPASS];
+    gload_k(0, kreg);
+    gload_v(0, vreg);
+    gload_k(1, k1);
+    lstore_k(0, kreg);
+    lstore_v(0, vreg);
+    lstore_k(1, k1);
+  }
+  gload_k(2, kreg);
+  gload_v(1, vreg);
+  __syncthreads();
+  if (n_act > 0) mma_s(0);
+  __syncthreads();
+  if (NG > 1 && grp == 1) __syncthreads();  // group 1 runs one phase behind group 0
+
+  // Every wave executes the same 2n barriers; the loop bodies hold no branch around an MFMA.
+  int i = 0;
+  for (; i + 1 < n_act; ++i) {
+    frag pf[2][2];
+    softmax_phase(i, pf);
+    lstore_k(i + 2, kreg);  // into the buffer S(i) was read from
+    lstore_v(i + 1, vreg);  // into the buffer P(i-1) V(i-1) was read from
+    __syncthreads();
+    gload_k(i + 3, kreg);  // in flight across this MFMA phase and the next softmax
+    gload_v(i + 2, vreg);
+    __builtin_amdgcn_s_setprio(1);
+    mfma_phase(std::true_type{}, std::true_type{}, i, pf);
+    __builtin_amdgcn_s_setprio(0);
+    __syncthreads();
+  }
+  if (i < n_act) {  // the wave's last sub-tile: nothing to prepare for a next one
+    frag pf[2][2];
+    softmax_phase(i, pf);
+    lstore_k(i + 2, kreg);
+    lstore_v(i + 1, vreg);
+    __syncthreads();
+    gload_k(i + 3, kreg);
+    gload_v(i + 2, vreg);
+    mfma_phase(std::true_type{}, std::false_type{}, i, pf);
+    __syncthreads();
+    ++i;
+  }
+  for (; i < n; ++i) {  // idle sub-tiles: keep staging for the other waves of the group
+    lstore_k(i + 2, kreg);
+    lstore_v(i + 1, vreg);
+    __syncthreads();
+    gload_k(i + 3, kreg);
+    gload_v(i + 2, vreg);
+    __syncthreads();
+  }
+  if (NG > 1 && grp == 0) __syncthreads();  // matches group 1's leading barrier
+
+  // ---- epilogue ----
+  // The groups exchange only (m, l) per row; each scales its own partial O by
+  // exp2((m - m_all) c) / l_all and stages it as fp32 rows in LDS (free now); then all
+  // waves walk the 128 x D tile row-major, add the groups' partials and write full rows:
+  // 16-byte coalesced stores instead of 8-byte pieces scattered over 32 rows per wave.
+  // A ring step's merge with the running (acc, lse) happens in the same pass (p.epi).
+  constexpr int TP = D + 4;  // floats per staged row
+  float* const tile = (float*)smem + grp * (FWD_BM * TP);
+  float* const ml = (float*)smem + NG * FWD_BM * TP;  // [NG][128](m, l), then lse_b[128]
+  float* const lsb = ml + NG * FWD_BM * 2;
+  const int rloc = w * 32 + ln;
+  const float l_own = l_run + xhalf(l_run);
+  float scale, lse_b;
+  if (NG > 1) {
+    if (hh == 0) {
+      ml[(grp * FWD_BM + rloc) * 2] = m_run;
+      ml[(grp * FWD_BM + rloc) * 2 + 1] = l_own;
+    }
+    __syncthreads();
+    const float m2 = ml[((grp ^ 1) * FWD_BM + rloc) * 2];
+    const float l2 = ml[((grp ^ 1) * FWD_BM + rloc) * 2 + 1];
+    const float m_all = fmaxf(m_run, m2);  // finite: group 0 always sees key 0
+    const float a1 = fast_exp2((m_run - m_all) * c);
+    const float a2 = fast_exp2((m2 - m_all) * c);
+    const float l_all = l_own * a1 + l2 * a2;
+    scale = a1 / l_all;
+    lse_b = (m_all * c + fast_log2(l_all)) * 0.6931471805599453f;
+  } else {
+    scale = 1.f / l_own;
+    lse_b = (m_run * c + fast_log2(l_own)) * 0.6931471805599453f;
+  }
 #pragma unroll
-      for (int db = 0; db < D / 32; ++db)
+  for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          u32x2 st;
-          st[0] = M::pack2(o[db][4 * g + 0] * inv, o[db][4 * g + 1] * inv);
-          st[1] = M::pack2(o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv);
-          *(u32x2*)(op + db * 32 + 8 * g + 4 * hh) = st;
+    for (int g = 0; g < 4; ++g) {
+      f32x4 st;
+      st[0] = o[db][4 * g + 0] * scale;
+      st[1] = o[db][4 * g + 1] * scale;
+      st[2] = o[db][4 * g + 2] * scale;
+      st[3] = o[db][4 * g + 3] * scale;
+      *(f32x4*)(tile + rloc * TP + db * 32 + 8 * g + 4 * hh) = st;
+    }
+  if (grp == 0 && hh == 0) lsb[rloc] = lse_b;
+  __syncthreads();
+  {
+    constexpr int CH = D / 8;  // 8-element chunks per row; the CH lanes of a row share a wave
+    const float* t0 = (const float*)smem;
+    const int epi = p.epi;
+    for (int cidx = tid; cidx < FWD_BM * CH; cidx += FWD_THREADS * NG) {
+      const int row = cidx / CH, ch = cidx % CH;
+      const int grow = q0 + row;
+      if (grow >= p.Sq) continue;
+      float x[8];
+      {
+        const f32x4 a = *(const f32x4*)(t0 + row * TP + ch * 8);
+        const f32x4 bq = *(const f32x4*)(t0 + row * TP + ch * 8 + 4);
+        x[0] = a[0]; x[1] = a[1]; x[2] = a[2]; x[3] = a[3];
+        x[4] = bq[0]; x[5] = bq[1]; x[6] = bq[2]; x[7] = bq[3];
+      }
+      if (NG > 1) {
+        const float* t1 = t0 + FWD_BM * TP;
+        const f32x4 a = *(const f32x4*)(t1 + row * TP + ch * 8);
+        const f32x4 bq = *(const f32x4*)(t1 + row * TP + ch * 8 + 4);
+        x[0] += a[0]; x[1] += a[1]; x[2] += a[2]; x[3] += a[3];
+        x[4] += bq[0]; x[5] += bq[1]; x[6] += bq[2]; x[7] += bq[3];
+      }
+      float lb = lsb[row];
+      const int64_t li = ((int64_t)b * p.H + h) * p.lse_bh + grow;
+      float* ap = p.acc + b * p.as.b + h * p.as.h + (int64_t)grow * p.as.s + ch * 8;
+      if (epi >= SPA_EPI_MERGE) {  // merge with the running accumulators (sp_aurora/utils.py:103-104)
+        const float la = p.lse[li];
+        const f32x4 a = *(const f32x4*)ap;
+        const f32x4 bq = *(const f32x4*)(ap + 4);
+        const float xa[8] = {a[0], a[1], a[2], a[3], bq[0], bq[1], bq[2], bq[3]};
+        const float d = lb - la;
+        float wgt, ln_;
+        if (d == d) {
+          const float e = __expf(-fabsf(d));
+          const float inv = 1.f / (1.f + e);
+          wgt = d >= 0.f ? inv : e * inv;  // sigmoid(lb - la)
+          ln_ = fmaxf(la, lb) + log1pf(e);
+        } else {
+          wgt = 0.f;
+          ln_ = la;
         }
-      if (hh == 0)
-        p.lse[((int64_t)b * p.H + h) * p.Sq + qrow] = (m_run * c + fast_log2(l_tot)) * 0.6931471805599453f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = xa[e] - wgt * (xa[e] - x[e]);
+        lb = ln_;
+      }
+      if (epi == SPA_EPI_INIT || epi == SPA_EPI_MERGE) {
+        f32x4 a, bq;
+        a[0] = x[0]; a[1] = x[1]; a[2] = x[2]; a[3] = x[3];
+        bq[0] = x[4]; bq[1] = x[5]; bq[2] = x[6]; bq[3] = x[7];
+        *(f32x4*)ap = a;
+        *(f32x4*)(ap + 4) = bq;
+      } else {
+        u32x4 st;
+        st[0] = M::pack2(x[0], x[1]);
+        st[1] = M::pack2(x[2], x[3]);
+        st[2] = M::pack2(x[4], x[5]);
+        st[3] = M::pack2(x[6], x[7]);
+        *(u32x4*)((T*)p.out + b * p.os.b + h * p.os.h + (int64_t)grow * p.os.s + ch * 8) = st;
+      }
+      if (ch == 0) p.lse[li] = lb;
     }
   }
 }
@@ -488,7 +668,7 @@ __global__ void __launch_bounds__(FWD_THREADS, 1) flash_fwd32_kernel(const FwdPa
         *(f32x4*)(op + db * 32 + 8 * g + 4 * hh) = st;
       }
     if (hh == 0)
-      p.lse[((int64_t)b * p.H + h) * p.Sq + qrow] = (m_run * c + fast_log2(l_tot)) * 0.6931471805599453f;
+      p.lse[((int64_t)b * p.H + h) * p.lse_bh + qrow] = (m_run * c + fast_log2(l_tot)) * 0.6931471805599453f;
   }
 }
 
@@ -527,6 +707,7 @@ hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t strea
     if (D == 64) return launch16<_Float16, 64>(p, stream);
     if (D == 32) return launch16<_Float16, 32>(p, stream);
   } else if (dtype == 0) {
+    if (p.epi != SPA_EPI_PLAIN) return hipErrorInvalidValue;  // fp32 ring steps merge with the separate kernel
     if (D == 128) return launch(flash_fwd32_kernel<128>, FWD_THREADS, Fwd32Cfg<128>::SMEM, p, stream);
     if (D == 64) return launch(flash_fwd32_kernel<64>, FWD_THREADS, Fwd32Cfg<64>::SMEM, p, stream);
     if (D == 32) return launch(flash_fwd32_kernel<32>, FWD_THREADS, Fwd32Cfg<32>::SMEM, p, stream);

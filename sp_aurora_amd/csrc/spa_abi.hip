@@ -106,6 +106,10 @@ int spa_flash_fwd(const void* q, const void* k, const void* v, void* out, float*
   p.scale_log2 = scale * 1.4426950408889634f;
   p.causal = mask_mode == SPA_MASK_CAUSAL;
   p.nqt = 0;
+  p.lse_bh = Sq;
+  p.acc = nullptr;
+  p.as = S3(o_strides);
+  p.epi = SPA_EPI_PLAIN;
   return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), "spa_flash_fwd");
 }
 

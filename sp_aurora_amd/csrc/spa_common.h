@@ -26,6 +26,18 @@ struct FwdParams {
   float scale_log2;  // scale * log2(e)
   int causal;        // 1: query row i sees keys j <= i (top-left aligned)
   int nqt;           // number of query tiles per (batch, head)
+  int64_t lse_bh;    // elements between consecutive (batch, head) rows of lse
+  // ring-step epilogue (16-bit kernels): what happens to the block result
+  float* acc;        // fp32 running output, [B,H,Sq,D] by `as` (SPA_EPI_INIT/MERGE/FINAL)
+  Strides3 as;
+  int epi;
+};
+
+enum {
+  SPA_EPI_PLAIN = 0,  // out <- block, lse <- block lse
+  SPA_EPI_INIT = 1,   // acc <- block (fp32), lse <- block lse            (first of several steps)
+  SPA_EPI_MERGE = 2,  // (acc, lse) <- merge((acc, lse), block)            (middle step)
+  SPA_EPI_FINAL = 3   // out <- cast(merge((acc, lse), block)), lse <- merged lse (last step)
 };
 
 struct BwdParams {
