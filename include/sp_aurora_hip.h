@@ -93,6 +93,27 @@ int spa_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* 
               const int64_t acc_strides[3], const int64_t blk_strides[3],
               int blk_dtype, int init, void* stream);
 
+/*
+ * Ring forward of rank `rank` (or of every rank, rank = -1) on ONE device that holds the whole
+ * sequence: q, k, v, out are [B,H,S,D] by strides, split into P contiguous chunks of s = S/P
+ * rows; lse is fp32 contiguous [B,H,S].  For rank r, step t = 0..P-1 uses KV chunk
+ * (r - t) mod P, is computed iff (mask_mode == SPA_MASK_NONE or t <= r), carries the causal
+ * mask iff (mask_mode == SPA_MASK_CAUSAL and t == 0), and is merged into the running
+ * (out, lse) in step order — the loop of intel_ring_flash_attn_forward
+ * (sp_aurora/intel_ring_flash_attn.py:72-148) with update_out_and_lse (sp_aurora/utils.py:103-104)
+ * folded into the epilogue of each block kernel for 16-bit types (fp32 uses spa_merge /
+ * spa_finalize kernels between steps).  One block-attention launch per visited (q chunk, kv
+ * chunk) pair; no collectives: the "ring" is the order in which the chunks are visited.
+ * workspace: device scratch of spa_ring_fwd_workspace_bytes() bytes (16-byte aligned), owned
+ * by the caller; it holds the fp32 running output of one rank between steps.
+ */
+int64_t spa_ring_fwd_workspace_bytes(int B, int H, int S, int D, int P, int dtype);
+int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
+                 int B, int H, int S, int D, int P, int rank,
+                 const int64_t q_strides[3], const int64_t k_strides[3],
+                 const int64_t v_strides[3], const int64_t o_strides[3],
+                 float scale, int mask_mode, int dtype, void* stream);
+
 /* out = cast(out_acc) — the `out.to(q.dtype)` that closes a ring forward
  * (sp_aurora/intel_ring_flash_attn.py:141-143). */
 int spa_finalize(void* out, const float* out_acc,

@@ -82,13 +82,14 @@ __global__ void __launch_bounds__(256) merge_kernel(float* __restrict__ out_acc,
                                                     const T* __restrict__ blk_out,
                                                     const float* __restrict__ blk_lse, int H, int Sq,
                                                     int cpr /* D/8 */, int64_t nrows, Strides3 as,
-                                                    Strides3 bs) {
+                                                    Strides3 bs, int64_t acc_lse_bh) {
   const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t row = gid / cpr;
   const int ch = (int)(gid % cpr);
   if (row >= nrows) return;
   const RowIdx r = decode_row(row, H, Sq);
-  const int64_t li = ((int64_t)r.b * H + r.h) * Sq + r.s;
+  const int64_t li = ((int64_t)r.b * H + r.h) * Sq + r.s;          // block lse: contiguous [B,H,Sq]
+  const int64_t la_i = ((int64_t)r.b * H + r.h) * acc_lse_bh + r.s;  // running lse: row pitch acc_lse_bh
   float* ap = out_acc + r.b * as.b + r.h * as.h + (int64_t)r.s * as.s + ch * 8;
   const T* bp = blk_out + r.b * bs.b + r.h * bs.h + (int64_t)r.s * bs.s + ch * 8;
   float xb[8];
@@ -96,10 +97,10 @@ __global__ void __launch_bounds__(256) merge_kernel(float* __restrict__ out_acc,
   const float lb = blk_lse[li];
   if (INIT) {
     Load8<float>::st(ap, xb);
-    if (ch == 0) lse_acc[li] = lb;
+    if (ch == 0) lse_acc[la_i] = lb;
     return;
   }
-  const float la = lse_acc[li];
+  const float la = lse_acc[la_i];
   float xa[8];
   Load8<float>::ld(ap, xa);
   // w = sigmoid(lb - la); lse' = max + log1p(exp(-|lb - la|))
@@ -117,7 +118,7 @@ __global__ void __launch_bounds__(256) merge_kernel(float* __restrict__ out_acc,
 #pragma unroll
   for (int i = 0; i < 8; ++i) xa[i] = xa[i] - w * (xa[i] - xb[i]);
   Load8<float>::st(ap, xa);
-  if (ch == 0) lse_acc[li] = ln;
+  if (ch == 0) lse_acc[la_i] = ln;
 }
 
 template <typename T>
@@ -159,14 +160,14 @@ __global__ void __launch_bounds__(256) delta_kernel(const T* __restrict__ out, c
 
 hipError_t spa_launch_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* blk_lse, int B,
                             int H, int Sq, int D, Strides3 as, Strides3 bs, int dtype, int init,
-                            hipStream_t stream) {
+                            int64_t acc_lse_bh, hipStream_t stream) {
   const int cpr = D / 8;
   const int64_t nrows = (int64_t)B * H * Sq;
   const int64_t nthreads = nrows * cpr;
   const dim3 grid((unsigned)((nthreads + 255) / 256));
 #define SPA_MERGE(T, I)                                                                              \
   hipLaunchKernelGGL((merge_kernel<T, I>), grid, dim3(256), 0, stream, out_acc, lse_acc, (const T*)blk_out, \
-                     blk_lse, H, Sq, cpr, nrows, as, bs)
+                     blk_lse, H, Sq, cpr, nrows, as, bs, acc_lse_bh)
   if (dtype == 0) { if (init) SPA_MERGE(float, true); else SPA_MERGE(float, false); }
   else if (dtype == 1) { if (init) SPA_MERGE(__bf16, true); else SPA_MERGE(__bf16, false); }
   else if (dtype == 2) { if (init) SPA_MERGE(_Float16, true); else SPA_MERGE(_Float16, false); }

@@ -12,7 +12,7 @@ hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t strea
 hipError_t spa_launch_flash_bwd(BwdParams p, int D, int dtype, hipStream_t stream);
 hipError_t spa_launch_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* blk_lse, int B,
                             int H, int Sq, int D, Strides3 as, Strides3 bs, int dtype, int init,
-                            hipStream_t stream);
+                            int64_t acc_lse_bh, hipStream_t stream);
 hipError_t spa_launch_finalize(void* out, const float* out_acc, int B, int H, int Sq, int D, Strides3 os,
                                Strides3 as, int dtype, hipStream_t stream);
 hipError_t spa_launch_delta(const void* out, const void* dout, float* delta, int B, int H, int Sq, int D,
@@ -125,8 +125,104 @@ int spa_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* 
     return fail(SPA_EALIGN, "spa_merge: pointers and row strides must be 16-byte aligned");
   if ((int64_t)B * H * Sq * (D / 8) / 256 > 0x7ffffff0LL) return fail(SPA_EINVAL, "spa_merge: grid too large");
   return launch_result(spa_launch_merge(out_acc, lse_acc, blk_out, blk_lse, B, H, Sq, D, S3(acc_strides),
-                                        S3(blk_strides), blk_dtype, init, (hipStream_t)stream),
+                                        S3(blk_strides), blk_dtype, init, Sq, (hipStream_t)stream),
                        "spa_merge");
+}
+
+int64_t spa_ring_fwd_workspace_bytes(int B, int H, int S, int D, int P, int dtype) {
+  if (B <= 0 || H <= 0 || S <= 0 || D <= 0 || P <= 0 || S % P != 0 || !dtype_ok(dtype)) return -1;
+  const int64_t s = S / P;
+  const int64_t acc = (int64_t)B * s * H * D * 4;
+  if (dtype != SPA_F32) return acc;
+  // fp32: running output, one block's output, one block's lse
+  return 2 * acc + (int64_t)B * H * s * 4;
+}
+
+int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace, int B,
+                 int H, int S, int D, int P, int rank, const int64_t q_strides[3], const int64_t k_strides[3],
+                 const int64_t v_strides[3], const int64_t o_strides[3], float scale, int mask_mode, int dtype,
+                 void* stream) {
+  if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "spa_ring_fwd: null pointer");
+  if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(SPA_EINVAL, "spa_ring_fwd: null strides");
+  if (!dims_ok(B, H, S, D)) return fail(SPA_EINVAL, "spa_ring_fwd: sizes must be positive");
+  if (P <= 0 || S % P != 0) return fail(SPA_EINVAL, "spa_ring_fwd: ring size %d must divide the sequence length %d", P, S);
+  if (rank < -1 || rank >= P) return fail(SPA_EINVAL, "spa_ring_fwd: rank %d outside [-1, %d)", rank, P);
+  if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "spa_ring_fwd: bad dtype %d", dtype);
+  if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "spa_ring_fwd: bad mask_mode %d", mask_mode);
+  if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "spa_ring_fwd: softmax scale must be positive and finite");
+  if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "spa_ring_fwd: head dim %d not in {32,64,128}", D);
+  const int esz = elem_size(dtype);
+  if (!aligned16(q, q_strides, esz) || !aligned16(k, k_strides, esz) || !aligned16(v, v_strides, esz) ||
+      !aligned16(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0 || ((uintptr_t)workspace & 15) != 0)
+    return fail(SPA_EALIGN, "spa_ring_fwd: pointers and row strides must be 16-byte aligned");
+  const bool causal = mask_mode == SPA_MASK_CAUSAL;
+  const int s = S / P;
+  const bool multi = P > 1 && (!causal || rank != 0);  // does some rank visit more than one block?
+  if (multi && !workspace) return fail(SPA_EINVAL, "spa_ring_fwd: workspace required when a rank visits several blocks");
+  if ((int64_t)B * H * ((s + 127) / 128) > 0x7fffffffLL) return fail(SPA_EINVAL, "spa_ring_fwd: grid too large");
+  hipStream_t st = (hipStream_t)stream;
+
+  // workspace carve-up; the running output is laid out [B, s, H, D]
+  float* acc = (float*)workspace;
+  const int64_t acc_elems = (int64_t)B * s * H * D;
+  Strides3 as;
+  as.b = (int64_t)s * H * D; as.h = D; as.s = (int64_t)H * D;
+  float* blk_out = acc + acc_elems;      // fp32 path only
+  float* blk_lse = blk_out + acc_elems;  // fp32 path only
+
+  FwdParams p;
+  p.B = B; p.H = H; p.Sq = s; p.Sk = s;
+  p.qs = S3(q_strides); p.ks = S3(k_strides); p.vs = S3(v_strides); p.os = S3(o_strides);
+  p.scale = scale;
+  p.scale_log2 = scale * 1.4426950408889634f;
+  p.nqt = 0;
+  p.lse_bh = S;
+  p.acc = acc;
+  p.as = as;
+
+  const int r_lo = rank < 0 ? 0 : rank, r_hi = rank < 0 ? P : rank + 1;
+  for (int r = r_lo; r < r_hi; ++r) {
+    const int nsteps = causal ? r + 1 : P;
+    const char* qr = (const char*)q + (int64_t)r * s * p.qs.s * esz;
+    char* outr = (char*)out + (int64_t)r * s * p.os.s * esz;
+    float* lser = lse + (int64_t)r * s;
+    for (int t = 0; t < nsteps; ++t) {
+      const int c = ((r - t) % P + P) % P;
+      p.q = qr;
+      p.k = (const char*)k + (int64_t)c * s * p.ks.s * esz;
+      p.v = (const char*)v + (int64_t)c * s * p.vs.s * esz;
+      p.causal = causal && t == 0;
+      p.lse = lser;
+      p.lse_bh = S;
+      hipError_t e;
+      if (dtype != SPA_F32) {
+        p.out = outr;
+        p.epi = nsteps == 1 ? SPA_EPI_PLAIN : t == 0 ? SPA_EPI_INIT : t + 1 == nsteps ? SPA_EPI_FINAL : SPA_EPI_MERGE;
+        e = spa_launch_flash_fwd(p, D, dtype, st);
+      } else if (nsteps == 1) {
+        p.out = outr;
+        p.epi = SPA_EPI_PLAIN;
+        e = spa_launch_flash_fwd(p, D, dtype, st);
+      } else {
+        // fp32: block result into scratch, then the stand-alone merge kernel
+        FwdParams pb = p;
+        pb.out = blk_out;
+        pb.os = as;
+        pb.lse = blk_lse;
+        pb.lse_bh = s;
+        pb.epi = SPA_EPI_PLAIN;
+        e = spa_launch_flash_fwd(pb, D, dtype, st);
+        if (e == hipSuccess)
+          e = spa_launch_merge(acc, lser, blk_out, blk_lse, B, H, s, D, as, as, SPA_F32, t == 0, S, st);
+        if (e == hipSuccess && t + 1 == nsteps) {
+          Strides3 os = p.os;
+          e = spa_launch_finalize(outr, acc, B, H, s, D, os, as, SPA_F32, st);
+        }
+      }
+      if (e != hipSuccess) return launch_result(e, "spa_ring_fwd");
+    }
+  }
+  return SPA_OK;
 }
 
 int spa_finalize(void* out, const float* out_acc, int B, int H, int Sq, int D, const int64_t o_strides[3],

@@ -76,6 +76,49 @@ def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None
     return out, lse
 
 
+def ring_fwd_workspace(q, ring_size, layout="bshd"):
+    """Scratch tensor spa_ring_fwd needs for this q and ring size (uint8, 16-byte aligned)."""
+    lib = _lib.load()
+    (B, H, S, D), _ = _bhs(q, layout)
+    nbytes = lib.spa_ring_fwd_workspace_bytes(B, H, S, D, int(ring_size), _dtype_code(q))
+    if nbytes < 0:
+        raise ValueError(f"ring_size={ring_size} must divide the sequence length {S}")
+    return torch.empty((nbytes,), dtype=torch.uint8, device=q.device)
+
+
+def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layout="bshd", out=None, lse=None,
+             workspace=None):
+    """Simulated ring forward of one rank (or all, rank=-1) over the full-sequence q,k,v: one C call
+    that enqueues every block-pair kernel in ring order.  Calls spa_ring_fwd.
+    Returns (out like q, lse fp32 [B,H,S]); with rank >= 0 only that rank's rows are written."""
+    lib = _lib.load()
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise TypeError("q, k, v must share a dtype")
+    (B, H, S, D), qs = _bhs(q, layout)
+    shp_k, ks = _bhs(k, layout)
+    shp_v, vs = _bhs(v, layout)
+    if shp_k != (B, H, S, D) or shp_v != (B, H, S, D):
+        raise ValueError(f"ring attention needs q, k, v of one shape, got {tuple(q.shape)} {tuple(k.shape)} {tuple(v.shape)}")
+    if softmax_scale is None:
+        softmax_scale = D ** (-0.5)
+    if out is None:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    if lse is None:
+        lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
+    if workspace is None:
+        workspace = ring_fwd_workspace(q, ring_size, layout)
+    _, os_ = _bhs(out, layout)
+    with torch.cuda.device(q.device):
+        _lib.check(lib.spa_ring_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), workspace.data_ptr(),
+            B, H, S, D, int(ring_size), int(rank),
+            _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
+            float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE,
+            _dtype_code(q), _stream()))
+    return out, lse
+
+
 def merge(out_acc, lse_acc, blk_out, blk_lse, layout="bshd", init=False):
     """In-place merge of (blk_out, blk_lse) into fp32 (out_acc, lse_acc).  Calls spa_merge."""
     lib = _lib.load()

@@ -44,12 +44,14 @@ class _RingWorkspace:
         self.blk_out = torch.empty((B, s, H, D), dtype=dtype, device=device)
         self.blk_lse = torch.empty((B, H, s), dtype=torch.float32, device=device)
         self.acc = torch.empty((B, s, H, D), dtype=torch.float32, device=device)
-        self.lse_r = torch.empty((B, H, s), dtype=torch.float32, device=device)
 
 
 def ring_flash_attn_forward_rank(q_local, k_chunks, v_chunks, rank, softmax_scale=None, causal=False,
                                  out=None, lse=None, workspace=None):
-    """What rank `rank` of a ring of P = len(k_chunks) computes, on this GPU.
+    """What rank `rank` of a ring of P = len(k_chunks) computes, on this GPU, spelled out with the
+    stand-alone kernels: block attention, then update_out_and_lse as its own pass, per step.
+    (ring_flash_attn_forward reaches the same result through the C ring driver, which folds the
+    merge into the attention kernel's epilogue.)
 
     Step t uses KV chunk (rank - t) mod P; it is computed iff `not causal or t <= rank`
     and carries the diagonal mask iff `causal and t == 0`
@@ -82,27 +84,18 @@ def ring_flash_attn_forward_rank(q_local, k_chunks, v_chunks, rank, softmax_scal
 
 def ring_flash_attn_forward(q, k, v, softmax_scale=None, causal=False, ring_size=1, out=None, lse=None,
                             workspace=None):
-    """All ranks of a simulated ring over contiguous shards of q,k,v [B,S,H,D].
-    Returns out [B,S,H,D] (q dtype) and lse fp32 [B,H,S]; `out`, `lse`, `workspace` may be
-    passed in to run without allocating."""
+    """All ranks of a simulated ring over contiguous shards of q,k,v [B,S,H,D]: one call into the
+    C ring driver, which enqueues the block-pair kernels in ring order and merges each step in the
+    kernel epilogue.  Returns out [B,S,H,D] (q dtype) and lse fp32 [B,H,S]; `out`, `lse`,
+    `workspace` (ops.ring_fwd_workspace) may be passed in to run without allocating."""
     B, S, H, D = q.shape
     P = int(ring_size)
     if P < 1 or S % P or (P > 1 and k.shape[1] != S):
         raise ValueError(f"ring_size={P} must divide the sequence length {S} (and k/v must match q)")
     if P == 1:
         return ops.flash_fwd(q, k, v, softmax_scale, causal, layout="bshd", out=out, lse=lse)
-    s = S // P
-    if out is None:
-        out = torch.empty((B, S, H, D), dtype=q.dtype, device=q.device)
-    if lse is None:
-        lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
-    ks, vs = list(k.split(s, dim=1)), list(v.split(s, dim=1))
-    ws = workspace or _RingWorkspace(B, s, H, D, q.dtype, q.device)
-    for r in range(P):
-        ring_flash_attn_forward_rank(q[:, r * s:(r + 1) * s], ks, vs, r, softmax_scale, causal,
-                                     out=out[:, r * s:(r + 1) * s], lse=ws.lse_r, workspace=ws)
-        lse[:, :, r * s:(r + 1) * s] = ws.lse_r
-    return out, lse
+    return ops.ring_fwd(q, k, v, P, softmax_scale, causal, rank=-1, layout="bshd", out=out, lse=lse,
+                        workspace=workspace)
 
 
 def make_ring_forward_step(q, k, v, softmax_scale=None, causal=False, ring_size=1):
@@ -112,7 +105,7 @@ def make_ring_forward_step(q, k, v, softmax_scale=None, causal=False, ring_size=
     P = int(ring_size)
     out = torch.empty((B, S, H, D), dtype=q.dtype, device=q.device)
     lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
-    ws = _RingWorkspace(B, S // P, H, D, q.dtype, q.device) if P > 1 else None
+    ws = ops.ring_fwd_workspace(q, P) if P > 1 else None
 
     def step():
         return ring_flash_attn_forward(q, k, v, softmax_scale, causal, P, out=out, lse=lse, workspace=ws)

@@ -372,3 +372,31 @@ def test_delta_kernel():
     got = ops.bwd_delta(o.to(DEV), do.to(DEV))
     want = (o.double() * do.double()).sum(-1).transpose(1, 2)
     assert torch.allclose(got.cpu().double(), want, atol=1e-4, rtol=1e-5)
+
+
+# ------------------------------------------------------------------ C ring driver
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+def test_ring_driver_matches_stepwise_path_and_oracle(causal, dtype):
+    """spa_ring_fwd (merge fused into the kernel epilogue) against the step-by-step path through
+    spa_flash_fwd + spa_merge + spa_finalize, and against the oracle's ring schedule; also a single
+    rank, as BASELINE config 2 runs it."""
+    P, B, s, H, D = 4, 2, 160, 3, 64
+    q, k, v = rand_qkv((B, P * s, H, D), 110, dtype)
+    dq, dk, dv = q.to(DEV), k.to(DEV), v.to(DEV)
+    out, lse = ops.ring_fwd(dq, dk, dv, P, None, causal)
+    want_out, want_lse = O.ring_forward(q, k, v, P, None, causal, out_dtype=torch.float64)
+    check_out(out, want_out, dtype)
+    check_lse(lse, want_lse)
+    ks, vs = list(dk.split(s, 1)), list(dv.split(s, 1))
+    for r in range(P):
+        o_r, l_r = spa.ring_flash_attn_forward_rank(dq[:, r * s:(r + 1) * s], ks, vs, r, None, causal)
+        tol = dict(atol=1e-6, rtol=1e-6) if dtype == torch.float32 else dict(atol=8e-3, rtol=8e-3)
+        assert torch.allclose(out[:, r * s:(r + 1) * s].float(), o_r.float(), **tol)
+        assert torch.allclose(lse[:, :, r * s:(r + 1) * s], l_r, atol=1e-5)
+    # one rank only: the other rows stay untouched
+    out2 = torch.full_like(out, 7.0)
+    lse2 = torch.full_like(lse, 7.0)
+    ops.ring_fwd(dq, dk, dv, P, None, causal, rank=2, out=out2, lse=lse2)
+    assert torch.equal(out2[:, 2 * s:3 * s], out[:, 2 * s:3 * s]) and torch.equal(lse2[:, :, 2 * s:3 * s], lse[:, :, 2 * s:3 * s])
+    assert (out2[:, :2 * s] == 7).all() and (out2[:, 3 * s:] == 7).all() and (lse2[:, :, :2 * s] == 7).all()
