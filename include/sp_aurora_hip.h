@@ -101,18 +101,27 @@ int spa_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* 
  * mask iff (mask_mode == SPA_MASK_CAUSAL and t == 0), and is merged into the running
  * (out, lse) in step order — the loop of intel_ring_flash_attn_forward
  * (sp_aurora/intel_ring_flash_attn.py:72-148) with update_out_and_lse (sp_aurora/utils.py:103-104)
- * folded into the epilogue of each block kernel for 16-bit types (fp32 uses spa_merge /
- * spa_finalize kernels between steps).  One block-attention launch per visited (q chunk, kv
- * chunk) pair; no collectives: the "ring" is the order in which the chunks are visited.
+ * folded into the block kernel for 16-bit types (fp32 uses spa_merge / spa_finalize kernels
+ * between steps).
+ * `fuse` chooses how the schedule maps onto launches (the results agree to rounding):
+ *   SPA_RING_PER_STEP   one block-attention launch per visited (q chunk, kv chunk) pair, as a
+ *                       multi-GPU ring would issue them; needs the workspace.
+ *   SPA_RING_PER_RANK   one launch per rank: a workgroup keeps its query tile and its output
+ *                       accumulators in registers and walks the rank's KV chunks in ring order,
+ *                       so the merge is the online softmax itself and no accumulator leaves the CU.
+ *   SPA_RING_ALL_RANKS  one launch for all requested ranks (heaviest first).
+ * fp32 always runs per step.  No collectives: the "ring" is the order in which chunks are visited.
  * workspace: device scratch of spa_ring_fwd_workspace_bytes() bytes (16-byte aligned), owned
- * by the caller; it holds the fp32 running output of one rank between steps.
+ * by the caller; it holds the fp32 running output of one rank between separate step launches
+ * (may be NULL for the fused modes).
  */
+enum { SPA_RING_PER_STEP = 0, SPA_RING_PER_RANK = 1, SPA_RING_ALL_RANKS = 2 };
 int64_t spa_ring_fwd_workspace_bytes(int B, int H, int S, int D, int P, int dtype);
 int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
                  int B, int H, int S, int D, int P, int rank,
                  const int64_t q_strides[3], const int64_t k_strides[3],
                  const int64_t v_strides[3], const int64_t o_strides[3],
-                 float scale, int mask_mode, int dtype, void* stream);
+                 float scale, int mask_mode, int dtype, int fuse, void* stream);
 
 /* out = cast(out_acc) — the `out.to(q.dtype)` that closes a ring forward
  * (sp_aurora/intel_ring_flash_attn.py:141-143). */

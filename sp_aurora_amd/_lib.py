@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, "libsp_aurora_hip.so")
 
 SPA_F32, SPA_BF16, SPA_F16 = 0, 1, 2
 SPA_MASK_NONE, SPA_MASK_CAUSAL = 0, 1
+SPA_RING_PER_STEP, SPA_RING_PER_RANK, SPA_RING_ALL_RANKS = 0, 1, 2
 
 _I64x3 = ctypes.c_int64 * 3
 _vp = ctypes.c_void_p
@@ -25,7 +26,7 @@ SIGNATURES = {
     "spa_device_info": (_i, [ctypes.c_char_p, _i]),
     "spa_flash_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _vp]),
     "spa_ring_fwd_workspace_bytes": (ctypes.c_int64, [_i, _i, _i, _i, _i, _i]),
-    "spa_ring_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _vp]),
+    "spa_ring_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _i, _vp]),
     "spa_merge": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _s3, _s3, _i, _i, _vp]),
     "spa_finalize": (_i, [_vp, _vp, _i, _i, _i, _i, _s3, _s3, _i, _vp]),
     "spa_relayout_s2h": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),

@@ -72,15 +72,19 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
 
   // Consecutive workgroup ids walk the heads first: with round-robin placement of
   // workgroups on the 8 XCDs, all query tiles of a head share one XCD's L2 for K/V.
+  // Then query tiles and ranks, heaviest first.
   int bid = blockIdx.x;
   const int h = bid % p.H;
   bid /= p.H;
-  const int qt = p.nqt - 1 - (bid % p.nqt);  // heaviest causal tiles first
-  const int b = bid / p.nqt;
+  const int qt = p.nqt - 1 - (bid % p.nqt);
+  bid /= p.nqt;
+  const int b = bid % p.B;
+  const int rank = p.rank0 + p.nranks - 1 - bid / p.B;
   const int q0 = qt * FWD_BM;
   const int qw0 = q0 + w * 32;
+  const int64_t qoff = (int64_t)rank * p.Sq;  // first row of this rank's query chunk
 
-  const T* qp = (const T*)p.q + b * p.qs.b + h * p.qs.h;
+  const T* qp = (const T*)p.q + b * p.qs.b + h * p.qs.h + qoff * p.qs.s;
   const T* kp = (const T*)p.k + b * p.ks.b + h * p.ks.h;
   const T* vp = (const T*)p.v + b * p.vs.b + h * p.vs.h;
 
@@ -92,10 +96,49 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   for (int ks = 0; ks < D / 16; ++ks)
     qf[ks] = as_frag<frag>(*(const u32x4*)(qp + (int64_t)qrow_c * p.qs.s + ks * 16 + hh * 8));
 
-  const int kv_end = p.causal ? (q0 + FWD_BM < p.Sk ? q0 + FWD_BM : p.Sk) : p.Sk;
-  const int n = (kv_end + FWD_BN * NG - 1) / (FWD_BN * NG);  // sub-tiles per group
-  // first key of this group's i-th sub-tile
-  auto key_of = [&](int i) { return (i * NG + grp) * FWD_BN; };
+  // ---- the schedule of this workgroup ----
+  // K/V hold P chunks of Sk keys.  Ring step t of rank r uses chunk (r - t) mod P; a causal ring
+  // has steps 0..r and masks step 0 (the rank's own chunk) only.  The launch covers steps
+  // [t_begin, t_end) of that schedule; a plain block call is P = 1, one step.
+  // A group's work is a sequence of 64-key sub-tiles: first those of the masked (diagonal)
+  // chunk up to the last key any row of the workgroup sees, then every full chunk.
+  constexpr int TILE = FWD_BN * NG;
+  const int nsteps = p.causal ? (rank + 1 < p.P ? rank + 1 : p.P) : p.P;
+  const int t_end = p.t_count < 0 || p.t_begin + p.t_count > nsteps ? nsteps : p.t_begin + p.t_count;
+  const bool diag = p.causal && p.t_begin == 0;
+  const int kv_end = q0 + FWD_BM < p.Sk ? q0 + FWD_BM : p.Sk;  // keys of the diagonal chunk in use
+  const int n_diag = diag ? (kv_end + TILE - 1) / TILE : 0;
+  const int npc = (p.Sk + TILE - 1) / TILE;                    // sub-tiles per full chunk
+  const int t_full0 = p.t_begin + (diag ? 1 : 0);              // first unmasked step
+  const int n = n_diag + (t_end - t_full0 > 0 ? (t_end - t_full0) * npc : 0);
+
+  struct Sub {
+    int krel;   // first key of the sub-tile, relative to its chunk
+    int krow;   // the same as a row of the K/V tensors
+    int kend;   // one past the chunk's last row
+    bool masked;
+  };
+  auto locate = [&](int i) {
+    Sub r;
+    int t, j;
+    if (i < n_diag) {
+      t = 0;
+      j = i;
+      r.masked = true;
+    } else {
+      const int x = i - n_diag;
+      const int tt = x / npc;
+      t = t_full0 + tt;
+      j = x - tt * npc;
+      r.masked = false;
+    }
+    int ch = (rank - t) % p.P;
+    ch = ch < 0 ? ch + p.P : ch;
+    r.krel = (j * NG + grp) * FWD_BN;
+    r.krow = ch * p.Sk + r.krel;
+    r.kend = ch * p.Sk + p.Sk;
+    return r;
+  };
   unsigned char* gbase = smem + grp * C::GROUP;
   auto kbuf = [&](int i) { return gbase + (i & 1) * C::KBYTES; };
   auto vbuf = [&](int i) { return gbase + 2 * C::KBYTES + (i & 1) * C::VBYTES; };
@@ -117,32 +160,32 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
 
   auto gload_k = [&](int i, u32x4 (&kreg)[C::KPASS]) {
     if (i >= n) return;
-    const int k0 = key_of(i);
-    if (k0 + FWD_BN <= p.Sk) {
-      const char* base = (const char*)kp + (int64_t)k0 * p.ks.s * (int64_t)sizeof(T);
+    const Sub sb = locate(i);
+    if (sb.krow + FWD_BN <= sb.kend) {
+      const char* base = (const char*)kp + (int64_t)sb.krow * p.ks.s * (int64_t)sizeof(T);
 #pragma unroll
       for (int j = 0; j < C::KPASS; ++j) kreg[j] = *(const u32x4*)(base + j * kpass + kvoff);
-    } else {  // ragged tail: rows past the last key re-read the last key (masked later)
+    } else {  // ragged tail: rows past the chunk's last key re-read that key (masked later)
 #pragma unroll
       for (int j = 0; j < C::KPASS; ++j) {
-        int r = k0 + kr + j * C::RPP;
-        r = r < p.Sk ? r : p.Sk - 1;
+        int r = sb.krow + kr + j * C::RPP;
+        r = r < sb.kend ? r : sb.kend - 1;
         kreg[j] = *(const u32x4*)(kp + (int64_t)r * p.ks.s + kc * 8);
       }
     }
   };
   auto gload_v = [&](int i, u32x4 (&vreg)[4]) {
     if (i >= n || !vact) return;
-    const int k0 = key_of(i);
-    if (k0 + FWD_BN <= p.Sk) {
-      const char* base = (const char*)vp + (int64_t)k0 * p.vs.s * (int64_t)sizeof(T);
+    const Sub sb = locate(i);
+    if (sb.krow + FWD_BN <= sb.kend) {
+      const char* base = (const char*)vp + (int64_t)sb.krow * p.vs.s * (int64_t)sizeof(T);
 #pragma unroll
       for (int j = 0; j < 4; ++j) vreg[j] = *(const u32x4*)(base + j * vrow + vvoff);
     } else {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        int r = k0 + vkg * 4 + j;
-        r = r < p.Sk ? r : p.Sk - 1;
+        int r = sb.krow + vkg * 4 + j;
+        r = r < sb.kend ? r : sb.kend - 1;
         vreg[j] = *(const u32x4*)(vp + (int64_t)r * p.vs.s + vdc * 8);
       }
     }
@@ -244,10 +287,12 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
 
   // VALU phase of step i: softmax of S(i) -> P(i) as MFMA operands, O rescaled if needed.
   auto softmax_phase = [&](int i, frag (&pfr)[2][2]) {
-    const int key0 = key_of(i);
-    const bool need_mask = (p.causal && key0 + FWD_BN - 1 > qw0) || (key0 + FWD_BN > p.Sk);
+    const Sub sb = locate(i);
+    const int key0 = sb.krel;
+    const bool causal_here = sb.masked;
+    const bool need_mask = (causal_here && key0 + FWD_BN - 1 > qw0) || (key0 + FWD_BN > p.Sk);
     if (need_mask) {
-      const int lim = p.causal ? (qrow < p.Sk - 1 ? qrow : p.Sk - 1) : p.Sk - 1;  // last visible key
+      const int lim = causal_here ? (qrow < p.Sk - 1 ? qrow : p.Sk - 1) : p.Sk - 1;  // last visible key
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -275,7 +320,8 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
 #pragma unroll
         for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
     }
-    const float mc = m_run * c;
+    // a row that has seen no key yet (a ragged chunk can leave a whole sub-tile empty) keeps m = -inf
+    const float mc = m_run == -INFINITY ? 0.f : m_run * c;
 
     float ps = 0.f;
 #pragma unroll
@@ -307,17 +353,6 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       }
   };
 
-  // Sub-tiles in which this wave has work form a prefix 0..n_act-1 of the group's n sub-tiles:
-  // a sub-tile is idle for the wave when it lies past the keys or after all of the wave's rows.
-  int n_act;
-  {
-    int last_key = kv_end - 1;
-    if (p.causal && qw0 + 31 < last_key) last_key = qw0 + 31;
-    const int last_sub = last_key / FWD_BN;
-    n_act = last_sub >= grp ? (last_sub - grp) / NG + 1 : 0;
-    n_act = n_act < n ? n_act : n;
-  }
-
   // ---- prologue: one round trip for Q, K(0), V(0), K(1); then K(2) / V(1) on their way ----
   u32x4 kreg[C::KPASS];
   u32x4 vreg[4];
@@ -333,13 +368,14 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   gload_k(2, kreg);
   gload_v(1, vreg);
   __syncthreads();
-  if (n_act > 0) mma_s(0);
+  mma_s(0);
   __syncthreads();
   if (NG > 1 && grp == 1) __syncthreads();  // group 1 runs one phase behind group 0
 
-  // Every wave executes the same 2n barriers; the loop bodies hold no branch around an MFMA.
-  int i = 0;
-  for (; i + 1 < n_act; ++i) {
+  // One loop, no branch around an MFMA, the same two barriers per step for every wave.  A wave
+  // whose rows see none of a diagonal sub-tile's keys (at most the last two sub-tiles of the
+  // diagonal chunk) simply gets P = 0 from the mask.
+  for (int i = 0; i + 1 < n; ++i) {
     frag pf[2][2];
     softmax_phase(i, pf);
     lstore_k(i + 2, kreg);  // into the buffer S(i) was read from
@@ -352,24 +388,11 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     __builtin_amdgcn_s_setprio(0);
     __syncthreads();
   }
-  if (i < n_act) {  // the wave's last sub-tile: nothing to prepare for a next one
+  {  // last sub-tile: nothing to prepare behind it
     frag pf[2][2];
-    softmax_phase(i, pf);
-    lstore_k(i + 2, kreg);
-    lstore_v(i + 1, vreg);
+    softmax_phase(n - 1, pf);
     __syncthreads();
-    gload_k(i + 3, kreg);
-    gload_v(i + 2, vreg);
-    mfma_phase(std::true_type{}, std::false_type{}, i, pf);
-    __syncthreads();
-    ++i;
-  }
-  for (; i < n; ++i) {  // idle sub-tiles: keep staging for the other waves of the group
-    lstore_k(i + 2, kreg);
-    lstore_v(i + 1, vreg);
-    __syncthreads();
-    gload_k(i + 3, kreg);
-    gload_v(i + 2, vreg);
+    mfma_phase(std::true_type{}, std::false_type{}, n - 1, pf);
     __syncthreads();
   }
   if (NG > 1 && grp == 0) __syncthreads();  // matches group 1's leading barrier
@@ -395,7 +418,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     __syncthreads();
     const float m2 = ml[((grp ^ 1) * FWD_BM + rloc) * 2];
     const float l2 = ml[((grp ^ 1) * FWD_BM + rloc) * 2 + 1];
-    const float m_all = fmaxf(m_run, m2);  // finite: group 0 always sees key 0
+    const float m_all = fmaxf(m_run, m2);  // finite: some group has seen key 0 of the first chunk
     const float a1 = fast_exp2((m_run - m_all) * c);
     const float a2 = fast_exp2((m2 - m_all) * c);
     const float l_all = l_own * a1 + l2 * a2;
@@ -441,7 +464,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         x[4] += bq[0]; x[5] += bq[1]; x[6] += bq[2]; x[7] += bq[3];
       }
       float lb = lsb[row];
-      const int64_t li = ((int64_t)b * p.H + h) * p.lse_bh + grow;
+      const int64_t li = ((int64_t)b * p.H + h) * p.lse_bh + qoff + grow;
       float* ap = p.acc + b * p.as.b + h * p.as.h + (int64_t)grow * p.as.s + ch * 8;
       if (epi >= SPA_EPI_MERGE) {  // merge with the running accumulators (sp_aurora/utils.py:103-104)
         const float la = p.lse[li];
@@ -475,7 +498,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         st[1] = M::pack2(x[2], x[3]);
         st[2] = M::pack2(x[4], x[5]);
         st[3] = M::pack2(x[6], x[7]);
-        *(u32x4*)((T*)p.out + b * p.os.b + h * p.os.h + (int64_t)grow * p.os.s + ch * 8) = st;
+        *(u32x4*)((T*)p.out + b * p.os.b + h * p.os.h + (qoff + grow) * p.os.s + ch * 8) = st;
       }
       if (ch == 0) p.lse[li] = lb;
     }
@@ -676,7 +699,7 @@ template <typename K>
 hipError_t launch(K kernel, int threads, int smem, const FwdParams& p, hipStream_t stream) {
   hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return e;
-  const dim3 grid((unsigned)((int64_t)p.B * p.H * p.nqt));
+  const dim3 grid((unsigned)((int64_t)p.B * p.H * p.nqt * p.nranks));
   hipLaunchKernelGGL(kernel, grid, dim3(threads), smem, stream, p);
   return hipGetLastError();
 }

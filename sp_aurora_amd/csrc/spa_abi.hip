@@ -110,6 +110,7 @@ int spa_flash_fwd(const void* q, const void* k, const void* v, void* out, float*
   p.acc = nullptr;
   p.as = S3(o_strides);
   p.epi = SPA_EPI_PLAIN;
+  p.P = 1; p.rank0 = 0; p.nranks = 1; p.t_begin = 0; p.t_count = -1;
   return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), "spa_flash_fwd");
 }
 
@@ -141,7 +142,7 @@ int64_t spa_ring_fwd_workspace_bytes(int B, int H, int S, int D, int P, int dtyp
 int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace, int B,
                  int H, int S, int D, int P, int rank, const int64_t q_strides[3], const int64_t k_strides[3],
                  const int64_t v_strides[3], const int64_t o_strides[3], float scale, int mask_mode, int dtype,
-                 void* stream) {
+                 int fuse, void* stream) {
   if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "spa_ring_fwd: null pointer");
   if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(SPA_EINVAL, "spa_ring_fwd: null strides");
   if (!dims_ok(B, H, S, D)) return fail(SPA_EINVAL, "spa_ring_fwd: sizes must be positive");
@@ -149,6 +150,7 @@ int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* 
   if (rank < -1 || rank >= P) return fail(SPA_EINVAL, "spa_ring_fwd: rank %d outside [-1, %d)", rank, P);
   if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "spa_ring_fwd: bad dtype %d", dtype);
   if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "spa_ring_fwd: bad mask_mode %d", mask_mode);
+  if (fuse < SPA_RING_PER_STEP || fuse > SPA_RING_ALL_RANKS) return fail(SPA_EINVAL, "spa_ring_fwd: bad fuse mode %d", fuse);
   if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "spa_ring_fwd: softmax scale must be positive and finite");
   if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "spa_ring_fwd: head dim %d not in {32,64,128}", D);
   const int esz = elem_size(dtype);
@@ -157,12 +159,15 @@ int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* 
     return fail(SPA_EALIGN, "spa_ring_fwd: pointers and row strides must be 16-byte aligned");
   const bool causal = mask_mode == SPA_MASK_CAUSAL;
   const int s = S / P;
+  if (dtype == SPA_F32) fuse = SPA_RING_PER_STEP;  // the fp32 kernel handles one block pair per launch
   const bool multi = P > 1 && (!causal || rank != 0);  // does some rank visit more than one block?
-  if (multi && !workspace) return fail(SPA_EINVAL, "spa_ring_fwd: workspace required when a rank visits several blocks");
-  if ((int64_t)B * H * ((s + 127) / 128) > 0x7fffffffLL) return fail(SPA_EINVAL, "spa_ring_fwd: grid too large");
+  if (fuse == SPA_RING_PER_STEP && multi && !workspace)
+    return fail(SPA_EINVAL, "spa_ring_fwd: workspace required when steps are separate launches");
+  const int r_lo = rank < 0 ? 0 : rank, r_hi = rank < 0 ? P : rank + 1;
+  if ((int64_t)B * H * ((s + 127) / 128) * (r_hi - r_lo) > 0x7fffffffLL) return fail(SPA_EINVAL, "spa_ring_fwd: grid too large");
   hipStream_t st = (hipStream_t)stream;
 
-  // workspace carve-up; the running output is laid out [B, s, H, D]
+  // workspace carve-up; the running output of one rank is laid out [B, s, H, D]
   float* acc = (float*)workspace;
   const int64_t acc_elems = (int64_t)B * s * H * D;
   Strides3 as;
@@ -171,52 +176,65 @@ int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* 
   float* blk_lse = blk_out + acc_elems;  // fp32 path only
 
   FwdParams p;
+  p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
   p.B = B; p.H = H; p.Sq = s; p.Sk = s;
   p.qs = S3(q_strides); p.ks = S3(k_strides); p.vs = S3(v_strides); p.os = S3(o_strides);
   p.scale = scale;
   p.scale_log2 = scale * 1.4426950408889634f;
+  p.causal = causal;
   p.nqt = 0;
   p.lse_bh = S;
   p.acc = acc;
   p.as = as;
+  p.P = P;
+  p.epi = SPA_EPI_PLAIN;
 
-  const int r_lo = rank < 0 ? 0 : rank, r_hi = rank < 0 ? P : rank + 1;
+  if (fuse == SPA_RING_ALL_RANKS) {  // one launch: every requested rank, every step
+    p.rank0 = r_lo; p.nranks = r_hi - r_lo; p.t_begin = 0; p.t_count = -1;
+    return launch_result(spa_launch_flash_fwd(p, D, dtype, st), "spa_ring_fwd");
+  }
   for (int r = r_lo; r < r_hi; ++r) {
+    p.rank0 = r; p.nranks = 1;
+    if (fuse == SPA_RING_PER_RANK) {  // one launch per rank: the workgroup walks the rank's chunks
+      p.t_begin = 0; p.t_count = -1;
+      hipError_t e = spa_launch_flash_fwd(p, D, dtype, st);
+      if (e != hipSuccess) return launch_result(e, "spa_ring_fwd");
+      continue;
+    }
     const int nsteps = causal ? r + 1 : P;
-    const char* qr = (const char*)q + (int64_t)r * s * p.qs.s * esz;
-    char* outr = (char*)out + (int64_t)r * s * p.os.s * esz;
-    float* lser = lse + (int64_t)r * s;
     for (int t = 0; t < nsteps; ++t) {
-      const int c = ((r - t) % P + P) % P;
-      p.q = qr;
-      p.k = (const char*)k + (int64_t)c * s * p.ks.s * esz;
-      p.v = (const char*)v + (int64_t)c * s * p.vs.s * esz;
-      p.causal = causal && t == 0;
-      p.lse = lser;
-      p.lse_bh = S;
       hipError_t e;
       if (dtype != SPA_F32) {
-        p.out = outr;
+        p.t_begin = t; p.t_count = 1;
         p.epi = nsteps == 1 ? SPA_EPI_PLAIN : t == 0 ? SPA_EPI_INIT : t + 1 == nsteps ? SPA_EPI_FINAL : SPA_EPI_MERGE;
         e = spa_launch_flash_fwd(p, D, dtype, st);
-      } else if (nsteps == 1) {
-        p.out = outr;
-        p.epi = SPA_EPI_PLAIN;
-        e = spa_launch_flash_fwd(p, D, dtype, st);
       } else {
-        // fp32: block result into scratch, then the stand-alone merge kernel
+        // fp32: one plain block pair per launch on explicit chunk pointers, merged by the stand-alone kernels
+        const int c = ((r - t) % P + P) % P;
         FwdParams pb = p;
-        pb.out = blk_out;
-        pb.os = as;
-        pb.lse = blk_lse;
-        pb.lse_bh = s;
+        pb.P = 1; pb.rank0 = 0; pb.nranks = 1; pb.t_begin = 0; pb.t_count = -1;
+        pb.q = (const char*)q + (int64_t)r * s * p.qs.s * esz;
+        pb.k = (const char*)k + (int64_t)c * s * p.ks.s * esz;
+        pb.v = (const char*)v + (int64_t)c * s * p.vs.s * esz;
+        pb.causal = causal && t == 0;
         pb.epi = SPA_EPI_PLAIN;
-        e = spa_launch_flash_fwd(pb, D, dtype, st);
-        if (e == hipSuccess)
-          e = spa_launch_merge(acc, lser, blk_out, blk_lse, B, H, s, D, as, as, SPA_F32, t == 0, S, st);
-        if (e == hipSuccess && t + 1 == nsteps) {
-          Strides3 os = p.os;
-          e = spa_launch_finalize(outr, acc, B, H, s, D, os, as, SPA_F32, st);
+        char* outr = (char*)out + (int64_t)r * s * p.os.s * esz;
+        float* lser = lse + (int64_t)r * s;
+        if (nsteps == 1) {
+          pb.out = outr;
+          pb.lse = lser;
+          pb.lse_bh = S;
+          e = spa_launch_flash_fwd(pb, D, dtype, st);
+        } else {
+          pb.out = blk_out;
+          pb.os = as;
+          pb.lse = blk_lse;
+          pb.lse_bh = s;
+          e = spa_launch_flash_fwd(pb, D, dtype, st);
+          if (e == hipSuccess)
+            e = spa_launch_merge(acc, lser, blk_out, blk_lse, B, H, s, D, as, as, SPA_F32, t == 0, S, st);
+          if (e == hipSuccess && t + 1 == nsteps)
+            e = spa_launch_finalize(outr, acc, B, H, s, D, p.os, as, SPA_F32, st);
         }
       }
       if (e != hipSuccess) return launch_result(e, "spa_ring_fwd");

@@ -27,6 +27,10 @@ struct FwdParams {
   int causal;        // 1: query row i sees keys j <= i (top-left aligned)
   int nqt;           // number of query tiles per (batch, head)
   int64_t lse_bh;    // elements between consecutive (batch, head) rows of lse
+  // ring schedule (16-bit kernels): K/V hold P chunks of Sk keys, q/out/lse hold P chunks of Sq
+  // rows; the launch runs ranks rank0 .. rank0+nranks-1, each over steps [t_begin, t_begin+t_count)
+  // of its schedule (t_count < 0: to the end).  A plain block call is P = 1, rank 0, all steps.
+  int P, rank0, nranks, t_begin, t_count;
   // ring-step epilogue (16-bit kernels): what happens to the block result
   float* acc;        // fp32 running output, [B,H,Sq,D] by `as` (SPA_EPI_INIT/MERGE/FINAL)
   Strides3 as;

@@ -86,10 +86,14 @@ def ring_fwd_workspace(q, ring_size, layout="bshd"):
     return torch.empty((nbytes,), dtype=torch.uint8, device=q.device)
 
 
+RING_FUSE = {"step": _lib.SPA_RING_PER_STEP, "rank": _lib.SPA_RING_PER_RANK, "all": _lib.SPA_RING_ALL_RANKS}
+
+
 def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layout="bshd", out=None, lse=None,
-             workspace=None):
+             workspace=None, fuse="rank"):
     """Simulated ring forward of one rank (or all, rank=-1) over the full-sequence q,k,v: one C call
-    that enqueues every block-pair kernel in ring order.  Calls spa_ring_fwd.
+    that enqueues the kernels in ring order.  Calls spa_ring_fwd.  `fuse`: "step" = one launch per
+    (q chunk, kv chunk) pair, "rank" = one launch per rank walking its chunks, "all" = one launch.
     Returns (out like q, lse fp32 [B,H,S]); with rank >= 0 only that rank's rows are written."""
     lib = _lib.load()
     q, k, v = _prep(q), _prep(k), _prep(v)
@@ -106,16 +110,19 @@ def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layo
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     if lse is None:
         lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
-    if workspace is None:
+    if fuse not in RING_FUSE:
+        raise ValueError(f"fuse must be one of {sorted(RING_FUSE)}, got {fuse!r}")
+    if workspace is None and (fuse == "step" or q.dtype == torch.float32):
         workspace = ring_fwd_workspace(q, ring_size, layout)
     _, os_ = _bhs(out, layout)
     with torch.cuda.device(q.device):
         _lib.check(lib.spa_ring_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), workspace.data_ptr(),
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            workspace.data_ptr() if workspace is not None else None,
             B, H, S, D, int(ring_size), int(rank),
             _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
             float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE,
-            _dtype_code(q), _stream()))
+            _dtype_code(q), RING_FUSE[fuse], _stream()))
     return out, lse
 
 

@@ -83,7 +83,7 @@ def ring_flash_attn_forward_rank(q_local, k_chunks, v_chunks, rank, softmax_scal
 
 
 def ring_flash_attn_forward(q, k, v, softmax_scale=None, causal=False, ring_size=1, out=None, lse=None,
-                            workspace=None):
+                            workspace=None, fuse="rank"):
     """All ranks of a simulated ring over contiguous shards of q,k,v [B,S,H,D]: one call into the
     C ring driver, which enqueues the block-pair kernels in ring order and merges each step in the
     kernel epilogue.  Returns out [B,S,H,D] (q dtype) and lse fp32 [B,H,S]; `out`, `lse`,
@@ -95,10 +95,10 @@ def ring_flash_attn_forward(q, k, v, softmax_scale=None, causal=False, ring_size
     if P == 1:
         return ops.flash_fwd(q, k, v, softmax_scale, causal, layout="bshd", out=out, lse=lse)
     return ops.ring_fwd(q, k, v, P, softmax_scale, causal, rank=-1, layout="bshd", out=out, lse=lse,
-                        workspace=workspace)
+                        workspace=workspace, fuse=fuse)
 
 
-def make_ring_forward_step(q, k, v, softmax_scale=None, causal=False, ring_size=1):
+def make_ring_forward_step(q, k, v, softmax_scale=None, causal=False, ring_size=1, fuse="rank"):
     """Preallocates every buffer ring_flash_attn_forward needs and returns a zero-argument
     callable that runs the whole ring forward into them and returns (out, lse)."""
     B, S, H, D = q.shape
@@ -108,7 +108,7 @@ def make_ring_forward_step(q, k, v, softmax_scale=None, causal=False, ring_size=
     ws = ops.ring_fwd_workspace(q, P) if P > 1 else None
 
     def step():
-        return ring_flash_attn_forward(q, k, v, softmax_scale, causal, P, out=out, lse=lse, workspace=ws)
+        return ring_flash_attn_forward(q, k, v, softmax_scale, causal, P, out=out, lse=lse, workspace=ws, fuse=fuse)
 
     return step
 

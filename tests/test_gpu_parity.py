@@ -384,10 +384,14 @@ def test_ring_driver_matches_stepwise_path_and_oracle(causal, dtype):
     P, B, s, H, D = 4, 2, 160, 3, 64
     q, k, v = rand_qkv((B, P * s, H, D), 110, dtype)
     dq, dk, dv = q.to(DEV), k.to(DEV), v.to(DEV)
-    out, lse = ops.ring_fwd(dq, dk, dv, P, None, causal)
+    out, lse = ops.ring_fwd(dq, dk, dv, P, None, causal, fuse="step")
     want_out, want_lse = O.ring_forward(q, k, v, P, None, causal, out_dtype=torch.float64)
     check_out(out, want_out, dtype)
     check_lse(lse, want_lse)
+    for fuse in ("rank", "all"):  # one launch per rank / one launch in all: same schedule, merged in registers
+        o_f, l_f = ops.ring_fwd(dq, dk, dv, P, None, causal, fuse=fuse)
+        check_out(o_f, want_out, dtype, what=f"out[{fuse}]")
+        check_lse(l_f, want_lse)
     ks, vs = list(dk.split(s, 1)), list(dv.split(s, 1))
     for r in range(P):
         o_r, l_r = spa.ring_flash_attn_forward_rank(dq[:, r * s:(r + 1) * s], ks, vs, r, None, causal)
@@ -397,6 +401,18 @@ def test_ring_driver_matches_stepwise_path_and_oracle(causal, dtype):
     # one rank only: the other rows stay untouched
     out2 = torch.full_like(out, 7.0)
     lse2 = torch.full_like(lse, 7.0)
-    ops.ring_fwd(dq, dk, dv, P, None, causal, rank=2, out=out2, lse=lse2)
+    ops.ring_fwd(dq, dk, dv, P, None, causal, rank=2, out=out2, lse=lse2, fuse="step")
     assert torch.equal(out2[:, 2 * s:3 * s], out[:, 2 * s:3 * s]) and torch.equal(lse2[:, :, 2 * s:3 * s], lse[:, :, 2 * s:3 * s])
     assert (out2[:, :2 * s] == 7).all() and (out2[:, 3 * s:] == 7).all() and (lse2[:, :, :2 * s] == 7).all()
+
+
+@pytest.mark.parametrize("fuse", ["step", "rank", "all"])
+@pytest.mark.parametrize("P,B,s,H,D,causal", [(8, 1, 128, 2, 128, True), (3, 2, 200, 2, 64, True), (4, 1, 72, 3, 32, False),
+                                              (2, 1, 1024, 2, 128, True), (5, 1, 64, 1, 128, True)])
+def test_ring_driver_modes_on_awkward_shapes(P, B, s, H, D, causal, fuse):
+    """Chunk lengths that are not multiples of the key tile, odd ring sizes, many ranks."""
+    q, k, v = rand_qkv((B, P * s, H, D), 111, torch.bfloat16)
+    want_out, want_lse = O.full_attention(q, k, v, None, causal)
+    out, lse = ops.ring_fwd(q.to(DEV), k.to(DEV), v.to(DEV), P, None, causal, fuse=fuse)
+    check_out(out, want_out, torch.bfloat16)
+    check_lse(lse, want_lse)
