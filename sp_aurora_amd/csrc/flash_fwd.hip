@@ -151,44 +151,34 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const bool vact = tg < C::VUNITS;
   // position of this key group inside the permuted 64-key row of V^T
   const int vpos = (vkg >> 3) * 32 + ((vkg >> 2) & 1) * 16 + (vkg & 1) * 8 + ((vkg >> 1) & 1) * 4;
-  // Loads are formed as (wave-uniform 64-bit base) + (per-lane 32-bit byte offset): the base
-  // moves with the sub-tile, the lane offset never changes.
+  // K/V sub-tiles are fetched with buffer loads: a wave-uniform descriptor per tensor, a
+  // constant 32-bit byte offset per lane, a scalar byte offset per (sub-tile, pass) — no per-lane
+  // address arithmetic in the loop — and the hardware's range check instead of clamps: a row past
+  // the end of the tensor reads as zero, a row past the end of its chunk but inside the tensor
+  // reads the next chunk's data; both are keys >= Sk, which the softmax masks to P = 0.
   const unsigned kvoff = (unsigned)((kr * p.ks.s + kc * 8) * (int64_t)sizeof(T));
   const unsigned vvoff = (unsigned)((vkg * 4 * p.vs.s + vdc * 8) * (int64_t)sizeof(T));
-  const int64_t kpass = (int64_t)C::RPP * p.ks.s * (int64_t)sizeof(T);
-  const int64_t vrow = p.vs.s * (int64_t)sizeof(T);
+  const unsigned krow_b = (unsigned)(p.ks.s * (int64_t)sizeof(T));  // bytes per K row
+  const unsigned vrow_b = (unsigned)(p.vs.s * (int64_t)sizeof(T));
+  const int64_t rows_all = (int64_t)p.P * p.Sk;
+  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)kp, 0, (int)(unsigned)(((rows_all - 1) * p.ks.s + D) * (int64_t)sizeof(T)), 0x00020000);
+  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)vp, 0, (int)(unsigned)(((rows_all - 1) * p.vs.s + D) * (int64_t)sizeof(T)), 0x00020000);
 
   auto gload_k = [&](int i, u32x4 (&kreg)[C::KPASS]) {
     if (i >= n) return;
     const Sub sb = locate(i);
-    if (sb.krow + FWD_BN <= sb.kend) {
-      const char* base = (const char*)kp + (int64_t)sb.krow * p.ks.s * (int64_t)sizeof(T);
 #pragma unroll
-      for (int j = 0; j < C::KPASS; ++j) kreg[j] = *(const u32x4*)(base + j * kpass + kvoff);
-    } else {  // ragged tail: rows past the chunk's last key re-read that key (masked later)
-#pragma unroll
-      for (int j = 0; j < C::KPASS; ++j) {
-        int r = sb.krow + kr + j * C::RPP;
-        r = r < sb.kend ? r : sb.kend - 1;
-        kreg[j] = *(const u32x4*)(kp + (int64_t)r * p.ks.s + kc * 8);
-      }
-    }
+    for (int j = 0; j < C::KPASS; ++j)
+      kreg[j] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, kvoff, (sb.krow + j * C::RPP) * krow_b, 0);
   };
   auto gload_v = [&](int i, u32x4 (&vreg)[4]) {
     if (i >= n || !vact) return;
     const Sub sb = locate(i);
-    if (sb.krow + FWD_BN <= sb.kend) {
-      const char* base = (const char*)vp + (int64_t)sb.krow * p.vs.s * (int64_t)sizeof(T);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) vreg[j] = *(const u32x4*)(base + j * vrow + vvoff);
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        int r = sb.krow + vkg * 4 + j;
-        r = r < sb.kend ? r : sb.kend - 1;
-        vreg[j] = *(const u32x4*)(vp + (int64_t)r * p.vs.s + vdc * 8);
-      }
-    }
+    for (int j = 0; j < 4; ++j)
+      vreg[j] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, vvoff, (sb.krow + j) * vrow_b, 0);
   };
   auto lstore_k = [&](int i, const u32x4 (&kreg)[C::KPASS]) {
     if (i >= n) return;

@@ -55,6 +55,11 @@ bool dims_ok(int B, int H, int S, int D) { return B > 0 && H > 0 && S > 0 && D >
 
 bool pow2_8_512(int D) { return D >= 8 && D <= 512 && (D & (D - 1)) == 0; }
 
+// The 16-bit forward kernel addresses K and V of one (batch, head) through 32-bit buffer offsets.
+bool span_ok(int64_t rows, int64_t row_stride, int D, int esz) {
+  return ((rows - 1) * row_stride + D) * esz < 0x7fffffffLL;
+}
+
 int launch_result(hipError_t e, const char* what) {
   if (e == hipSuccess) return SPA_OK;
   if (e == hipErrorInvalidValue) return fail(SPA_EUNSUPPORTED, "%s: no kernel for this head dim / dtype", what);
@@ -98,6 +103,8 @@ int spa_flash_fwd(const void* q, const void* k, const void* v, void* out, float*
       !aligned16(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0)
     return fail(SPA_EALIGN, "spa_flash_fwd: pointers and row strides must be 16-byte aligned");
   if ((int64_t)B * H * ((Sq + 127) / 128) > 0x7fffffffLL) return fail(SPA_EINVAL, "spa_flash_fwd: grid too large");
+  if (!span_ok(Sk, k_strides[2], D, esz) || !span_ok(Sk, v_strides[2], D, esz))
+    return fail(SPA_EUNSUPPORTED, "spa_flash_fwd: K/V of one (batch, head) span more than 2 GiB");
   FwdParams p;
   p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
   p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
@@ -157,6 +164,8 @@ int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* 
   if (!aligned16(q, q_strides, esz) || !aligned16(k, k_strides, esz) || !aligned16(v, v_strides, esz) ||
       !aligned16(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0 || ((uintptr_t)workspace & 15) != 0)
     return fail(SPA_EALIGN, "spa_ring_fwd: pointers and row strides must be 16-byte aligned");
+  if (!span_ok(S, k_strides[2], D, esz) || !span_ok(S, v_strides[2], D, esz))
+    return fail(SPA_EUNSUPPORTED, "spa_ring_fwd: K/V of one (batch, head) span more than 2 GiB");
   const bool causal = mask_mode == SPA_MASK_CAUSAL;
   const int s = S / P;
   if (dtype == SPA_F32) fuse = SPA_RING_PER_STEP;  // the fp32 kernel handles one block pair per launch
