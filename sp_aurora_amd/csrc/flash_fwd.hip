@@ -139,6 +139,45 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     r.kend = ch * p.Sk + p.Sk;
     return r;
   };
+  // The loop walks the sub-tiles in order with three cursors (softmax at i, V loads at i+2,
+  // K loads at i+3); a cursor steps without divisions.
+  struct Cursor {
+    int i, j, t;
+    Sub sb;
+  };
+  auto cursor_at = [&](int i) {
+    Cursor c;
+    c.i = i;
+    if (i < n_diag) {
+      c.t = 0;
+      c.j = i;
+    } else {
+      const int x = i - n_diag;
+      const int tt = x / npc;
+      c.t = t_full0 + tt;
+      c.j = x - tt * npc;
+    }
+    c.sb = locate(i);
+    return c;
+  };
+  auto cursor_next = [&](Cursor& c) {
+    ++c.i;
+    ++c.j;
+    if (c.i == n_diag) {
+      c.j = 0;
+      c.t = t_full0;
+    } else if (c.i > n_diag && c.j == npc) {
+      c.j = 0;
+      ++c.t;
+    }
+    int ch = rank - c.t;
+    ch = ch < 0 ? ch + p.P : ch;
+    ch = ch < 0 ? 0 : ch;  // only past the end of the schedule, where nothing is used
+    c.sb.masked = c.i < n_diag;
+    c.sb.krel = (c.j * NG + grp) * FWD_BN;
+    c.sb.krow = ch * p.Sk + c.sb.krel;
+    c.sb.kend = ch * p.Sk + p.Sk;
+  };
   unsigned char* gbase = smem + grp * C::GROUP;
   auto kbuf = [&](int i) { return gbase + (i & 1) * C::KBYTES; };
   auto vbuf = [&](int i) { return gbase + 2 * C::KBYTES + (i & 1) * C::VBYTES; };
@@ -179,6 +218,18 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       vreg[j] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, vvoff, (sb.krow + j) * vrow_b, 0);
+  };
+  auto gload_k_at = [&](const Cursor& c, u32x4 (&kreg)[C::KPASS]) {
+    if (c.i >= n) return;
+#pragma unroll
+    for (int j = 0; j < C::KPASS; ++j)
+      kreg[j] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, kvoff, (c.sb.krow + j * C::RPP) * krow_b, 0);
+  };
+  auto gload_v_at = [&](const Cursor& c, u32x4 (&vreg)[4]) {
+    if (c.i >= n || !vact) return;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      vreg[j] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, vvoff, (c.sb.krow + j) * vrow_b, 0);
   };
   auto lstore_k = [&](int i, const u32x4 (&kreg)[C::KPASS]) {
     if (i >= n) return;
@@ -276,8 +327,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   };
 
   // VALU phase of step i: softmax of S(i) -> P(i) as MFMA operands, O rescaled if needed.
-  auto softmax_phase = [&](int i, frag (&pfr)[2][2]) {
-    const Sub sb = locate(i);
+  auto softmax_phase = [&](const Sub& sb, frag (&pfr)[2][2]) {
     const int key0 = sb.krel;
     const bool causal_here = sb.masked;
     const bool need_mask = (causal_here && key0 + FWD_BN - 1 > qw0) || (key0 + FWD_BN > p.Sk);
@@ -365,22 +415,26 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // One loop, no branch around an MFMA, the same two barriers per step for every wave.  A wave
   // whose rows see none of a diagonal sub-tile's keys (at most the last two sub-tiles of the
   // diagonal chunk) simply gets P = 0 from the mask.
+  Cursor cs = cursor_at(0), cv = cursor_at(2), ck = cursor_at(3);
   for (int i = 0; i + 1 < n; ++i) {
     frag pf[2][2];
-    softmax_phase(i, pf);
+    softmax_phase(cs.sb, pf);
     lstore_k(i + 2, kreg);  // into the buffer S(i) was read from
     lstore_v(i + 1, vreg);  // into the buffer P(i-1) V(i-1) was read from
     __syncthreads();
-    gload_k(i + 3, kreg);  // in flight across this MFMA phase and the next softmax
-    gload_v(i + 2, vreg);
+    gload_k_at(ck, kreg);  // K(i+3), V(i+2): in flight across this MFMA phase and the next softmax
+    gload_v_at(cv, vreg);
     __builtin_amdgcn_s_setprio(1);
     mfma_phase(std::true_type{}, std::true_type{}, i, pf);
     __builtin_amdgcn_s_setprio(0);
+    cursor_next(cs);
+    cursor_next(cv);
+    cursor_next(ck);
     __syncthreads();
   }
   {  // last sub-tile: nothing to prepare behind it
     frag pf[2][2];
-    softmax_phase(n - 1, pf);
+    softmax_phase(cs.sb, pf);
     __syncthreads();
     mfma_phase(std::true_type{}, std::false_type{}, n - 1, pf);
     __syncthreads();
