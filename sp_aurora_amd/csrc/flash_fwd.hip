@@ -255,20 +255,6 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   };
 
   f32x16 s[2];
-  auto mma_s = [&](int i) {  // S(i)^T = K(i) Q^T
-    const unsigned char* kb = kbuf(i);
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-#pragma unroll
-      for (int v = 0; v < 16; ++v) s[t][v] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks) {
-        const frag a = as_frag<frag>(*(const u32x4*)(kb + (t * 32 + ln) * C::KP + (ks * 16 + hh * 8) * 2));
-        s[t] = M::run(a, qf[ks], s[t]);
-      }
-    }
-  };
-
   f32x16 o[D / 32];
 #pragma unroll
   for (int i = 0; i < D / 32; ++i)
@@ -342,11 +328,17 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         }
     }
 
-    float mx = s[0][0];
+    // four independent chains instead of one 32-long dependent one
+    float mxa = fmaxf(s[0][0], s[0][1]), mxb = fmaxf(s[0][8], s[0][9]);
+    float mxc = fmaxf(s[1][0], s[1][1]), mxd = fmaxf(s[1][8], s[1][9]);
 #pragma unroll
-    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[0][v]);
-#pragma unroll
-    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[1][v]);
+    for (int v = 2; v < 8; v += 2) {
+      mxa = fmaxf(fmaxf(mxa, s[0][v]), s[0][v + 1]);
+      mxb = fmaxf(fmaxf(mxb, s[0][v + 8]), s[0][v + 9]);
+      mxc = fmaxf(fmaxf(mxc, s[1][v]), s[1][v + 1]);
+      mxd = fmaxf(fmaxf(mxd, s[1][v + 8]), s[1][v + 9]);
+    }
+    float mx = fmaxf(fmaxf(mxa, mxb), fmaxf(mxc, mxd));
     mx = fmaxf(mx, xhalf(mx));
     // Lazy rescale: the reference max only moves when some row's max grew by more than
     // 2^8 in the exp2 domain; until then P <= 256, harmless in fp32 sums and bf16 operands.
@@ -363,16 +355,16 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     // a row that has seen no key yet (a ragged chunk can leave a whole sub-tile empty) keeps m = -inf
     const float mc = m_run == -INFINITY ? 0.f : m_run * c;
 
-    float ps = 0.f;
+    float ps[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const float e = fast_exp2(__builtin_fmaf(s[t][v], c, -mc));
         s[t][v] = e;
-        ps += e;
+        ps[v & 3] += e;
       }
-    l_run += ps;
+    l_run += (ps[0] + ps[1]) + (ps[2] + ps[3]);
     asm volatile("" : "+v"(l_run));  // keep the row sum in this phase as well (see below)
 
 #pragma unroll
@@ -408,7 +400,10 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   gload_k(2, kreg);
   gload_v(1, vreg);
   __syncthreads();
-  mma_s(0);
+  {
+    frag none[2][2];
+    mfma_phase(std::false_type{}, std::true_type{}, -1, none);  // S(0), operands prefetched through the window
+  }
   __syncthreads();
   if (NG > 1 && grp == 1) __syncthreads();  // group 1 runs one phase behind group 0
 
