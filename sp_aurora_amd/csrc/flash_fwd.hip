@@ -190,13 +190,18 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const bool vact = tg < C::VUNITS;
   // position of this key group inside the permuted 64-key row of V^T
   const int vpos = (vkg >> 3) * 32 + ((vkg >> 2) & 1) * 16 + (vkg & 1) * 8 + ((vkg >> 1) & 1) * 4;
-  // K/V sub-tiles are fetched with buffer loads: a wave-uniform descriptor per tensor, a
-  // constant 32-bit byte offset per lane, a scalar byte offset per (sub-tile, pass) — no per-lane
-  // address arithmetic in the loop — and the hardware's range check instead of clamps: a row past
-  // the end of the tensor reads as zero, a row past the end of its chunk but inside the tensor
-  // reads the next chunk's data; both are keys >= Sk, which the softmax masks to P = 0.
+  // K/V sub-tiles are fetched with buffer loads: a wave-uniform descriptor per tensor and a 32-bit
+  // byte offset per lane (a lane constant plus the sub-tile's uniform row offset: one add per load),
+  // and the hardware's range check instead of clamps and branches: a row past the end of the tensor
+  // reads as zero, a row past the end of its chunk but inside the tensor reads the next chunk's
+  // data; both are keys >= Sk, which the softmax masks to P = 0.  The range check covers the
+  // per-lane offset only, so the whole offset travels there and the scalar offset stays 0; a load
+  // that must not happen (past the end of the schedule, a lane without a share of V) gets an
+  // offset beyond any tensor and returns zeros (both at once wrap to offset 0: the tensor's first
+  // bytes, valid memory, never used).
+  constexpr unsigned OFF_NONE = 0x80000000u;
   const unsigned kvoff = (unsigned)((kr * p.ks.s + kc * 8) * (int64_t)sizeof(T));
-  const unsigned vvoff = (unsigned)((vkg * 4 * p.vs.s + vdc * 8) * (int64_t)sizeof(T));
+  const unsigned vvoff = vact ? (unsigned)((vkg * 4 * p.vs.s + vdc * 8) * (int64_t)sizeof(T)) : OFF_NONE;
   const unsigned krow_b = (unsigned)(p.ks.s * (int64_t)sizeof(T));  // bytes per K row
   const unsigned vrow_b = (unsigned)(p.vs.s * (int64_t)sizeof(T));
   const int64_t rows_all = (int64_t)p.P * p.Sk;
@@ -204,32 +209,28 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       (void*)kp, 0, (int)(unsigned)(((rows_all - 1) * p.ks.s + D) * (int64_t)sizeof(T)), 0x00020000);
   const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
       (void*)vp, 0, (int)(unsigned)(((rows_all - 1) * p.vs.s + D) * (int64_t)sizeof(T)), 0x00020000);
-
+  // load number q of a sub-tile whose first row is krow: passes of K first, then V's four rows
+  constexpr int NLOADS = C::KPASS + 4;
+  auto gload_one = [&](int q, bool kon, int k_row, bool von, int v_row, u32x4 (&kreg)[C::KPASS], u32x4 (&vreg)[4]) {
+    if (q < C::KPASS) {
+      const unsigned u = kon ? (unsigned)(k_row + q * C::RPP) * krow_b : OFF_NONE;
+      kreg[q] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, kvoff + u, 0, 0);
+    } else {
+      const unsigned u = von ? (unsigned)(v_row + q - C::KPASS) * vrow_b : OFF_NONE;
+      vreg[q - C::KPASS] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, vvoff + u, 0, 0);
+    }
+  };
   auto gload_k = [&](int i, u32x4 (&kreg)[C::KPASS]) {
-    if (i >= n) return;
-    const Sub sb = locate(i);
+    u32x4 dummy[4];
+    const Sub sb = locate(i < n ? i : 0);
 #pragma unroll
-    for (int j = 0; j < C::KPASS; ++j)
-      kreg[j] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, kvoff, (sb.krow + j * C::RPP) * krow_b, 0);
+    for (int q = 0; q < C::KPASS; ++q) gload_one(q, i < n, sb.krow, false, 0, kreg, dummy);
   };
   auto gload_v = [&](int i, u32x4 (&vreg)[4]) {
-    if (i >= n || !vact) return;
-    const Sub sb = locate(i);
+    u32x4 dummy[C::KPASS];
+    const Sub sb = locate(i < n ? i : 0);
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      vreg[j] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, vvoff, (sb.krow + j) * vrow_b, 0);
-  };
-  auto gload_k_at = [&](const Cursor& c, u32x4 (&kreg)[C::KPASS]) {
-    if (c.i >= n) return;
-#pragma unroll
-    for (int j = 0; j < C::KPASS; ++j)
-      kreg[j] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, kvoff, (c.sb.krow + j * C::RPP) * krow_b, 0);
-  };
-  auto gload_v_at = [&](const Cursor& c, u32x4 (&vreg)[4]) {
-    if (c.i >= n || !vact) return;
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      vreg[j] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, vvoff, (c.sb.krow + j) * vrow_b, 0);
+    for (int q = 0; q < 4; ++q) gload_one(C::KPASS + q, false, 0, i < n, sb.krow, dummy, vreg);
   };
   auto lstore_k = [&](int i, const u32x4 (&kreg)[C::KPASS]) {
     if (i >= n) return;
@@ -267,7 +268,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // MFMA phase of step i: O += V(i)^T P(i) (if PV) followed by S(i+1) = K(i+1) Q^T (if NS).
   // The LDS operand of MFMA number j is fetched LOOK MFMAs ahead of its use, so the whole
   // phase runs off a rolling window of LOOK fragments instead of stalling on every read.
-  auto mfma_phase = [&](auto do_pv, auto do_s, int i, frag (&pfr)[2][2]) {
+  auto mfma_phase = [&](auto do_pv, auto do_s, int i, frag (&pfr)[2][2], auto&& side) {
     constexpr bool PV = decltype(do_pv)::value, NS = decltype(do_s)::value;
     constexpr int NPV = PV ? (D / 32) * 4 : 0;
     constexpr int NSS = NS ? (D / 16) * 2 : 0;
@@ -309,6 +310,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
           s[t] = M::run(a, qf[ks], s[t]);
         }
       }
+      side(j);
     }
   };
 
@@ -402,7 +404,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   __syncthreads();
   {
     frag none[2][2];
-    mfma_phase(std::false_type{}, std::true_type{}, -1, none);  // S(0), operands prefetched through the window
+    mfma_phase(std::false_type{}, std::true_type{}, -1, none, [](int) {});  // S(0), operands prefetched through the window
   }
   __syncthreads();
   if (NG > 1 && grp == 1) __syncthreads();  // group 1 runs one phase behind group 0
@@ -417,10 +419,16 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     lstore_k(i + 2, kreg);  // into the buffer S(i) was read from
     lstore_v(i + 1, vreg);  // into the buffer P(i-1) V(i-1) was read from
     __syncthreads();
-    gload_k_at(ck, kreg);  // K(i+3), V(i+2): in flight across this MFMA phase and the next softmax
-    gload_v_at(cv, vreg);
+    // K(i+3), V(i+2): one load every few MFMAs, in flight across the rest of this phase and the
+    // next softmax
+    const bool kon = ck.i < n, von = cv.i < n;
     __builtin_amdgcn_s_setprio(1);
-    mfma_phase(std::true_type{}, std::true_type{}, i, pf);
+    mfma_phase(std::true_type{}, std::true_type{}, i, pf, [&](int j) {
+      constexpr int TOTAL = (D / 32) * 4 + (D / 16) * 2;
+#pragma unroll
+      for (int q = 0; q < NLOADS; ++q)
+        if ((q * TOTAL + TOTAL / 2) / NLOADS == j) gload_one(q, kon, ck.sb.krow, von, cv.sb.krow, kreg, vreg);
+    });
     __builtin_amdgcn_s_setprio(0);
     cursor_next(cs);
     cursor_next(cv);
@@ -431,7 +439,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     frag pf[2][2];
     softmax_phase(cs.sb, pf);
     __syncthreads();
-    mfma_phase(std::true_type{}, std::false_type{}, n - 1, pf);
+    mfma_phase(std::true_type{}, std::false_type{}, n - 1, pf, [](int) {});
     __syncthreads();
   }
   if (NG > 1 && grp == 0) __syncthreads();  // matches group 1's leading barrier
