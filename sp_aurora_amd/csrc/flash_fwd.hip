@@ -41,18 +41,41 @@ constexpr int FWD_THREADS = 256;  // threads of one wave group (4 waves x 32 que
 
 template <int D, int NG>
 struct Fwd16Cfg {
-  static constexpr int KP = D * 2 + 16;       // K tile row pitch in bytes (+16: bank spread)
-  static constexpr int VP = FWD_BN * 2 + 16;  // V^T tile row pitch in bytes
-  static constexpr int KBYTES = FWD_BN * KP;
-  static constexpr int VBYTES = D * VP;
-  static constexpr int GROUP = 2 * KBYTES + 2 * VBYTES;  // one group's K[2] and V^T[2] buffers
+  static constexpr int ROWB = D * 2;           // bytes per K / V row in LDS: no padding, the tiles are swizzled
+  static constexpr int TILEB = FWD_BN * ROWB;  // one K or V sub-tile
+  static constexpr int GROUP = 4 * TILEB;      // one group's K[2] and V[2] buffers
   static constexpr int EPI = (NG * FWD_BM * (D + 4) + NG * FWD_BM * 2 + FWD_BM) * 4;  // epilogue staging
   static constexpr int SMEM = NG * GROUP > EPI ? NG * GROUP : EPI;
-  static constexpr int CPR = D / 8;              // 16-byte chunks per row
-  static constexpr int RPP = FWD_THREADS / CPR;  // K rows fetched per pass
-  static constexpr int KPASS = FWD_BN / RPP;     // passes per K sub-tile
-  static constexpr int VUNITS = 16 * CPR;        // (4 keys x 8 dims) units per V sub-tile
+  static constexpr int CPR = D / 8;                         // 16-byte chunks per row
+  static constexpr int NDMA = TILEB / (FWD_THREADS * 16);   // direct loads per thread and sub-tile
+  static constexpr int RPD = FWD_THREADS / CPR;             // rows one round of the group's loads covers
 };
+
+// A sub-tile lives in LDS as its rows back to back, each row's 16-byte chunks permuted by an XOR
+// with a function of the row, so that the reads of one instruction spread over all banks:
+// K is read 16 bytes per lane by 16 consecutive rows at one chunk index; V is read by the
+// transposing 8-byte read, a half wave covering 4 rows x 64 bytes.
+template <int D>
+__device__ __forceinline__ int k_swizzle(int row) {
+  constexpr int CPR = D / 8;
+  return (row / (16 / CPR)) % CPR;
+}
+template <int D>
+__device__ __forceinline__ int v_swizzle(int row) {
+  return D == 128 ? (row & 3) << 2 : D == 64 ? ((row >> 1) & 1) << 2 : 0;
+}
+
+typedef __attribute__((address_space(3))) unsigned char lds_u8;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+// 16 bytes per lane from a buffer straight into LDS at lds_addr + 16 * lane (lds_addr wave-uniform);
+// out-of-range lanes store zeros.  Counts on vmcnt like any load.
+__device__ __forceinline__ void load_to_lds_b128(u32x4 rsrc, unsigned voffset, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :
+               : "s"(lds_addr), "v"(voffset), "s"(rsrc)
+               : "memory");
+}
 
 template <typename T, int D, int NG>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams p) {
@@ -178,82 +201,81 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     c.sb.krow = ch * p.Sk + c.sb.krel;
     c.sb.kend = ch * p.Sk + p.Sk;
   };
-  unsigned char* gbase = smem + grp * C::GROUP;
-  auto kbuf = [&](int i) { return gbase + (i & 1) * C::KBYTES; };
-  auto vbuf = [&](int i) { return gbase + 2 * C::KBYTES + (i & 1) * C::VBYTES; };
-
-  // ---- global -> register -> LDS staging of one K / V sub-tile by the group's 256 threads ----
-  const int kc = tg % C::CPR;
-  const int kr = tg / C::CPR;
-  const int vkg = tg & 15;  // group of 4 consecutive keys
-  const int vdc = tg >> 4;  // chunk of 8 head dims
-  const bool vact = tg < C::VUNITS;
-  // position of this key group inside the permuted 64-key row of V^T
-  const int vpos = (vkg >> 3) * 32 + ((vkg >> 2) & 1) * 16 + (vkg & 1) * 8 + ((vkg >> 1) & 1) * 4;
-  // K/V sub-tiles are fetched with buffer loads: a wave-uniform descriptor per tensor and a 32-bit
-  // byte offset per lane (a lane constant plus the sub-tile's uniform row offset: one add per load),
-  // and the hardware's range check instead of clamps and branches: a row past the end of the tensor
-  // reads as zero, a row past the end of its chunk but inside the tensor reads the next chunk's
-  // data; both are keys >= Sk, which the softmax masks to P = 0.  The range check covers the
-  // per-lane offset only, so the whole offset travels there and the scalar offset stays 0; a load
-  // that must not happen (past the end of the schedule, a lane without a share of V) gets an
-  // offset beyond any tensor and returns zeros (both at once wrap to offset 0: the tensor's first
-  // bytes, valid memory, never used).
+  // ---- global -> LDS: direct loads, no registers in between ----
+  // Thread tg of the group owns slot tg of every round of 256 16-byte slots; round j of a
+  // sub-tile covers rows j * RPD + tg / CPR.  LDS slot (row, pos) receives the row's chunk
+  // pos ^ swizzle(row), so the permutation happens on the global side, in the lane's offset.
+  // Buffer loads: a wave-uniform descriptor per tensor and a 32-bit byte offset per lane (a lane
+  // constant plus the sub-tile's uniform row offset), and the hardware's range check instead of
+  // clamps and branches: a row past the end of the tensor arrives as zeros, a row past the end of
+  // its chunk but inside the tensor is the next chunk's data; both are keys >= Sk, which the
+  // softmax masks to P = 0.  The range check covers the per-lane offset only, so the whole offset
+  // travels there.  A load that is not wanted (past the end of the schedule) gets an offset beyond
+  // any tensor and stores zeros into a buffer nobody reads.
   constexpr unsigned OFF_NONE = 0x80000000u;
-  const unsigned kvoff = (unsigned)((kr * p.ks.s + kc * 8) * (int64_t)sizeof(T));
-  const unsigned vvoff = vact ? (unsigned)((vkg * 4 * p.vs.s + vdc * 8) * (int64_t)sizeof(T)) : OFF_NONE;
+  const int drow = tg / C::CPR, dpos = tg % C::CPR;
+  const unsigned kdoff = (unsigned)((drow * p.ks.s + ((dpos ^ k_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(T));
+  const unsigned vdoff = (unsigned)((drow * p.vs.s + ((dpos ^ v_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(T));
   const unsigned krow_b = (unsigned)(p.ks.s * (int64_t)sizeof(T));  // bytes per K row
   const unsigned vrow_b = (unsigned)(p.vs.s * (int64_t)sizeof(T));
   const int64_t rows_all = (int64_t)p.P * p.Sk;
-  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)kp, 0, (int)(unsigned)(((rows_all - 1) * p.ks.s + D) * (int64_t)sizeof(T)), 0x00020000);
-  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)vp, 0, (int)(unsigned)(((rows_all - 1) * p.vs.s + D) * (int64_t)sizeof(T)), 0x00020000);
-  // load number q of a sub-tile whose first row is krow: passes of K first, then V's four rows
-  constexpr int NLOADS = C::KPASS + 4;
-  auto gload_one = [&](int q, bool kon, int k_row, bool von, int v_row, u32x4 (&kreg)[C::KPASS], u32x4 (&vreg)[4]) {
-    if (q < C::KPASS) {
-      const unsigned u = kon ? (unsigned)(k_row + q * C::RPP) * krow_b : OFF_NONE;
-      kreg[q] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, kvoff + u, 0, 0);
+  auto descriptor = [&](const T* base, int64_t row_stride) {
+    const uint64_t a = (uint64_t)base;
+    u32x4 r;
+    r[0] = __builtin_amdgcn_readfirstlane((unsigned)a);
+    r[1] = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32) & 0xffffu);  // stride 0: raw buffer
+    r[2] = __builtin_amdgcn_readfirstlane((unsigned)(((rows_all - 1) * row_stride + D) * (int64_t)sizeof(T)));
+    r[3] = 0x00020000u;
+    return r;
+  };
+  const u32x4 krsrc = descriptor(kp, p.ks.s);
+  const u32x4 vrsrc = descriptor(vp, p.vs.s);
+  // LDS byte addresses of this group's buffers and of this wave's 1 KB share of a round
+  const unsigned lds_group = (unsigned)(uintptr_t)(lds_u8*)smem + grp * C::GROUP;
+  const unsigned lds_wave = lds_group + w * 1024;
+  auto k_lds = [&](int i) { return (unsigned)((i & 1) * C::TILEB); };                  // relative to lds_group
+  auto v_lds = [&](int i) { return (unsigned)(2 * C::TILEB + (i & 1) * C::TILEB); };
+  // load number q of the pair (K sub-tile with first row k_row into buffer kb, V sub-tile v_row into vb)
+  constexpr int NLOADS = 2 * C::NDMA;
+  auto load_one = [&](int q, bool kon, int k_row, unsigned kb, bool von, int v_row, unsigned vb) {
+    if (q < C::NDMA) {
+      const unsigned u = kon ? (unsigned)(k_row + q * C::RPD) * krow_b : OFF_NONE;
+      load_to_lds_b128(krsrc, kdoff + u, lds_wave + kb + q * (FWD_THREADS * 16));
     } else {
-      const unsigned u = von ? (unsigned)(v_row + q - C::KPASS) * vrow_b : OFF_NONE;
-      vreg[q - C::KPASS] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, vvoff + u, 0, 0);
+      const int r = q - C::NDMA;
+      const unsigned u = von ? (unsigned)(v_row + r * C::RPD) * vrow_b : OFF_NONE;
+      load_to_lds_b128(vrsrc, vdoff + u, lds_wave + vb + r * (FWD_THREADS * 16));
     }
   };
-  auto gload_k = [&](int i, u32x4 (&kreg)[C::KPASS]) {
-    u32x4 dummy[4];
+  auto load_k = [&](int i) {
     const Sub sb = locate(i < n ? i : 0);
 #pragma unroll
-    for (int q = 0; q < C::KPASS; ++q) gload_one(q, i < n, sb.krow, false, 0, kreg, dummy);
+    for (int q = 0; q < C::NDMA; ++q) load_one(q, i < n, sb.krow, k_lds(i), false, 0, 0);
   };
-  auto gload_v = [&](int i, u32x4 (&vreg)[4]) {
-    u32x4 dummy[C::KPASS];
+  auto load_v = [&](int i) {
     const Sub sb = locate(i < n ? i : 0);
 #pragma unroll
-    for (int q = 0; q < 4; ++q) gload_one(C::KPASS + q, false, 0, i < n, sb.krow, dummy, vreg);
+    for (int q = 0; q < C::NDMA; ++q) load_one(C::NDMA + q, false, 0, 0, i < n, sb.krow, v_lds(i));
   };
-  auto lstore_k = [&](int i, const u32x4 (&kreg)[C::KPASS]) {
-    if (i >= n) return;
-    unsigned char* kb = kbuf(i);
+  auto loads_landed = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };  // vmcnt(0)
+
+  // ---- LDS -> MFMA operands ----
+  // K (A operand of S^T = K Q^T): lane (key = ln, half hh) reads chunk 2 ks + hh of its row.
+  // V (A operand of O^T += V^T P^T): the transposing read hands lane (dim, hh) four consecutive
+  // keys of one head dim; in a block of 16 lanes, lane 4 e + c supplies the address of 8 bytes
+  // (4 dims) of key e, and lane x receives dim x of keys 0..3.
+  unsigned kra[D / 16], vra[D / 32];
 #pragma unroll
-    for (int j = 0; j < C::KPASS; ++j) *(u32x4*)(kb + (kr + j * C::RPP) * C::KP + kc * 16) = kreg[j];
-  };
-  auto lstore_v = [&](int i, const u32x4 (&vreg)[4]) {
-    if (i >= n || !vact) return;
-    unsigned char* vb = vbuf(i);
-    // 4 keys x 8 dims in registers -> 8 rows (dims) of 4 consecutive keys
+  for (int ks = 0; ks < D / 16; ++ks) kra[ks] = lds_group + ln * C::ROWB + (((2 * ks + hh) ^ k_swizzle<D>(ln)) * 16);
+  {
+    const int blk = lane >> 4, e = (lane >> 2) & 3, c4 = lane & 3;
+    const int krl = 4 * hh + e;
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      const unsigned a0 = vreg[0][m], a1 = vreg[1][m], a2 = vreg[2][m], a3 = vreg[3][m];
-      u32x2 even, odd;
-      even[0] = __builtin_amdgcn_perm(a1, a0, 0x05040100u);  // lo16(a0) | lo16(a1) << 16
-      even[1] = __builtin_amdgcn_perm(a3, a2, 0x05040100u);
-      odd[0] = __builtin_amdgcn_perm(a1, a0, 0x07060302u);   // hi16(a0) | hi16(a1) << 16
-      odd[1] = __builtin_amdgcn_perm(a3, a2, 0x07060302u);
-      *(u32x2*)(vb + (vdc * 8 + 2 * m) * C::VP + vpos * 2) = even;
-      *(u32x2*)(vb + (vdc * 8 + 2 * m + 1) * C::VP + vpos * 2) = odd;
+    for (int db = 0; db < D / 32; ++db) {
+      const int chunk = db * 4 + (blk & 1) * 2 + (c4 >> 1);
+      vra[db] = lds_group + krl * C::ROWB + ((chunk ^ v_swizzle<D>(krl)) * 16) + (c4 & 1) * 8;
     }
-  };
+  }
 
   f32x16 s[2];
   f32x16 o[D / 32];
@@ -274,16 +296,29 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     constexpr int NSS = NS ? (D / 16) * 2 : 0;
     constexpr int TOTAL = NPV + NSS;
     constexpr int LOOK = 8;
-    const unsigned char* vb = vbuf(i) + ln * C::VP + hh * 16;
-    const unsigned char* kb = kbuf(i + 1) + ln * C::KP + hh * 16;
+    const unsigned vb = v_lds(i), kb = k_lds(i + 1);
+    unsigned va[D / 32], ka[D / 16];
+#pragma unroll
+    for (int db = 0; db < (PV ? D / 32 : 0); ++db) va[db] = vra[db] + vb;
+#pragma unroll
+    for (int ks = 0; ks < (NS ? D / 16 : 0); ++ks) ka[ks] = kra[ks] + kb;
     auto fetch = [&](int j) -> frag {
       if (j < NPV) {  // j = (t*2+u)*(D/32) + db : consecutive MFMAs hit different accumulators
         const int db = j % (D / 32), tu = j / (D / 32);
-        return as_frag<frag>(*(const u32x4*)(vb + db * 32 * C::VP + tu * 32));
+        const lds_u8* a = (const lds_u8*)(uintptr_t)va[db] + tu * 16 * C::ROWB;
+        const u32x2 r0 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)a));
+        const u32x2 r1 = __builtin_bit_cast(
+            u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(a + 8 * C::ROWB)));
+        u32x4 x;
+        x[0] = r0[0];
+        x[1] = r0[1];
+        x[2] = r1[0];
+        x[3] = r1[1];
+        return as_frag<frag>(x);
       }
       const int jj = j - NPV;  // jj = ks*2 + t
       const int t = jj & 1, ks = jj >> 1;
-      return as_frag<frag>(*(const u32x4*)(kb + t * 32 * C::KP + ks * 32));
+      return as_frag<frag>(*(const __attribute__((address_space(3))) u32x4*)((const lds_u8*)(uintptr_t)ka[ks] + t * 32 * C::ROWB));
     };
     frag win[LOOK];
 #pragma unroll
@@ -387,24 +422,15 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       }
   };
 
-  // ---- prologue: one round trip for Q, K(0), V(0), K(1); then K(2) / V(1) on their way ----
-  u32x4 kreg[C::KPASS];
-  u32x4 vreg[4];
-  {
-    u32x4 k1[C::KPASS];
-    gload_k(0, kreg);
-    gload_v(0, vreg);
-    gload_k(1, k1);
-    lstore_k(0, kreg);
-    lstore_v(0, vreg);
-    lstore_k(1, k1);
-  }
-  gload_k(2, kreg);
-  gload_v(1, vreg);
+  // ---- prologue: K(0), V(0), K(1) on their way into LDS together with Q into registers ----
+  load_k(0);
+  load_v(0);
+  load_k(1);
+  loads_landed();
   __syncthreads();
   {
     frag none[2][2];
-    mfma_phase(std::false_type{}, std::true_type{}, -1, none, [](int) {});  // S(0), operands prefetched through the window
+    mfma_phase(std::false_type{}, std::true_type{}, -1, none, [](int) {});  // S(0)
   }
   __syncthreads();
   if (NG > 1 && grp == 1) __syncthreads();  // group 1 runs one phase behind group 0
@@ -412,22 +438,22 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // One loop, no branch around an MFMA, the same two barriers per step for every wave.  A wave
   // whose rows see none of a diagonal sub-tile's keys (at most the last two sub-tiles of the
   // diagonal chunk) simply gets P = 0 from the mask.
-  Cursor cs = cursor_at(0), cv = cursor_at(2), ck = cursor_at(3);
+  // MFMA phase i reads V(i) and K(i+1); the other two buffers are free then and receive V(i+1)
+  // and K(i+2), which must have landed when the next VALU phase ends.
+  Cursor cs = cursor_at(0), cv = cursor_at(1), ck = cursor_at(2);
   for (int i = 0; i + 1 < n; ++i) {
     frag pf[2][2];
     softmax_phase(cs.sb, pf);
-    lstore_k(i + 2, kreg);  // into the buffer S(i) was read from
-    lstore_v(i + 1, vreg);  // into the buffer P(i-1) V(i-1) was read from
+    loads_landed();
     __syncthreads();
-    // K(i+3), V(i+2): one load every few MFMAs, in flight across the rest of this phase and the
-    // next softmax
     const bool kon = ck.i < n, von = cv.i < n;
+    const unsigned kb = k_lds(i), vb = v_lds(i + 1);
     __builtin_amdgcn_s_setprio(1);
     mfma_phase(std::true_type{}, std::true_type{}, i, pf, [&](int j) {
       constexpr int TOTAL = (D / 32) * 4 + (D / 16) * 2;
 #pragma unroll
       for (int q = 0; q < NLOADS; ++q)
-        if ((q * TOTAL + TOTAL / 2) / NLOADS == j) gload_one(q, kon, ck.sb.krow, von, cv.sb.krow, kreg, vreg);
+        if ((q * TOTAL + TOTAL / 2) / NLOADS == j) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb);
     });
     __builtin_amdgcn_s_setprio(0);
     cursor_next(cs);
@@ -438,6 +464,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   {  // last sub-tile: nothing to prepare behind it
     frag pf[2][2];
     softmax_phase(cs.sb, pf);
+    loads_landed();
     __syncthreads();
     mfma_phase(std::true_type{}, std::false_type{}, n - 1, pf, [](int) {});
     __syncthreads();
