@@ -3,18 +3,37 @@
 
 Workload = BASELINE config 3: bf16, B=1, S=8192 in P=8 chunks of 1024, H=32, D=128, causal;
 every rank's Q chunk against its prefix of KV chunks in ring order (8 diagonal + 28 full block
-pairs), merged per step, cast at the end.  One "step" is that whole 36-pair sweep; inputs are
-resident in HBM before the timed region.  value = causal-adjusted TFLOP/s of the whole sweep
-(549.76 GFLOP / step time), merges and casts included.
+pairs), partial results merged per step, cast at the end.  One "step" is that whole 36-pair
+sweep; inputs are resident in HBM before the timed region.  value = causal-adjusted TFLOP/s of
+the whole sweep (549.76 GFLOP / step time).
 
-Prints ONE JSON line (see the keys below).  `roofline` is for the dominant kernel, the block
-attention forward: algorithmic FLOPs per launch / average launch duration, the latter measured
-here with events on the launch stream over the timed sweep (its 36 launches are all this kernel).
-`cpu_baseline` times the oracle's restatement of the reference's op sequence (SDPA for out + a
-second q k^T / logsumexp for lse, sp_aurora/intel_flash_attn_optimized.py:156-193) on the host
-cores, on one diagonal + one full block pair of the same workload.
+The sweep is run through the C entry point spa_ring_fwd in its three schedules, all producing
+the same (out, lse):
+  all   one launch for the whole sweep: a workgroup keeps its query tile and accumulators in
+        registers and walks its rank's KV chunks in ring order (the step merge is the online
+        softmax).  This is `value`.
+  rank  one launch per rank (what one GPU of a real ring would run when its KV is resident).
+  step  one launch per (rank, ring step), running accumulators in HBM, the merge in the
+        kernel's epilogue (what a rank runs when each chunk arrives over the wire).
+The other two are reported beside it.
+
+Prints ONE JSON line.  `roofline` is for the dominant kernel, the block attention forward:
+algorithmic FLOPs per launch / average launch duration, the latter measured here with events on
+the launch stream over the timed region (in the `all` schedule the sweep is one launch of that
+kernel).  `cpu_baseline` times the oracle's restatement of the reference's op sequence (SDPA for
+out + a second q k^T / logsumexp for lse, sp_aurora/intel_flash_attn_optimized.py:156-193) on
+the host cores, on diagonal + full block pairs of the same workload.
+
+Two helper modes for the HBM traffic figure (roofline.traffic):
+  --traffic-leg          additionally runs a plain device copy of known size, so that a
+                         `rocprofv3 --pmc FETCH_SIZE` (or WRITE_SIZE) run of this script holds
+                         both the attention kernel and a calibration kernel
+  --pmc-summary F W      reads the two counter_collection.csv files of such runs and writes
+                         profiles/flash_fwd_traffic.json (no GPU needed)
 """
 import argparse
+import csv
+import glob
 import json
 import os
 import sys
@@ -29,6 +48,8 @@ HBM_PEAK_GBPS = 8000.0
 B, S, H, D, P = 1, 8192, 32, 128, 8
 SEED = 2
 INPUT_SCALE = 0.5
+COPY_BYTES = 1 << 30  # calibration copy of the traffic leg: reads and writes this many bytes
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "flash_fwd_traffic.json")
 
 
 def sweep_flops():
@@ -36,6 +57,14 @@ def sweep_flops():
     full = 4.0 * B * H * s * s * D
     n_diag, n_full = P, P * (P - 1) // 2
     return n_full * full + n_diag * full / 2, n_diag + n_full, full
+
+
+def algorithmic_bytes():
+    """Bytes the sweep must move: per block pair its K and V chunk in (36 pairs: on a real ring
+    they are 36 kernel inputs on 8 GPUs), per rank its Q chunk in, out and lse out."""
+    chunk = B * (S // P) * H * D * 2
+    n_pairs = P + P * (P - 1) // 2
+    return n_pairs * 2 * chunk + P * chunk + P * chunk + B * H * S * 4
 
 
 def make_inputs(torch, device):
@@ -96,22 +125,73 @@ def cpu_baseline(torch, budget_s=15.0):
     }
 
 
+def pmc_summary(fetch_dir, write_dir):
+    """FETCH_SIZE / WRITE_SIZE (KiB per dispatch) of the attention kernel, each scaled by what the
+    same counter reads for the calibration copy of COPY_BYTES."""
+    def read(d, counter):
+        files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
+        if not files:
+            raise SystemExit(f"no counter_collection.csv under {d}")
+        attn, copy = [], []
+        for f in files:
+            for row in csv.DictReader(open(f)):
+                if row.get("Counter_Name") != counter:
+                    continue
+                name, val = row["Kernel_Name"], float(row["Counter_Value"])
+                if "flash_fwd16_kernel" in name:
+                    attn.append(val)
+                elif "copy" in name.lower() or "elementwise" in name.lower():
+                    copy.append(val)
+        if not attn or not copy:
+            raise SystemExit(f"{counter}: attention or calibration kernel missing in {d}")
+        copy_kib = max(copy)  # the 1 GiB copy dwarfs any other elementwise kernel of the run
+        return sum(attn) / len(attn), copy_kib, len(attn)
+
+    f_attn, f_copy, n = read(fetch_dir, "FETCH_SIZE")
+    w_attn, w_copy, _ = read(write_dir, "WRITE_SIZE")
+    f_factor = (COPY_BYTES / 1024.0) / f_copy   # true KiB per counted KiB
+    w_factor = (COPY_BYTES / 1024.0) / w_copy
+    fetch_b = f_attn * f_factor * 1024.0
+    write_b = w_attn * w_factor * 1024.0
+    res = {
+        "kernel": "flash_fwd16_kernel<bf16,128,2>, config 3, schedule all (one launch per sweep)",
+        "dispatches_averaged": n,
+        "fetch_size_kib_per_dispatch": f_attn,
+        "write_size_kib_per_dispatch": w_attn,
+        "copy_fetch_size_kib": f_copy,
+        "copy_write_size_kib": w_copy,
+        "copy_bytes": COPY_BYTES,
+        "fetch_factor": f_factor,
+        "write_factor": w_factor,
+        "hbm_fetch_bytes_per_launch": fetch_b,
+        "hbm_write_bytes_per_launch": write_b,
+        "hbm_bytes_per_launch": fetch_b + write_b,
+        "algorithmic_bytes_per_launch": algorithmic_bytes(),
+    }
+    json.dump(res, open(TRAFFIC_JSON, "w"), indent=1)
+    print(json.dumps(res, indent=1))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50,
+                    help="the first ~50 launches after an idle period run slower while the GPU settles its clocks")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
-    ap.add_argument("--traffic-json", default=os.path.join(ROOT, "profiles", "flash_fwd_traffic.json"),
-                    help="HBM bytes per launch derived from rocprofv3 --pmc runs, if present")
+    ap.add_argument("--only-all", action="store_true", help="skip the rank / step schedules (profiling runs)")
+    ap.add_argument("--traffic-leg", action="store_true", help="also run the calibration copy (for --pmc runs)")
+    ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"))
     args = ap.parse_args()
+    if args.pmc_summary:
+        pmc_summary(*args.pmc_summary)
+        return
     if args.gpus != 1:
         print("bench.py: this build measures one GPU (the ring is simulated on it); --gpus must be 1", file=sys.stderr)
         sys.exit(2)
 
     import torch
     import sp_aurora_amd as spa
-    from sp_aurora_amd import ops
 
     if not torch.cuda.is_available():
         print("bench.py: no HIP device visible", file=sys.stderr)
@@ -122,43 +202,40 @@ def main():
     scale = D ** -0.5
     total_flops, n_pairs, full_flops = sweep_flops()
 
-    step = spa.ring.make_ring_forward_step(q, k, v, scale, True, P)  # preallocated buffers, no allocation per step
+    # preallocated buffers, no allocation per step
+    steps = {m: spa.ring.make_ring_forward_step(q, k, v, scale, True, P, fuse=m) for m in ("all", "rank", "step")}
 
+    step = steps["all"]
     for _ in range(args.warmup):
         step()
     ms = time_region(torch, step, args.steps)
     tflops = total_flops / (ms * 1e-3) / 1e12
 
-    # ---- dominant kernel: every launch of the timed sweep IS the block attention kernel (the
-    # merge rides in its epilogue), and the trace shows no gaps between them, so its average
-    # launch duration is the event-timed step divided by the number of launches.
-    k_ms = ms / n_pairs
-    flops_per_launch = total_flops / n_pairs
-    achieved = flops_per_launch / (k_ms * 1e-3) / 1e12
+    other = {}
+    if not args.only_all:
+        for m in ("rank", "step"):
+            for _ in range(max(3, args.warmup // 4)):
+                steps[m]()
+            t = time_region(torch, steps[m], max(5, args.steps // 4))
+            other[m] = {"ms_per_step": round(t, 4), "tflops": round(total_flops / (t * 1e-3) / 1e12, 2),
+                        "launches_per_step": P if m == "rank" else n_pairs}
 
-    # auxiliary: the same 36 block pairs as stand-alone block attention calls (plain epilogue,
-    # no merge), one Python call per launch
-    s = S // P
-    blk_out = torch.empty((B, s, H, D), dtype=torch.bfloat16, device=dev)
-    blk_lse = torch.empty((B, H, s), dtype=torch.float32, device=dev)
-    qs, ks, vs = q.split(s, 1), k.split(s, 1), v.split(s, 1)
-
-    def attention_only():
-        for r in range(P):
-            for t in range(r + 1):
-                ops.flash_fwd(qs[r], ks[r - t], vs[r - t], scale, t == 0, layout="bshd", out=blk_out, lse=blk_lse)
-
-    for _ in range(3):
-        attention_only()
-    plain_us = time_region(torch, attention_only, max(5, args.steps // 2)) / n_pairs * 1e3
+    if args.traffic_leg:
+        src = torch.empty(COPY_BYTES, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
 
     traffic = None
-    if os.path.exists(args.traffic_json):
+    if os.path.exists(TRAFFIC_JSON):
         try:
-            traffic = json.load(open(args.traffic_json)).get("hbm_bytes_per_launch")
+            traffic = json.load(open(TRAFFIC_JSON)).get("hbm_bytes_per_launch")
         except (ValueError, OSError):
             traffic = None
 
+    # dominant kernel: in the `all` schedule the timed region is args.steps launches of the
+    # attention kernel and nothing else, so its average launch duration is ms
+    achieved = total_flops / (ms * 1e-3) / 1e12
     line = {
         "metric": "fwd attn TFLOP/s + % bf16 MFMA peak, ring-step causal S=8K H32 D128",
         "value": round(tflops, 2),
@@ -174,23 +251,25 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "config 3: simulated ring P=8 on one GPU, bf16 B=1 S=8192 (8 chunks of 1024) H=32 D=128 causal, "
-                        "8 diagonal + 28 full block pairs, merge per step, seed 2 N(0,1)*0.5",
+                        "8 diagonal + 28 full block pairs in ring order, step merge, seed 2 N(0,1)*0.5; "
+                        "schedule 'all' (one launch walks every rank's ring)",
             "flops_per_step": total_flops,
             "block_pairs": n_pairs,
         },
         "pct_of_bf16_mfma_peak": round(100.0 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
+        "other_schedules": other,
         "roofline": {
             "bound": "mfma",
-            "kernel": "flash_fwd16_kernel<bf16,128>",
+            "kernel": "flash_fwd16_kernel<bf16,128,2>",
             "achieved": round(achieved, 2),
             "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
             "traffic": traffic,
-            "avg_launch_us": round(k_ms * 1e3, 2),
-            "flops_per_launch": flops_per_launch,
-            "launches_per_step": n_pairs,
-            "plain_block_call_us": round(plain_us, 2),
+            "avg_launch_us": round(ms * 1e3, 2),
+            "flops_per_launch": total_flops,
+            "launches_per_step": 1,
+            "algorithmic_bytes_per_launch": algorithmic_bytes(),
         },
     }
     if not args.no_cpu_baseline:
