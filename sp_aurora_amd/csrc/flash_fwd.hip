@@ -1,11 +1,13 @@
 // Block flash-attention forward for gfx950: out = softmax(q k^T * scale + mask) v and
-// fp32 lse = logsumexp(q k^T * scale + mask), one launch per (q chunk, kv chunk) pair.
+// fp32 lse = logsumexp(q k^T * scale + mask), for one (q chunk, kv chunk) pair or for a whole
+// ring schedule of kv chunks per launch.
 // Stands in for intel_flash_attn_forward (sp_aurora/intel_flash_attn.py:18-126) /
-// intel_flash_attn_forward_optimized (sp_aurora/intel_flash_attn_optimized.py:95-225):
+// intel_flash_attn_forward_optimized (sp_aurora/intel_flash_attn_optimized.py:95-225) and, with
+// the schedule, for the step loop around it (sp_aurora/intel_ring_flash_attn.py:72-148):
 // one Q.K^T instead of the reference's two, scores never leave the CU.
 //
 // Work decomposition (16-bit kernel)
-//   workgroup = 128 query rows of one (batch, head); a wave owns 32 of them.
+//   workgroup = 128 query rows of one (batch, head, rank); a wave owns 32 of them.
 //   Both contractions are computed TRANSPOSED on v_mfma_f32_32x32x16:
 //     S^T[key][qrow] = K[key][:] . Q[qrow][:]      A = K tile (LDS), B = Q (registers)
 //     O^T[d][qrow]  += V^T[d][key] . P^T[key][qrow] A = V^T tile (LDS), B = P^T (registers)
@@ -14,16 +16,17 @@
 //   per-lane reduction plus one exchange with lane^32, the rescale of O is a
 //   per-lane scalar, and the S^T accumulators are, register for register,
 //   the B operand of the second contraction: P never touches LDS.
-//   The contraction index of an MFMA may be permuted freely as long as A and
-//   B agree; V^T is stored in LDS with keys permuted (bits 2 and 3 of the key
-//   index within a 32-key block swapped) so that the 8 keys a lane needs for
-//   one P^T operand are one 16-byte LDS read.
+//
+//   K and V sub-tiles (64 keys) travel from global memory straight into LDS (buffer loads
+//   with the LDS bit), rows back to back with their 16-byte chunks XOR-permuted against bank
+//   conflicts.  K operands are 16-byte LDS reads; V stays row-major in LDS and is transposed
+//   by the read (ds_read_b64_tr_b16), two reads per operand.
 //
 //   Two wave groups (8 waves, two per SIMD) share the query rows and take alternate
 //   64-key sub-tiles; each group streams its own sub-tiles through its own
 //   double-buffered LDS.  A wave's loop is software-pipelined into two phases,
-//       VALU phase:  softmax of S(i) -> P(i);  stage K(i+2), V(i+1) into LDS
-//       MFMA phase:  issue the next global loads;  O += V(i)^T P(i);  S(i+1) = K(i+1) Q^T
+//       VALU phase:  softmax of S(i) -> P(i);  wait for the loads issued one phase ago
+//       MFMA phase:  O += V(i)^T P(i);  S(i+1) = K(i+1) Q^T;  loads of V(i+1), K(i+2) in between
 //   separated by workgroup barriers, and group 1 runs one barrier behind group 0, so at
 //   any time one wave of a SIMD is in its MFMA phase while its neighbour is in its VALU
 //   phase (ping-pong).  The groups' partial (O, m, l) are combined through LDS at the end.
