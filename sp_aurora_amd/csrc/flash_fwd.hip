@@ -41,6 +41,7 @@ namespace {
 constexpr int FWD_BM = 128;  // query rows per workgroup
 constexpr int FWD_BN = 64;   // keys per LDS sub-tile
 constexpr int FWD_THREADS = 256;  // threads of one wave group (4 waves x 32 query rows)
+constexpr int FWD_LOOK = 8;       // MFMA operands are fetched from LDS this many MFMAs ahead
 
 template <int D, int NG>
 struct Fwd16Cfg {
@@ -298,7 +299,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     constexpr int NPV = PV ? (D / 32) * 4 : 0;
     constexpr int NSS = NS ? (D / 16) * 2 : 0;
     constexpr int TOTAL = NPV + NSS;
-    constexpr int LOOK = 8;
+    constexpr int LOOK = FWD_LOOK;
     const unsigned vb = v_lds(i), kb = k_lds(i + 1);
     unsigned va[D / 32], ka[D / 16];
 #pragma unroll
