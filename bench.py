@@ -24,6 +24,11 @@ kernel).  `cpu_baseline` times the oracle's restatement of the reference's op se
 out + a second q k^T / logsumexp for lse, sp_aurora/intel_flash_attn_optimized.py:156-193) on
 the host cores, on diagonal + full block pairs of the same workload.
 
+`--workload` selects the other measured rows of the path instead (one JSON line each, same keys,
+`metric` named after the row): `relayout` = the Ulysses re-layout of BASELINE config 4 (HBM
+bound), `merge` = update_out_and_lse on one config-3 chunk (HBM bound), `backward` = the ring
+backward of BASELINE config 5 (MFMA bound).
+
 Two helper modes for the HBM traffic figure (roofline.traffic):
   --traffic-leg          additionally runs a plain device copy of known size, so that a
                          `rocprofv3 --pmc FETCH_SIZE` (or WRITE_SIZE) run of this script holds
@@ -172,6 +177,64 @@ def pmc_summary(fetch_dir, write_dir):
     print(json.dumps(res, indent=1))
 
 
+def side_workload(torch, name, steps, warmup):
+    """The other rows of the path: one JSON line with the same keys, roofline against its own bound."""
+    import sp_aurora_amd as spa
+    from sp_aurora_amd import ops
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(3)
+    rnd = lambda shape, dt=torch.bfloat16: torch.randn(shape, generator=g, dtype=torch.float32).to(dt).to(dev)
+    if name == "relayout":
+        Pn, Bn, sn, Hn, Dn = 8, 1, 2048, 32, 128
+        x = rnd((Pn, Bn, sn, Hn, Dn))
+        y = torch.empty((Pn, Bn, Pn * sn, Hn // Pn, Dn), dtype=x.dtype, device=dev)
+        back = torch.empty_like(x)
+        fn = lambda: (ops.relayout_s2h(x, Pn, out=y), ops.relayout_h2s(y, Pn, out=back))
+        units, unit_bytes = 2, 2 * x.numel() * 2   # two launches per step, each reads and writes the tensor once
+        bound, kernel, metric = "hbm", "relayout_kernel<16>", "Ulysses re-layout GB/s, config 4 [8,1,2048,32,128] bf16, s2h + h2s"
+        work = {"workload": "config 4 re-layout: [P=8,B=1,s=2048,H=32,D=128] bf16 -> [8,1,16384,4,128] and back", "bytes_per_launch": unit_bytes}
+    elif name == "merge":
+        Bn, sn, Hn, Dn = 1, 1024, 32, 128
+        acc = torch.randn((Bn, sn, Hn, Dn), generator=g, dtype=torch.float32).to(dev)
+        lse = torch.randn((Bn, Hn, sn), generator=g, dtype=torch.float32).to(dev)
+        blk = rnd((Bn, sn, Hn, Dn))
+        blk_lse = torch.randn((Bn, Hn, sn), generator=g, dtype=torch.float32).to(dev)
+        fn = lambda: ops.merge(acc, lse, blk, blk_lse, layout="bshd")
+        units, unit_bytes = 1, acc.numel() * 10 + lse.numel() * 12
+        bound, kernel, metric = "hbm", "merge_kernel<bf16>", "update_out_and_lse GB/s, one config-3 chunk [1,1024,32,128]"
+        work = {"workload": "merge of a bf16 block into the fp32 running (out, lse) of one config-3 rank", "bytes_per_launch": unit_bytes}
+    elif name == "backward":
+        Bn, Sn, Hn, Dn, Pn = 1, 32768, 16, 128, 16
+        qkv = rnd((Bn, Sn, 3, Hn, Dn))
+        dout = rnd((Bn, Sn, Hn, Dn))
+        q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+        scale = Dn ** -0.5
+        out, lse = spa.ring.ring_flash_attn_forward(q, k, v, scale, True, Pn, fuse="all")
+        fn = lambda: spa.ring.ring_flash_attn_backward(dout, q, k, v, out, lse, scale, True, Pn)
+        fwd_flops = 4.0 * Bn * Hn * Sn * Sn * Dn / 2
+        units, unit_flops = 1, 2.5 * fwd_flops   # five GEMMs of the algorithm (the two kernels recompute S and dP: 7 executed)
+        bound, kernel, metric = "mfma", "flash_bwd_dq_kernel + flash_bwd_dkdv_kernel", "ring backward TFLOP/s (5-GEMM count, causal-adjusted), config 5 S=32K H16 D128 P=16"
+        work = {"workload": "config 5 backward: bf16 qkv [1,32768,3,16,128] causal, ring of 16 chunks, dq/dk/dv by block-wise recompute", "flops_per_step": unit_flops}
+    else:
+        raise SystemExit(f"unknown workload {name}")
+    for _ in range(warmup):
+        fn()
+    ms = time_region(torch, fn, steps)
+    if bound == "hbm":
+        achieved = units * unit_bytes / (ms * 1e-3) / 1e9
+        peak, unit = HBM_PEAK_GBPS, "GB/s"
+    else:
+        achieved = unit_flops / (ms * 1e-3) / 1e12
+        peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+    print(json.dumps({
+        "metric": metric, "value": round(achieved, 2), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic", "config": work,
+        "roofline": {"bound": bound, "kernel": kernel, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+                     "frac": round(achieved / peak, 4), "traffic": None},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -182,6 +245,7 @@ def main():
     ap.add_argument("--only-all", action="store_true", help="skip the rank / step schedules (profiling runs)")
     ap.add_argument("--traffic-leg", action="store_true", help="also run the calibration copy (for --pmc runs)")
     ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"))
+    ap.add_argument("--workload", default="config3", choices=["config3", "relayout", "merge", "backward"])
     args = ap.parse_args()
     if args.pmc_summary:
         pmc_summary(*args.pmc_summary)
@@ -198,6 +262,10 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload != "config3":
+        side_workload(torch, args.workload, args.steps if args.workload != "backward" else min(args.steps, 5),
+                      args.warmup if args.workload != "backward" else min(args.warmup, 2))
+        return
     q, k, v = make_inputs(torch, dev)
     scale = D ** -0.5
     total_flops, n_pairs, full_flops = sweep_flops()

@@ -8,97 +8,107 @@
 //   dq kernel   : workgroup = 128 query rows (4 waves x 32), walks key tiles of 64.
 //                 S^T = K Q^T and dP^T = V dO^T land with a lane owning one query row,
 //                 so lse/delta are per-lane scalars and dS^T is, register for register,
-//                 the B operand of dQ^T = K^T dS^T (K^T staged transposed in LDS).
+//                 the B operand of dQ^T = K^T dS^T.
 //   dkdv kernel : workgroup = 128 keys (4 waves x 32), walks query tiles of 64.
 //                 S = Q K^T and dP = dO V^T land with a lane owning one key, so P and dS
-//                 are the B operands of dV^T = dO^T P and dK^T = Q^T dS (Q^T, dO^T staged
-//                 transposed in LDS).
-// The MFMA contraction index is permuted the same way on both operands (bits 2 and 3 of the
-// index inside a 32-block swapped) so that every operand is one 16-byte LDS read.
+//                 are the B operands of dV^T = dO^T P and dK^T = Q^T dS.
+//
+// Streamed tiles (K, V / Q, dO; 64 rows) travel from global memory straight into LDS, several
+// tiles ahead, rows back to back with their 16-byte chunks XOR-permuted so that both ways of
+// reading a tile run without bank conflicts: rows as 16-byte reads (A operands of the S / dP
+// contractions) and, through the transposing read, columns (A operands K^T, Q^T, dO^T of the
+// gradient contractions).  No transposed copies exist.
+//
+// One wave per SIMD, software-pipelined inside the wave at half-tile (32 rows) granularity:
+// the MFMAs that produce S and dP of half-tile g+1 are interleaved, one to one, with the
+// element-wise work (exp, dS) on half-tile g, followed by the gradient MFMAs of half-tile g.
+// MFMA operands come from LDS through a rolling window that runs ahead of the MFMAs and is
+// carried across loop iterations; one workgroup barrier per 64-row tile.
 // Accumulators are fp32 in HBM and are ADDED to (read-modify-write by the owning lane).
 #include "spa_common.h"
 
 namespace {
 
 constexpr int BWD_THREADS = 256;
-constexpr int BWD_ROWS = 64;  // rows (keys or queries) per streamed LDS tile
+constexpr int BWD_ROWS = 64;    // rows (keys or queries) per streamed LDS tile
+constexpr int BWD_STAGES = 4;   // tiles resident or on their way
+constexpr int BWD_LOOK_MAX = 8; // operands are fetched from LDS up to this many MFMAs ahead
+constexpr unsigned OFF_NONE = 0x80000000u;  // a buffer offset beyond any tensor: the load stores zeros
 
 template <int D>
-struct TileCfg {
-  static constexpr int KP = D * 2 + 16;          // row pitch of a row-major tile, bytes
-  static constexpr int VP = BWD_ROWS * 2 + 16;   // row pitch of a transposed tile, bytes
-  static constexpr int ROWB = BWD_ROWS * KP;     // bytes of a row-major tile
-  static constexpr int TRB = D * VP;             // bytes of a transposed tile
-  static constexpr int CPR = D / 8;
-  static constexpr int RPP = BWD_THREADS / CPR;
-  static constexpr int PASS = BWD_ROWS / RPP;
-  static constexpr int UNITS = 16 * CPR;
+struct BwdCfg {
+  static constexpr int ROWB = D * 2;             // bytes per tile row
+  static constexpr int TILEB = BWD_ROWS * ROWB;  // one tile
+  static constexpr int CPR = D / 8;              // 16-byte chunks per row
+  static constexpr int NDMA = TILEB / (BWD_THREADS * 16);  // direct loads per thread and tile
+  static constexpr int RPD = BWD_THREADS / CPR;  // rows one round of the workgroup's loads covers
 };
 
-// ---- streamed tile, row-major: 64 rows x D elements ----
-template <typename T, int D>
-__device__ __forceinline__ void rows_gload(u32x4 (&reg)[TileCfg<D>::PASS], const T* base, int64_t stride,
-                                           int row0, int nrows, int tid) {
-  typedef TileCfg<D> C;
-#pragma unroll
-  for (int i = 0; i < C::PASS; ++i) {
-    int r = row0 + tid / C::CPR + i * C::RPP;
-    r = r < nrows ? r : nrows - 1;
-    reg[i] = *(const u32x4*)(base + (int64_t)r * stride + (tid % C::CPR) * 8);
-  }
-}
-
+// Chunk permutation of a tile row, good for both read patterns: 16 consecutive rows at one chunk
+// index fall into 16 different 16-byte bank groups, and so do the 4 rows x 4 chunks a half wave
+// covers with one transposing read.  Depends on row % 16 only.
 template <int D>
-__device__ __forceinline__ void rows_lstore(unsigned char* lds, const u32x4 (&reg)[TileCfg<D>::PASS], int tid) {
-  typedef TileCfg<D> C;
-#pragma unroll
-  for (int i = 0; i < C::PASS; ++i)
-    *(u32x4*)(lds + (tid / C::CPR + i * C::RPP) * C::KP + (tid % C::CPR) * 16) = reg[i];
+__device__ __forceinline__ int tile_swizzle(int row) {
+  return D == 128 ? ((row & 3) << 2) | ((row >> 2) & 3)
+         : D == 64 ? (((row >> 1) & 1) << 2) | ((row >> 2) & 3)
+                   : (row >> 2) & 3;
 }
 
-// ---- streamed tile, transposed: D rows x 64 (permuted) columns; a thread moves 4 rows x 8 dims ----
-template <typename T, int D>
-__device__ __forceinline__ void tr_gload(u32x4 (&reg)[4], const T* base, int64_t stride, int row0, int nrows,
-                                         int tid) {
-  if (tid < TileCfg<D>::UNITS) {
-    const int g = tid & 15, dc = tid >> 4;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      int r = row0 + g * 4 + j;
-      r = r < nrows ? r : nrows - 1;
-      reg[j] = *(const u32x4*)(base + (int64_t)r * stride + dc * 8);
-    }
-  }
-}
-
+// Per-lane LDS offsets (relative to a tile) of the two read patterns.
 template <int D>
-__device__ __forceinline__ void tr_lstore(unsigned char* lds, const u32x4 (&reg)[4], int tid) {
-  typedef TileCfg<D> C;
-  if (tid < C::UNITS) {
-    const int g = tid & 15, dc = tid >> 4;
-    const int pos = (g >> 3) * 32 + ((g >> 2) & 1) * 16 + (g & 1) * 8 + ((g >> 1) & 1) * 4;
+struct TileReads {
+  unsigned row[D / 16];     // chunk 2 ks + hh of row ln (+ 32 rows: second half)
+  unsigned tr[D / 32][2];   // transposing read of 4 dims of row 8 h8 + 4 hh + e (+ 16 u rows, + 32 rows)
+  __device__ __forceinline__ void init(int lane) {
+    typedef BwdCfg<D> C;
+    const int ln = lane & 31, hh = lane >> 5;
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      const unsigned a0 = reg[0][m], a1 = reg[1][m], a2 = reg[2][m], a3 = reg[3][m];
-      u32x2 even, odd;
-      even[0] = (a0 & 0xffffu) | (a1 << 16);
-      even[1] = (a2 & 0xffffu) | (a3 << 16);
-      odd[0] = (a0 >> 16) | (a1 & 0xffff0000u);
-      odd[1] = (a2 >> 16) | (a3 & 0xffff0000u);
-      *(u32x2*)(lds + (dc * 8 + 2 * m) * C::VP + pos * 2) = even;
-      *(u32x2*)(lds + (dc * 8 + 2 * m + 1) * C::VP + pos * 2) = odd;
-    }
+    for (int ks = 0; ks < D / 16; ++ks) row[ks] = ln * C::ROWB + (((2 * ks + hh) ^ tile_swizzle<D>(ln)) * 16);
+    const int blk = lane >> 4, e = (lane >> 2) & 3, c4 = lane & 3;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int h8 = 0; h8 < 2; ++h8) {
+        const int r = 8 * h8 + 4 * hh + e;
+        const int chunk = db * 4 + (blk & 1) * 2 + (c4 >> 1);
+        tr[db][h8] = r * C::ROWB + ((chunk ^ tile_swizzle<D>(r)) * 16) + (c4 & 1) * 8;
+      }
   }
-}
+};
 
-template <typename F, int D>
-__device__ __forceinline__ F row_frag(const unsigned char* lds, int row, int ks, int hh) {
-  return as_frag<F>(*(const u32x4*)(lds + row * TileCfg<D>::KP + (ks * 16 + hh * 8) * 2));
-}
+// Global side of the direct loads: thread tid owns 16-byte slot tid of every round of 256 slots;
+// round j covers rows j * RPD + tid / CPR.  Slot (row, pos) receives chunk pos ^ swizzle(row).
+template <typename T, int D>
+struct TileLoader {
+  u32x4 rsrc;
+  unsigned lane_off;  // bytes
+  unsigned row_b;     // bytes per tensor row
+  __device__ __forceinline__ void init(const T* base, int64_t row_stride, int rows, int tid) {
+    typedef BwdCfg<D> C;
+    rsrc = buffer_descriptor(base, (unsigned)((((int64_t)rows - 1) * row_stride + D) * (int64_t)sizeof(T)));
+    const int drow = tid / C::CPR, dpos = tid % C::CPR;
+    lane_off = (unsigned)((drow * row_stride + ((dpos ^ tile_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(T));
+    row_b = (unsigned)(row_stride * (int64_t)sizeof(T));
+  }
+  // round q of the tile whose first tensor row is row0 (on = false: store zeros) into LDS at lds_wave
+  __device__ __forceinline__ void load(int q, bool on, int row0, unsigned lds_wave) const {
+    typedef BwdCfg<D> C;
+    const unsigned u = on ? (unsigned)(row0 + q * C::RPD) * row_b : OFF_NONE;
+    load_to_lds_b128(rsrc, lane_off + u, lds_wave + q * (BWD_THREADS * 16));
+  }
+};
 
-template <typename F, int D>
-__device__ __forceinline__ F tr_frag(const unsigned char* lds, int row, int t, int u, int hh) {
-  return as_frag<F>(*(const u32x4*)(lds + row * TileCfg<D>::VP + (t * 32 + u * 16 + hh * 8) * 2));
+// One MFMA operand from two transposing reads (rows 0..3 and 8..11 of a lane's group of 16).
+template <typename F>
+__device__ __forceinline__ F frag_tr(unsigned addr_lo, unsigned addr_hi) {
+  const u32x2 r0 = lds_read_tr16_b64(addr_lo);
+  const u32x2 r1 = lds_read_tr16_b64(addr_hi);
+  u32x4 x;
+  x[0] = r0[0];
+  x[1] = r0[1];
+  x[2] = r1[0];
+  x[3] = r1[1];
+  return as_frag<F>(x);
 }
 
 __device__ __forceinline__ void zero16(f32x16& x) {
@@ -106,25 +116,34 @@ __device__ __forceinline__ void zero16(f32x16& x) {
   for (int v = 0; v < 16; ++v) x[v] = 0.f;
 }
 
+template <int N>
+__device__ __forceinline__ void wait_loads_but() {  // until at most N of this wave's loads are in flight
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
 // ------------------------------------------------------------------------------------------
 // dQ kernel
 // ------------------------------------------------------------------------------------------
 template <int D>
 struct DqCfg {
-  typedef TileCfg<D> C;
-  static constexpr int STAGE = 2 * C::ROWB + C::TRB;  // K rows, V rows, K^T
-  static constexpr int SMEM = 2 * STAGE;
+  typedef BwdCfg<D> C;
+  static constexpr int STAGE = 2 * C::TILEB;  // K tile, V tile
+  static constexpr int SMEM = BWD_STAGES * STAGE;
+  static constexpr int NL = 2 * C::NDMA;      // loads per thread and stage
 };
 
 template <typename T, int D>
 __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dq_kernel(const BwdParams p) {
-  typedef TileCfg<D> C;
+  typedef BwdCfg<D> C;
+  typedef DqCfg<D> G;
   typedef Mma16<T> M;
   typedef typename M::frag frag;
   extern __shared__ __align__(16) unsigned char smem[];
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, w = tid >> 6, ln = lane & 31, hh = lane >> 5;
+  const int lane = tid & 63, ln = lane & 31, hh = lane >> 5;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   int bid = blockIdx.x;
   const int h = bid % p.H;
@@ -152,83 +171,144 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dq_kernel(const BwdP
   const float l2 = p.lse[li] * 1.4426950408889634f;
   const float dl = p.delta[li];
   const float c = p.scale_log2;
+  const int lim = p.causal ? (qrow < p.Sk - 1 ? qrow : p.Sk - 1) : p.Sk - 1;  // last visible key
 
   const int kv_end = p.causal ? (q0 + 128 < p.Sk ? q0 + 128 : p.Sk) : p.Sk;
-  const int nt = (kv_end + BWD_ROWS - 1) / BWD_ROWS;
+  const int nt = (kv_end + BWD_ROWS - 1) / BWD_ROWS;  // key tiles this workgroup visits
 
-  u32x4 kreg[C::PASS], vreg[C::PASS], ktreg[4];
-  auto gload = [&](int it) {
-    rows_gload<T, D>(kreg, kp, p.ks.s, it * BWD_ROWS, p.Sk, tid);
-    rows_gload<T, D>(vreg, vp, p.vs.s, it * BWD_ROWS, p.Sk, tid);
-    tr_gload<T, D>(ktreg, kp, p.ks.s, it * BWD_ROWS, p.Sk, tid);
-  };
-  auto lstore = [&](int stage) {
-    unsigned char* sb = smem + stage * DqCfg<D>::STAGE;
-    rows_lstore<D>(sb, kreg, tid);
-    rows_lstore<D>(sb + C::ROWB, vreg, tid);
-    tr_lstore<D>(sb + 2 * C::ROWB, ktreg, tid);
+  TileLoader<T, D> kld, vld;
+  kld.init(kp, p.ks.s, p.Sk, tid);
+  vld.init(vp, p.vs.s, p.Sk, tid);
+  TileReads<D> rd;
+  rd.init(lane);
+  const unsigned lds0 = (unsigned)(uintptr_t)(lds_u8*)smem;
+  auto stage_of = [&](int i) { return lds0 + (unsigned)((i & (BWD_STAGES - 1)) * G::STAGE); };
+  auto issue_tile = [&](int i) {  // K and V tile i -> its stage
+    const unsigned dst = stage_of(i) + w * 1024;
+#pragma unroll
+    for (int q = 0; q < C::NDMA; ++q) kld.load(q, i < nt, i * BWD_ROWS, dst);
+#pragma unroll
+    for (int q = 0; q < C::NDMA; ++q) vld.load(q, i < nt, i * BWD_ROWS, dst + C::TILEB);
   };
 
   f32x16 dq[D / 32];
 #pragma unroll
   for (int i = 0; i < D / 32; ++i) zero16(dq[i]);
 
-  gload(0);
-  lstore(0);
+  // Half-tile g = 2 i + t is keys [32 g, 32 g + 32).  One pass of the loop body handles tile i:
+  //   list 2i  : S^T, dP^T of half 2i+1 (tile i, rows 32..63)   | dS^T of half 2i   | dQ of half 2i
+  //   list 2i+1: S^T, dP^T of half 2i+2 (tile i+1, rows 0..31)  | dS^T of half 2i+1 | dQ of half 2i+1
+  // NA MFMAs produce, the element-wise work rides between them, NB MFMAs consume.
+  constexpr int NA = 2 * (D / 16), NB = 2 * (D / 32), NLIST = NA + NB, NBODY = 2 * NLIST;
+  constexpr int BWD_LOOK = NA < BWD_LOOK_MAX ? NA : BWD_LOOK_MAX;
+  static_assert(NBODY % BWD_LOOK == 0 && BWD_LOOK <= NA, "the operand window must tile the loop body");
+
+  issue_tile(0);
+  issue_tile(1);
+  issue_tile(2);
+  wait_loads_but<2 * G::NL>();
   __syncthreads();
 
-  for (int it = 0; it < nt; ++it) {
-    const int cur = it & 1;
-    const int key0 = it * BWD_ROWS;
-    const bool more = it + 1 < nt;
-    if (more) gload(it + 1);
-
-    const bool active = !(p.causal && key0 > qw0 + 31);
-    if (active) {
-      const unsigned char* kb = smem + cur * DqCfg<D>::STAGE;
-      const unsigned char* vb = kb + C::ROWB;
-      const unsigned char* ktb = kb + 2 * C::ROWB;
-
-      f32x16 s[2], dp[2];
+  f32x16 sc, dc, sn, dn;  // S^T, dP^T of the current / next half-tile
+  {
+    zero16(sc);
+    zero16(dc);
+    const unsigned kb = stage_of(0);
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        zero16(s[t]);
-        zero16(dp[t]);
-#pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) {
-          s[t] = M::run(row_frag<frag, D>(kb, t * 32 + ln, ks, hh), qf[ks], s[t]);
-          dp[t] = M::run(row_frag<frag, D>(vb, t * 32 + ln, ks, hh), dof[ks], dp[t]);
-        }
-      }
-
-      const int lim = p.causal ? (qrow < p.Sk - 1 ? qrow : p.Sk - 1) : p.Sk - 1;  // last visible key
-      frag dsf[2][2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int key = key0 + t * 32 + 8 * (v >> 2) + 4 * hh + (v & 3);
-          const float pr = key > lim ? 0.f : fast_exp2(__builtin_fmaf(s[t][v], c, -l2));
-          s[t][v] = pr * (dp[t][v] - dl);
-        }
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-          dsf[t][u] = M::pack(s[t][8 * u + 0], s[t][8 * u + 1], s[t][8 * u + 2], s[t][8 * u + 3],
-                              s[t][8 * u + 4], s[t][8 * u + 5], s[t][8 * u + 6], s[t][8 * u + 7]);
-      }
-
-#pragma unroll
-      for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int u = 0; u < 2; ++u)
-            dq[db] = M::run(tr_frag<frag, D>(ktb, db * 32 + ln, t, u, hh), dsf[t][u], dq[db]);
+    for (int ks = 0; ks < D / 16; ++ks) {
+      sc = M::run(as_frag<frag>(lds_read_b128(kb + rd.row[ks])), qf[ks], sc);
+      dc = M::run(as_frag<frag>(lds_read_b128(kb + C::TILEB + rd.row[ks])), dof[ks], dc);
     }
-
-    if (more) lstore(cur ^ 1);
-    __syncthreads();
   }
+
+  // operand fetch number J of the body of tile i (J >= NBODY: the first operands of the next body)
+  unsigned row_cur[D / 16], row_nxt[D / 16], tr_cur[D / 32][2];
+  auto set_addresses = [&](int i) {
+    const unsigned a = stage_of(i), n = stage_of(i + 1);
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      row_cur[ks] = a + rd.row[ks];
+      row_nxt[ks] = n + rd.row[ks];
+    }
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int h8 = 0; h8 < 2; ++h8) tr_cur[db][h8] = a + rd.tr[db][h8];
+  };
+  auto fetch = [&](int J) -> frag {
+    const int body = J / NBODY, j2 = J % NBODY;
+    const int list = j2 / NLIST, j = j2 % NLIST;
+    if (j < NA) {  // j = 2 ks + which: K row (S^T) or V row (dP^T) of the half-tile being produced
+      const int ks = j >> 1, which = j & 1;
+      // list 0 of this body: tile i rows 32..; list 1: tile i+1 rows 0..; list 0 of the next body: tile i+1 rows 32..
+      const unsigned base = (body == 0 && list == 0) ? row_cur[ks] + 32 * C::ROWB
+                            : (body == 0)           ? row_nxt[ks]
+                                                    : row_nxt[ks] + 32 * C::ROWB;
+      return as_frag<frag>(lds_read_b128(base + which * C::TILEB));
+    }
+    const int jb = j - NA;  // jb = u * (D/32) + db : K^T operand of half-tile `list` of tile i
+    const int db = jb % (D / 32), u = jb / (D / 32);
+    const unsigned off = (list * 32 + u * 16) * C::ROWB;
+    return frag_tr<frag>(tr_cur[db][0] + off, tr_cur[db][1] + off);
+  };
+
+  frag win[BWD_LOOK];
+  frag dsf[2];
+  set_addresses(0);
+#pragma unroll
+  for (int j = 0; j < BWD_LOOK; ++j) win[j] = fetch(j);
+  for (int i = 0; i < nt; ++i) {
+    // tile i+1 must have landed before this body reads it; tile i-1 is free for tile i+3
+    wait_loads_but<G::NL>();
+    __syncthreads();
+    issue_tile(i + 3);
+    set_addresses(i);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int list = 0; list < 2; ++list) {
+      const int key0 = (2 * i + list) * 32;  // first key of the half-tile whose dS is formed in this list
+      if (p.causal && key0 + 31 > qw0) {     // diagonal: hide the keys after each lane's query
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          if (key0 + 8 * (v >> 2) + 4 * hh + (v & 3) > lim) sc[v] = -INFINITY;
+      }
+      zero16(sn);
+      zero16(dn);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < NLIST; ++j) {
+        const int J = list * NLIST + j;
+        const frag a = win[J % BWD_LOOK];
+        win[J % BWD_LOOK] = fetch(J + BWD_LOOK);
+        __builtin_amdgcn_sched_barrier(0);
+        if (j < NA) {
+          const int ks = j >> 1;
+          if (j & 1)
+            dn = M::run(a, dof[ks], dn);
+          else
+            sn = M::run(a, qf[ks], sn);
+          // element-wise work on the current half-tile, spread over the producing MFMAs
+#pragma unroll
+          for (int v = 0; v < 16; ++v)
+            if (v * NA / 16 == j) {
+              const float pr = fast_exp2(__builtin_fmaf(sc[v], c, -l2));
+              sc[v] = pr * (dc[v] - dl);
+            }
+          if (j == NA / 2 - 1)
+            dsf[0] = M::pack(sc[0], sc[1], sc[2], sc[3], sc[4], sc[5], sc[6], sc[7]);
+          if (j == NA - 1) dsf[1] = M::pack(sc[8], sc[9], sc[10], sc[11], sc[12], sc[13], sc[14], sc[15]);
+        } else {
+          const int jb = j - NA;
+          const int db = jb % (D / 32), u = jb / (D / 32);
+          dq[db] = M::run(a, dsf[u], dq[db]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      sc = sn;
+      dc = dn;
+    }
+  }
+  wait_loads_but<0>();  // nothing may still be writing LDS when the workgroup ends
 
   if (qrow < p.Sq) {
     float* dqp = p.dq + b * p.dqs.b + h * p.dqs.h + (int64_t)qrow * p.dqs.s;
@@ -252,21 +332,24 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dq_kernel(const BwdP
 // ------------------------------------------------------------------------------------------
 template <int D>
 struct DkvCfg {
-  typedef TileCfg<D> C;
-  static constexpr int STAT = 2 * BWD_ROWS * 4;               // lse*log2e and delta of the tile rows
-  static constexpr int STAGE = 2 * C::ROWB + 2 * C::TRB + STAT;  // Q rows, dO rows, Q^T, dO^T, stats
-  static constexpr int SMEM = 2 * STAGE;
+  typedef BwdCfg<D> C;
+  static constexpr int STAT = 2 * BWD_ROWS * 4;       // lse and delta of the tile's query rows
+  static constexpr int STAGE = 2 * C::TILEB + STAT;   // Q tile, dO tile, stats
+  static constexpr int SMEM = BWD_STAGES * STAGE;
+  static constexpr int NL = 2 * C::NDMA + 1;          // loads per thread and stage
 };
 
 template <typename T, int D>
 __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const BwdParams p) {
-  typedef TileCfg<D> C;
+  typedef BwdCfg<D> C;
+  typedef DkvCfg<D> G;
   typedef Mma16<T> M;
   typedef typename M::frag frag;
   extern __shared__ __align__(16) unsigned char smem[];
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, w = tid >> 6, ln = lane & 31, hh = lane >> 5;
+  const int lane = tid & 63, ln = lane & 31, hh = lane >> 5;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   int bid = blockIdx.x;
   const int h = bid % p.H;
@@ -294,36 +377,29 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
   }
   const float c = p.scale_log2;
 
-  // causal: query rows below the first key of this workgroup see none of its keys
+  // causal: query rows before the first key of this workgroup see none of its keys
   const int it0 = p.causal ? k0 / BWD_ROWS : 0;
-  const int nt = (p.Sq + BWD_ROWS - 1) / BWD_ROWS;
+  const int nt = (p.Sq + BWD_ROWS - 1) / BWD_ROWS;  // query tiles it0 .. nt-1 are visited
 
-  u32x4 qreg[C::PASS], doreg[C::PASS], qtreg[4], dotreg[4];
-  float st_l = 0.f, st_d = 0.f;
-  auto gload = [&](int it) {
-    const int r0 = it * BWD_ROWS;
-    rows_gload<T, D>(qreg, qp, p.qs.s, r0, p.Sq, tid);
-    rows_gload<T, D>(doreg, dop, p.dos.s, r0, p.Sq, tid);
-    tr_gload<T, D>(qtreg, qp, p.qs.s, r0, p.Sq, tid);
-    tr_gload<T, D>(dotreg, dop, p.dos.s, r0, p.Sq, tid);
-    if (tid < BWD_ROWS) {
-      int r = r0 + tid;
-      r = r < p.Sq ? r : p.Sq - 1;
-      st_l = lsep[r] * 1.4426950408889634f;
-      st_d = delp[r];
-    }
-  };
-  auto lstore = [&](int stage) {
-    unsigned char* sb = smem + stage * DkvCfg<D>::STAGE;
-    rows_lstore<D>(sb, qreg, tid);
-    rows_lstore<D>(sb + C::ROWB, doreg, tid);
-    tr_lstore<D>(sb + 2 * C::ROWB, qtreg, tid);
-    tr_lstore<D>(sb + 2 * C::ROWB + C::TRB, dotreg, tid);
-    if (tid < BWD_ROWS) {
-      float* stp = (float*)(sb + 2 * C::ROWB + 2 * C::TRB);
-      stp[tid] = st_l;
-      stp[BWD_ROWS + tid] = st_d;
-    }
+  TileLoader<T, D> qld, dold;
+  qld.init(qp, p.qs.s, p.Sq, tid);
+  dold.init(dop, p.dos.s, p.Sq, tid);
+  // per-row statistics: waves 0, 2 fetch the tile's 64 lse values, waves 1, 3 its 64 delta values
+  // (the pairs store the same bytes to the same place, which keeps every wave's load count equal)
+  const u32x4 stat_rsrc = buffer_descriptor((w & 1) ? delp : lsep, (unsigned)p.Sq * 4u);
+  TileReads<D> rd;
+  rd.init(lane);
+  const unsigned lds0 = (unsigned)(uintptr_t)(lds_u8*)smem;
+  auto stage_of = [&](int i) { return lds0 + (unsigned)((i & (BWD_STAGES - 1)) * G::STAGE); };
+  auto issue_tile = [&](int i) {  // Q and dO tile i and their statistics -> stage
+    const unsigned st = stage_of(i);
+    const unsigned dst = st + w * 1024;
+#pragma unroll
+    for (int q = 0; q < C::NDMA; ++q) qld.load(q, i < nt, i * BWD_ROWS, dst);
+#pragma unroll
+    for (int q = 0; q < C::NDMA; ++q) dold.load(q, i < nt, i * BWD_ROWS, dst + C::TILEB);
+    load_to_lds_b32(stat_rsrc, i < nt ? (unsigned)(i * BWD_ROWS + lane) * 4u : OFF_NONE,
+                    st + 2 * C::TILEB + (w & 1) * (BWD_ROWS * 4));
   };
 
   f32x16 dk[D / 32], dv[D / 32];
@@ -333,78 +409,141 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
     zero16(dv[i]);
   }
 
-  if (it0 < nt) {
-    gload(it0);
-    lstore(it0 & 1);
-  }
-  __syncthreads();
+  // Half-tile g = 2 i + t is query rows [32 g, 32 g + 32).  Body of tile i:
+  //   list 2i  : S, dP of half 2i+1 (tile i rows 32..63)  | P, dS of half 2i   | dV, dK from half 2i
+  //   list 2i+1: S, dP of half 2i+2 (tile i+1 rows 0..31) | P, dS of half 2i+1 | dV, dK from half 2i+1
+  constexpr int NA = 2 * (D / 16), NB = 4 * (D / 32), NLIST = NA + NB, NBODY = 2 * NLIST;
+  constexpr int BWD_LOOK = NA < BWD_LOOK_MAX ? NA : BWD_LOOK_MAX;
+  static_assert(NBODY % BWD_LOOK == 0 && BWD_LOOK <= NA, "the operand window must tile the loop body");
 
-  for (int it = it0; it < nt; ++it) {
-    const int cur = it & 1;
-    const int r0 = it * BWD_ROWS;
-    const bool more = it + 1 < nt;
-    if (more) gload(it + 1);
+  if (it0 < nt) {  // uniform; a workgroup whose keys no query sees adds nothing
+    issue_tile(it0);
+    issue_tile(it0 + 1);
+    issue_tile(it0 + 2);
+    wait_loads_but<2 * G::NL>();
+    __syncthreads();
 
-    // a wave whose keys all come after this query tile contributes nothing to it
-    const bool active = !(p.causal && r0 + BWD_ROWS - 1 < kw0);
-    if (active) {
-      const unsigned char* qb = smem + cur * DkvCfg<D>::STAGE;
-      const unsigned char* dob = qb + C::ROWB;
-      const unsigned char* qtb = qb + 2 * C::ROWB;
-      const unsigned char* dotb = qtb + C::TRB;
-      const float* stp = (const float*)(dotb + C::TRB);
-
-      f32x16 s[2], dp[2];
+    f32x16 sc, dc, sn, dn;
+    {
+      zero16(sc);
+      zero16(dc);
+      const unsigned qb = stage_of(it0);
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        zero16(s[t]);
-        zero16(dp[t]);
-#pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) {
-          s[t] = M::run(row_frag<frag, D>(qb, t * 32 + ln, ks, hh), kf[ks], s[t]);
-          dp[t] = M::run(row_frag<frag, D>(dob, t * 32 + ln, ks, hh), vf[ks], dp[t]);
-        }
+      for (int ks = 0; ks < D / 16; ++ks) {
+        sc = M::run(as_frag<frag>(lds_read_b128(qb + rd.row[ks])), kf[ks], sc);
+        dc = M::run(as_frag<frag>(lds_read_b128(qb + C::TILEB + rd.row[ks])), vf[ks], dc);
       }
+    }
 
-      frag pf[2][2], dsf[2][2];
+    unsigned row_cur[D / 16], row_nxt[D / 16], tr_cur[D / 32][2];
+    unsigned stat_cur;
+    auto set_addresses = [&](int i) {
+      const unsigned a = stage_of(i), n = stage_of(i + 1);
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const f32x4 l4 = *(const f32x4*)(stp + t * 32 + 8 * g + 4 * hh);
-          const f32x4 d4 = *(const f32x4*)(stp + BWD_ROWS + t * 32 + 8 * g + 4 * hh);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int v = 4 * g + e;
-            const int qi = r0 + t * 32 + 8 * g + 4 * hh + e;  // query row of this accumulator
-            const bool dead = qi >= p.Sq || (p.causal && krow > qi);
-            const float pr = dead ? 0.f : fast_exp2(__builtin_fmaf(s[t][v], c, -l4[e]));
-            s[t][v] = pr;
-            dp[t][v] = pr * (dp[t][v] - d4[e]);
-          }
-        }
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          pf[t][u] = M::pack(s[t][8 * u + 0], s[t][8 * u + 1], s[t][8 * u + 2], s[t][8 * u + 3],
-                             s[t][8 * u + 4], s[t][8 * u + 5], s[t][8 * u + 6], s[t][8 * u + 7]);
-          dsf[t][u] = M::pack(dp[t][8 * u + 0], dp[t][8 * u + 1], dp[t][8 * u + 2], dp[t][8 * u + 3],
-                              dp[t][8 * u + 4], dp[t][8 * u + 5], dp[t][8 * u + 6], dp[t][8 * u + 7]);
-        }
+      for (int ks = 0; ks < D / 16; ++ks) {
+        row_cur[ks] = a + rd.row[ks];
+        row_nxt[ks] = n + rd.row[ks];
       }
-
 #pragma unroll
       for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int u = 0; u < 2; ++u) {
-            dv[db] = M::run(tr_frag<frag, D>(dotb, db * 32 + ln, t, u, hh), pf[t][u], dv[db]);
-            dk[db] = M::run(tr_frag<frag, D>(qtb, db * 32 + ln, t, u, hh), dsf[t][u], dk[db]);
-          }
-    }
+        for (int h8 = 0; h8 < 2; ++h8) tr_cur[db][h8] = a + rd.tr[db][h8];
+      stat_cur = a + 2 * C::TILEB + 16 * hh;
+    };
+    auto fetch = [&](int J) -> frag {
+      const int body = J / NBODY, j2 = J % NBODY;
+      const int list = j2 / NLIST, j = j2 % NLIST;
+      if (j < NA) {  // j = 2 ks + which: Q row (S) or dO row (dP) of the half-tile being produced
+        const int ks = j >> 1, which = j & 1;
+        const unsigned base = (body == 0 && list == 0) ? row_cur[ks] + 32 * C::ROWB
+                              : (body == 0)           ? row_nxt[ks]
+                                                      : row_nxt[ks] + 32 * C::ROWB;
+        return as_frag<frag>(lds_read_b128(base + which * C::TILEB));
+      }
+      // jb = (u * (D/32) + db) * 2 + which: dO^T (for dV) or Q^T (for dK) operand of half-tile `list`
+      const int jb = j - NA;
+      const int which = jb & 1, db = (jb >> 1) % (D / 32), u = (jb >> 1) / (D / 32);
+      const unsigned off = (which ? 0 : C::TILEB) + (list * 32 + u * 16) * C::ROWB;
+      return frag_tr<frag>(tr_cur[db][0] + off, tr_cur[db][1] + off);
+    };
 
-    if (more) lstore(cur ^ 1);
-    __syncthreads();
+    frag win[BWD_LOOK];
+    frag pf[2], dsf[2];
+    set_addresses(it0);
+#pragma unroll
+    for (int j = 0; j < BWD_LOOK; ++j) win[j] = fetch(j);
+    for (int i = it0; i < nt; ++i) {
+      wait_loads_but<G::NL>();
+      __syncthreads();
+      issue_tile(i + 3);
+      set_addresses(i);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int list = 0; list < 2; ++list) {
+        const int r0 = (2 * i + list) * 32;  // first query row of the half-tile whose P, dS are formed here
+        if (p.causal && kw0 + 31 > r0) {     // diagonal: a key sees only the queries at or after it
+#pragma unroll
+          for (int v = 0; v < 16; ++v)
+            if (krow > r0 + 8 * (v >> 2) + 4 * hh + (v & 3)) sc[v] = -INFINITY;
+        }
+        // lse (times -log2 e) and delta of this lane's 16 query rows
+        float nl[16], de[16];
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          // (whole-vector casts: a bit cast of one element of a vector reads element 0)
+          const f32x4 l4 = __builtin_bit_cast(f32x4, lds_read_b128(stat_cur + (list * 32 + 8 * g4) * 4));
+          const f32x4 d4 = __builtin_bit_cast(f32x4, lds_read_b128(stat_cur + (BWD_ROWS + list * 32 + 8 * g4) * 4));
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            nl[4 * g4 + e] = l4[e] * -1.4426950408889634f;
+            de[4 * g4 + e] = d4[e];
+          }
+        }
+        zero16(sn);
+        zero16(dn);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < NLIST; ++j) {
+          const int J = list * NLIST + j;
+          const frag a = win[J % BWD_LOOK];
+          win[J % BWD_LOOK] = fetch(J + BWD_LOOK);
+          __builtin_amdgcn_sched_barrier(0);
+          if (j < NA) {
+            const int ks = j >> 1;
+            if (j & 1)
+              dn = M::run(a, vf[ks], dn);
+            else
+              sn = M::run(a, kf[ks], sn);
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+              if (v * NA / 16 == j) {
+                const float pr = fast_exp2(__builtin_fmaf(sc[v], c, nl[v]));
+                sc[v] = pr;
+                dc[v] = pr * (dc[v] - de[v]);
+              }
+            if (j == NA / 2 - 1) {
+              pf[0] = M::pack(sc[0], sc[1], sc[2], sc[3], sc[4], sc[5], sc[6], sc[7]);
+              dsf[0] = M::pack(dc[0], dc[1], dc[2], dc[3], dc[4], dc[5], dc[6], dc[7]);
+            }
+            if (j == NA - 1) {
+              pf[1] = M::pack(sc[8], sc[9], sc[10], sc[11], sc[12], sc[13], sc[14], sc[15]);
+              dsf[1] = M::pack(dc[8], dc[9], dc[10], dc[11], dc[12], dc[13], dc[14], dc[15]);
+            }
+          } else {
+            const int jb = j - NA;
+            const int which = jb & 1, db = (jb >> 1) % (D / 32), u = (jb >> 1) / (D / 32);
+            if (which)
+              dk[db] = M::run(a, dsf[u], dk[db]);
+            else
+              dv[db] = M::run(a, pf[u], dv[db]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        sc = sn;
+        dc = dn;
+      }
+    }
+    wait_loads_but<0>();
   }
 
   if (krow < p.Sk) {

@@ -69,18 +69,6 @@ __device__ __forceinline__ int v_swizzle(int row) {
   return D == 128 ? (row & 3) << 2 : D == 64 ? ((row >> 1) & 1) << 2 : 0;
 }
 
-typedef __attribute__((address_space(3))) unsigned char lds_u8;
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-
-// 16 bytes per lane from a buffer straight into LDS at lds_addr + 16 * lane (lds_addr wave-uniform);
-// out-of-range lanes store zeros.  Counts on vmcnt like any load.
-__device__ __forceinline__ void load_to_lds_b128(u32x4 rsrc, unsigned voffset, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-               :
-               : "s"(lds_addr), "v"(voffset), "s"(rsrc)
-               : "memory");
-}
-
 template <typename T, int D, int NG>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams p) {
   typedef Fwd16Cfg<D, NG> C;

@@ -119,5 +119,46 @@ static __device__ __forceinline__ float xhalf(float x) {
   return __shfl_xor(x, 32, 64);
 }
 
+// ---- LDS helpers shared by the attention kernels ----
+typedef __attribute__((address_space(3))) unsigned char lds_u8;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+// 16 bytes per lane from a buffer straight into LDS at lds_addr + 16 * lane (lds_addr wave-uniform);
+// out-of-range lanes store zeros.  Counts on vmcnt like any load.  Issued from inline asm: the
+// compiler knows nothing of it, so the caller orders it against LDS reads (vmcnt wait + barrier).
+static __device__ __forceinline__ void load_to_lds_b128(u32x4 rsrc, unsigned voffset, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :
+               : "s"(lds_addr), "v"(voffset), "s"(rsrc)
+               : "memory");
+}
+// The same for 4 bytes per lane: LDS at lds_addr + 4 * lane.
+static __device__ __forceinline__ void load_to_lds_b32(u32x4 rsrc, unsigned voffset, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds"
+               :
+               : "s"(lds_addr), "v"(voffset), "s"(rsrc)
+               : "memory");
+}
+// Raw buffer descriptor (stride 0) over `bytes` bytes at base; every component wave-uniform.
+static __device__ __forceinline__ u32x4 buffer_descriptor(const void* base, unsigned bytes) {
+  const unsigned long long a = (unsigned long long)base;
+  u32x4 r;
+  r[0] = __builtin_amdgcn_readfirstlane((unsigned)a);
+  r[1] = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32) & 0xffffu);
+  r[2] = __builtin_amdgcn_readfirstlane(bytes);
+  r[3] = 0x00020000u;
+  return r;
+}
+// Transposing LDS read: in a block of 16 lanes, lane 4 e + c supplies the address of 8 bytes
+// (4 elements) of row e, and lane x receives element x (of the 16 the row's four pieces hold)
+// of rows 0..3.
+static __device__ __forceinline__ u32x2 lds_read_tr16_b64(unsigned lds_addr) {
+  return __builtin_bit_cast(
+      u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(lds_u8*)(uintptr_t)lds_addr));
+}
+static __device__ __forceinline__ u32x4 lds_read_b128(unsigned lds_addr) {
+  return *(const __attribute__((address_space(3))) u32x4*)(lds_u8*)(uintptr_t)lds_addr;
+}
+
 static __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 static __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
