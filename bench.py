@@ -210,11 +210,17 @@ def side_workload(torch, name, steps, warmup):
         q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
         scale = Dn ** -0.5
         out, lse = spa.ring.ring_flash_attn_forward(q, k, v, scale, True, Pn, fuse="all")
-        fn = lambda: spa.ring.ring_flash_attn_backward(dout, q, k, v, out, lse, scale, True, Pn)
+        fn = lambda: spa.ring.ring_flash_attn_backward(dout, q, k, v, out, lse, scale, True, Pn, fuse="all")
+        fn_step = lambda: spa.ring.ring_flash_attn_backward(dout, q, k, v, out, lse, scale, True, Pn, fuse="step")
         fwd_flops = 4.0 * Bn * Hn * Sn * Sn * Dn / 2
         units, unit_flops = 1, 2.5 * fwd_flops   # five GEMMs of the algorithm (the two kernels recompute S and dP: 7 executed)
         bound, kernel, metric = "mfma", "flash_bwd_dq_kernel + flash_bwd_dkdv_kernel", "ring backward TFLOP/s (5-GEMM count, causal-adjusted), config 5 S=32K H16 D128 P=16"
-        work = {"workload": "config 5 backward: bf16 qkv [1,32768,3,16,128] causal, ring of 16 chunks, dq/dk/dv by block-wise recompute", "flops_per_step": unit_flops}
+        work = {"workload": "config 5 backward: bf16 qkv [1,32768,3,16,128] causal, ring of 16 chunks, dq/dk/dv by block-wise "
+                            "recompute with the global lse; value = the 136 block pairs walked inside one launch per kernel "
+                            "(delta pre-pass, fp32 accumulator zeroing and the final casts included)", "flops_per_step": unit_flops}
+        fn_step()
+        t_step = time_region(torch, fn_step, 3)
+        work["one_launch_per_block_pair"] = {"ms_per_step": round(t_step, 3), "tflops": round(unit_flops / (t_step * 1e-3) / 1e12, 2)}
     else:
         raise SystemExit(f"unknown workload {name}")
     for _ in range(warmup):

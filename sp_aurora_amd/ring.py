@@ -113,7 +113,8 @@ def make_ring_forward_step(q, k, v, softmax_scale=None, causal=False, ring_size=
     return step
 
 
-def ring_flash_attn_backward(dout, q, k, v, out, softmax_lse, softmax_scale=None, causal=False, ring_size=1):
+def ring_flash_attn_backward(dout, q, k, v, out, softmax_lse, softmax_scale=None, causal=False, ring_size=1,
+                             fuse="all"):
     """dq, dk, dv of ring attention by block-wise recompute with the global lse.
 
     The schedule is the reference's (sp_aurora/intel_ring_flash_attn.py:192-271): per visited
@@ -121,7 +122,15 @@ def ring_flash_attn_backward(dout, q, k, v, out, softmax_lse, softmax_scale=None
     dk/dv summed per kv chunk over the q chunks that visited it (:257-258,267), cast at the
     end (:271).  Each block uses P = exp(S - lse) with the lse of the WHOLE ring, which makes
     the sum the exact gradient (the reference normalises each block on its own, :229-244).
+
+    fuse="step" launches one backward block per visited pair, in the reference's order, adding
+    into the fp32 accumulators (what a rank of a real ring does as chunks arrive); fuse="all"
+    walks the same pairs inside one launch of each kernel (the blocks of a simulated ring tile
+    the causal / full score matrix exactly, and with a shared global lse their sum is the
+    backward of attention over the whole sequence), accumulators in registers.
     """
+    if fuse not in ("step", "all"):
+        raise ValueError(f"fuse must be 'step' or 'all', got {fuse!r}")
     B, S, H, D = q.shape
     P = int(ring_size)
     lse = softmax_lse if softmax_lse.is_contiguous() else softmax_lse.contiguous()
@@ -129,7 +138,7 @@ def ring_flash_attn_backward(dout, q, k, v, out, softmax_lse, softmax_scale=None
     dq = torch.zeros((B, S, H, D), dtype=torch.float32, device=q.device)
     dk = torch.zeros((B, k.shape[1], H, D), dtype=torch.float32, device=q.device)
     dv = torch.zeros((B, k.shape[1], H, D), dtype=torch.float32, device=q.device)
-    if P == 1:
+    if P == 1 or fuse == "all":
         ops.flash_bwd(q, k, v, dout, lse, delta, dq, dk, dv, softmax_scale, causal, layout="bshd")
     else:
         s = S // P

@@ -348,6 +348,23 @@ def test_backward_matches_autograd_of_full_attention(B, S, H, D, causal, P, dtyp
         check_grad(got, w, dtype, "d" + name)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_ring_backward_schedules_agree(causal):
+    """One launch per visited block pair (the reference's schedule, intel_ring_flash_attn.py:192-271)
+    and the single pass over the same pairs give the same gradients, both equal to the oracle's."""
+    B, S, H, D, P = 1, 384, 2, 128, 3
+    q, k, v, dout = rand_qkv((B, S, H, D), 105, torch.bfloat16, n=4)
+    want = O.attn_backward_autograd(q, k, v, dout, None, causal)
+    qd, kd, vd, dd = (t.to(DEV) for t in (q, k, v, dout))
+    out, lse = spa.ring.ring_flash_attn_forward(qd, kd, vd, None, causal, P)
+    res = {f: spa.ring.ring_flash_attn_backward(dd, qd, kd, vd, out, lse, None, causal, P, fuse=f) for f in ("step", "all")}
+    for f, grads in res.items():
+        for got, w, name in zip(grads, want, "qkv"):
+            check_grad(got, w, torch.bfloat16, f"{f} d{name}")
+    with pytest.raises(ValueError):
+        spa.ring.ring_flash_attn_backward(dd, qd, kd, vd, out, lse, None, causal, P, fuse="rank")
+
+
 def test_backward_packed_and_operator_entry():
     B, S, H, D = 1, 256, 2, 128
     qkv = rand((B, S, 3, H, D), 101, torch.bfloat16)
