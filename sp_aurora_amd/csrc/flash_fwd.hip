@@ -43,16 +43,24 @@ constexpr int FWD_BN = 64;   // keys per LDS sub-tile
 constexpr int FWD_THREADS = 256;  // threads of one wave group (4 waves x 32 query rows)
 constexpr int FWD_LOOK = 8;       // MFMA operands are fetched from LDS this many MFMAs ahead
 
-template <int D, int NG>
+// SHARE = false: the NG wave groups work on the same 128 query rows and take alternate sub-tiles,
+// each through LDS buffers of its own.  SHARE = true (NG = 2): the groups work on different query
+// rows (256 per workgroup), every group takes every sub-tile, and all 8 waves fill one set of
+// buffers together: half the global -> LDS traffic per FLOP and half as many workgroups.
+template <int D, int NG, bool SHARE>
 struct Fwd16Cfg {
   static constexpr int ROWB = D * 2;           // bytes per K / V row in LDS: no padding, the tiles are swizzled
   static constexpr int TILEB = FWD_BN * ROWB;  // one K or V sub-tile
-  static constexpr int GROUP = 4 * TILEB;      // one group's K[2] and V[2] buffers
-  static constexpr int EPI = (NG * FWD_BM * (D + 4) + NG * FWD_BM * 2 + FWD_BM) * 4;  // epilogue staging
-  static constexpr int SMEM = NG * GROUP > EPI ? NG * GROUP : EPI;
+  static constexpr int GROUP = 4 * TILEB;      // one set of K[2] and V[2] buffers
+  static constexpr int BMW = SHARE ? NG * FWD_BM : FWD_BM;  // query rows per workgroup
+  static constexpr int EPI = (NG * FWD_BM * (D + 4) + NG * FWD_BM * 2 + BMW) * 4;  // epilogue staging
+  static constexpr int TILES = SHARE ? GROUP : NG * GROUP;
+  static constexpr int SMEM = TILES > EPI ? TILES : EPI;
   static constexpr int CPR = D / 8;                         // 16-byte chunks per row
-  static constexpr int NDMA = TILEB / (FWD_THREADS * 16);   // direct loads per thread and sub-tile
-  static constexpr int RPD = FWD_THREADS / CPR;             // rows one round of the group's loads covers
+  static constexpr int DTHREADS = SHARE ? NG * FWD_THREADS : FWD_THREADS;  // threads filling one buffer
+  static constexpr int NDMA = TILEB / (DTHREADS * 16);      // direct loads per thread and sub-tile
+  static constexpr int RPD = DTHREADS / CPR;                // rows one round of loads covers
+  static_assert(!SHARE || (NG == 2 && NDMA >= 1), "shared buffers: two groups, at least one load per thread");
 };
 
 // A sub-tile lives in LDS as its rows back to back, each row's 16-byte chunks permuted by an XOR
@@ -69,9 +77,9 @@ __device__ __forceinline__ int v_swizzle(int row) {
   return D == 128 ? (row & 3) << 2 : D == 64 ? ((row >> 1) & 1) << 2 : 0;
 }
 
-template <typename T, int D, int NG>
+template <typename T, int D, int NG, bool SHARE>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams p) {
-  typedef Fwd16Cfg<D, NG> C;
+  typedef Fwd16Cfg<D, NG, SHARE> C;
   typedef Mma16<T> M;
   typedef typename M::frag frag;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -81,7 +89,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int w = wave & 3;     // which 32 query rows
   const int grp = wave >> 2;  // which key sub-tiles
-  const int tg = tid & (FWD_THREADS - 1);  // thread index inside the group
+  const int tg = SHARE ? tid : tid & (FWD_THREADS - 1);  // thread index among those filling one buffer
   const int ln = lane & 31;
   const int hh = lane >> 5;
 
@@ -95,8 +103,8 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   bid /= p.nqt;
   const int b = bid % p.B;
   const int rank = p.rank0 + p.nranks - 1 - bid / p.B;
-  const int q0 = qt * FWD_BM;
-  const int qw0 = q0 + w * 32;
+  const int q0 = qt * C::BMW;
+  const int qw0 = q0 + (SHARE ? grp * FWD_BM : 0) + w * 32;
   const int64_t qoff = (int64_t)rank * p.Sq;  // first row of this rank's query chunk
 
   const T* qp = (const T*)p.q + b * p.qs.b + h * p.qs.h + qoff * p.qs.s;
@@ -117,11 +125,12 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // [t_begin, t_end) of that schedule; a plain block call is P = 1, one step.
   // A group's work is a sequence of 64-key sub-tiles: first those of the masked (diagonal)
   // chunk up to the last key any row of the workgroup sees, then every full chunk.
-  constexpr int TILE = FWD_BN * NG;
+  constexpr int TILE = SHARE ? FWD_BN : FWD_BN * NG;  // keys between two sub-tiles of one group
+  constexpr int KSTEP = SHARE ? 1 : NG;
   const int nsteps = p.causal ? (rank + 1 < p.P ? rank + 1 : p.P) : p.P;
   const int t_end = p.t_count < 0 || p.t_begin + p.t_count > nsteps ? nsteps : p.t_begin + p.t_count;
   const bool diag = p.causal && p.t_begin == 0;
-  const int kv_end = q0 + FWD_BM < p.Sk ? q0 + FWD_BM : p.Sk;  // keys of the diagonal chunk in use
+  const int kv_end = q0 + C::BMW < p.Sk ? q0 + C::BMW : p.Sk;  // keys of the diagonal chunk in use
   const int n_diag = diag ? (kv_end + TILE - 1) / TILE : 0;
   const int npc = (p.Sk + TILE - 1) / TILE;                    // sub-tiles per full chunk
   const int t_full0 = p.t_begin + (diag ? 1 : 0);              // first unmasked step
@@ -149,7 +158,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     }
     int ch = (rank - t) % p.P;
     ch = ch < 0 ? ch + p.P : ch;
-    r.krel = (j * NG + grp) * FWD_BN;
+    r.krel = (j * KSTEP + (SHARE ? 0 : grp)) * FWD_BN;
     r.krow = ch * p.Sk + r.krel;
     r.kend = ch * p.Sk + p.Sk;
     return r;
@@ -189,7 +198,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     ch = ch < 0 ? ch + p.P : ch;
     ch = ch < 0 ? 0 : ch;  // only past the end of the schedule, where nothing is used
     c.sb.masked = c.i < n_diag;
-    c.sb.krel = (c.j * NG + grp) * FWD_BN;
+    c.sb.krel = (c.j * KSTEP + (SHARE ? 0 : grp)) * FWD_BN;
     c.sb.krow = ch * p.Sk + c.sb.krel;
     c.sb.kend = ch * p.Sk + p.Sk;
   };
@@ -223,8 +232,8 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const u32x4 krsrc = descriptor(kp, p.ks.s);
   const u32x4 vrsrc = descriptor(vp, p.vs.s);
   // LDS byte addresses of this group's buffers and of this wave's 1 KB share of a round
-  const unsigned lds_group = (unsigned)(uintptr_t)(lds_u8*)smem + grp * C::GROUP;
-  const unsigned lds_wave = lds_group + w * 1024;
+  const unsigned lds_group = (unsigned)(uintptr_t)(lds_u8*)smem + (SHARE ? 0 : grp * C::GROUP);
+  const unsigned lds_wave = lds_group + (SHARE ? wave : w) * 1024;
   auto k_lds = [&](int i) { return (unsigned)((i & 1) * C::TILEB); };                  // relative to lds_group
   auto v_lds = [&](int i) { return (unsigned)(2 * C::TILEB + (i & 1) * C::TILEB); };
   // load number q of the pair (K sub-tile with first row k_row into buffer kb, V sub-tile v_row into vb)
@@ -232,11 +241,11 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   auto load_one = [&](int q, bool kon, int k_row, unsigned kb, bool von, int v_row, unsigned vb) {
     if (q < C::NDMA) {
       const unsigned u = kon ? (unsigned)(k_row + q * C::RPD) * krow_b : OFF_NONE;
-      load_to_lds_b128(krsrc, kdoff + u, lds_wave + kb + q * (FWD_THREADS * 16));
+      load_to_lds_b128(krsrc, kdoff + u, lds_wave + kb + q * (C::DTHREADS * 16));
     } else {
       const int r = q - C::NDMA;
       const unsigned u = von ? (unsigned)(v_row + r * C::RPD) * vrow_b : OFF_NONE;
-      load_to_lds_b128(vrsrc, vdoff + u, lds_wave + vb + r * (FWD_THREADS * 16));
+      load_to_lds_b128(vrsrc, vdoff + u, lds_wave + vb + r * (C::DTHREADS * 16));
     }
   };
   auto load_k = [&](int i) {
@@ -432,25 +441,35 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // diagonal chunk) simply gets P = 0 from the mask.
   // MFMA phase i reads V(i) and K(i+1); the other two buffers are free then and receive V(i+1)
   // and K(i+2), which must have landed when the next VALU phase ends.
+  // With shared buffers both groups load their share of the same two sub-tiles in the same
+  // phase of the workgroup: group 0 during its MFMA phase, group 1 (one phase behind) at the start
+  // of its VALU phase; each waits for its loads before the barrier two phases later.
+  constexpr bool LOAD_IN_VALU_PHASE_G1 = SHARE;
+  const bool early = LOAD_IN_VALU_PHASE_G1 && grp == 1;  // wave-uniform
   Cursor cs = cursor_at(0), cv = cursor_at(1), ck = cursor_at(2);
   for (int i = 0; i + 1 < n; ++i) {
     frag pf[2][2];
-    softmax_phase(cs.sb, pf);
-    loads_landed();
-    __syncthreads();
     const bool kon = ck.i < n, von = cv.i < n;
     const unsigned kb = k_lds(i), vb = v_lds(i + 1);
+    if (early) {
+#pragma unroll
+      for (int q = 0; q < NLOADS; ++q) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb);
+    }
+    softmax_phase(cs.sb, pf);
+    if (!early) loads_landed();
+    __syncthreads();
     __builtin_amdgcn_s_setprio(1);
     mfma_phase(std::true_type{}, std::true_type{}, i, pf, [&](int j) {
       constexpr int TOTAL = (D / 32) * 4 + (D / 16) * 2;
 #pragma unroll
       for (int q = 0; q < NLOADS; ++q)
-        if ((q * TOTAL + TOTAL / 2) / NLOADS == j) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb);
+        if ((q * TOTAL + TOTAL / 2) / NLOADS == j && !early) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb);
     });
     __builtin_amdgcn_s_setprio(0);
     cursor_next(cs);
     cursor_next(cv);
     cursor_next(ck);
+    if (early) loads_landed();
     __syncthreads();
   }
   {  // last sub-tile: nothing to prepare behind it
@@ -471,12 +490,12 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // A ring step's merge with the running (acc, lse) happens in the same pass (p.epi).
   constexpr int TP = D + 4;  // floats per staged row
   float* const tile = (float*)smem + grp * (FWD_BM * TP);
-  float* const ml = (float*)smem + NG * FWD_BM * TP;  // [NG][128](m, l), then lse_b[128]
+  float* const ml = (float*)smem + NG * FWD_BM * TP;  // [NG][128](m, l), then lse_b[rows of the workgroup]
   float* const lsb = ml + NG * FWD_BM * 2;
   const int rloc = w * 32 + ln;
   const float l_own = l_run + xhalf(l_run);
   float scale, lse_b;
-  if (NG > 1) {
+  if (NG > 1 && !SHARE) {
     if (hh == 0) {
       ml[(grp * FWD_BM + rloc) * 2] = m_run;
       ml[(grp * FWD_BM + rloc) * 2 + 1] = l_own;
@@ -505,13 +524,13 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       st[3] = o[db][4 * g + 3] * scale;
       *(f32x4*)(tile + rloc * TP + db * 32 + 8 * g + 4 * hh) = st;
     }
-  if (grp == 0 && hh == 0) lsb[rloc] = lse_b;
+  if ((SHARE || grp == 0) && hh == 0) lsb[(SHARE ? grp * FWD_BM : 0) + rloc] = lse_b;
   __syncthreads();
   {
     constexpr int CH = D / 8;  // 8-element chunks per row; the CH lanes of a row share a wave
     const float* t0 = (const float*)smem;
     const int epi = p.epi;
-    for (int cidx = tid; cidx < FWD_BM * CH; cidx += FWD_THREADS * NG) {
+    for (int cidx = tid; cidx < C::BMW * CH; cidx += FWD_THREADS * NG) {
       const int row = cidx / CH, ch = cidx % CH;
       const int grow = q0 + row;
       if (grow >= p.Sq) continue;
@@ -522,7 +541,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         x[0] = a[0]; x[1] = a[1]; x[2] = a[2]; x[3] = a[3];
         x[4] = bq[0]; x[5] = bq[1]; x[6] = bq[2]; x[7] = bq[3];
       }
-      if (NG > 1) {
+      if (NG > 1 && !SHARE) {
         const float* t1 = t0 + FWD_BM * TP;
         const f32x4 a = *(const f32x4*)(t1 + row * TP + ch * 8);
         const f32x4 bq = *(const f32x4*)(t1 + row * TP + ch * 8 + 4);
@@ -770,16 +789,35 @@ hipError_t launch(K kernel, int threads, int smem, const FwdParams& p, hipStream
   return hipGetLastError();
 }
 
-// Two wave groups once there are at least two 64-key sub-tiles to split.
+// Two wave groups once there are at least two 64-key sub-tiles to split; 256-row workgroups with
+// shared K/V buffers once that still leaves every CU at least two workgroups.
 template <typename T, int D>
-hipError_t launch16(const FwdParams& p, hipStream_t stream) {
+hipError_t launch16(FwdParams p, hipStream_t stream) {
   static const int force = []() {
     const char* e = getenv("SPA_FWD_GROUPS");
     return e ? atoi(e) : 0;
   }();
+  static const int force_share = []() {
+    const char* e = getenv("SPA_FWD_SHARE");
+    return e ? atoi(e) : -1;
+  }();
+  static const int cus = []() {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    return n;
+  }();
   const bool two = force ? force == 2 : p.Sk > FWD_BN;
-  if (two) return launch(flash_fwd16_kernel<T, D, 2>, 2 * FWD_THREADS, Fwd16Cfg<D, 2>::SMEM, p, stream);
-  return launch(flash_fwd16_kernel<T, D, 1>, FWD_THREADS, Fwd16Cfg<D, 1>::SMEM, p, stream);
+  if (two && D >= 64) {
+    const int nqt2 = (p.Sq + 2 * FWD_BM - 1) / (2 * FWD_BM);
+    const int64_t wgs = (int64_t)p.B * p.H * nqt2 * p.nranks;
+    const bool share = force_share >= 0 ? force_share != 0 : wgs >= 2 * (int64_t)cus;
+    if (share) {
+      p.nqt = nqt2;
+      return launch(flash_fwd16_kernel<T, D, 2, (D >= 64)>, 2 * FWD_THREADS, Fwd16Cfg<D, 2, (D >= 64)>::SMEM, p, stream);
+    }
+  }
+  if (two) return launch(flash_fwd16_kernel<T, D, 2, false>, 2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+  return launch(flash_fwd16_kernel<T, D, 1, false>, FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
 }
 
 }  // namespace
