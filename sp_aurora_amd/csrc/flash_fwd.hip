@@ -288,21 +288,25 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   float l_run = 0.f;        // this lane's share of the running row sum
   const float c = p.scale_log2;
 
+  // per-lane LDS addresses of the operands of MFMA phase i: V(i) and K(i+1); computed before the
+  // barrier that opens the phase
+  auto operand_addresses = [&](int i, unsigned (&va)[D / 32], unsigned (&ka)[D / 16]) {
+    const unsigned vb = v_lds(i), kb = k_lds(i + 1);
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db) va[db] = vra[db] + vb;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) ka[ks] = kra[ks] + kb;
+  };
+
   // MFMA phase of step i: O += V(i)^T P(i) (if PV) followed by S(i+1) = K(i+1) Q^T (if NS).
   // The LDS operand of MFMA number j is fetched LOOK MFMAs ahead of its use, so the whole
   // phase runs off a rolling window of LOOK fragments instead of stalling on every read.
-  auto mfma_phase = [&](auto do_pv, auto do_s, int i, frag (&pfr)[2][2], auto&& side) {
+  auto mfma_phase = [&](auto do_pv, auto do_s, const unsigned (&va)[D / 32], const unsigned (&ka)[D / 16], frag (&pfr)[2][2], auto&& side) {
     constexpr bool PV = decltype(do_pv)::value, NS = decltype(do_s)::value;
     constexpr int NPV = PV ? (D / 32) * 4 : 0;
     constexpr int NSS = NS ? (D / 16) * 2 : 0;
     constexpr int TOTAL = NPV + NSS;
     constexpr int LOOK = FWD_LOOK;
-    const unsigned vb = v_lds(i), kb = k_lds(i + 1);
-    unsigned va[D / 32], ka[D / 16];
-#pragma unroll
-    for (int db = 0; db < (PV ? D / 32 : 0); ++db) va[db] = vra[db] + vb;
-#pragma unroll
-    for (int ks = 0; ks < (NS ? D / 16 : 0); ++ks) ka[ks] = kra[ks] + kb;
     auto fetch = [&](int j) -> frag {
       if (j < NPV) {  // j = (t*2+u)*(D/32) + db : consecutive MFMAs hit different accumulators
         const int db = j % (D / 32), tu = j / (D / 32);
@@ -431,7 +435,9 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   __syncthreads();
   {
     frag none[2][2];
-    mfma_phase(std::false_type{}, std::true_type{}, -1, none, [](int) {});  // S(0)
+    unsigned va[D / 32], ka[D / 16];
+    operand_addresses(-1, va, ka);
+    mfma_phase(std::false_type{}, std::true_type{}, va, ka, none, [](int) {});  // S(0)
   }
   __syncthreads();
   if (NG > 1 && grp == 1) __syncthreads();  // group 1 runs one phase behind group 0
@@ -456,10 +462,12 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       for (int q = 0; q < NLOADS; ++q) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb);
     }
     softmax_phase(cs.sb, pf);
+    unsigned va[D / 32], ka[D / 16];
+    operand_addresses(i, va, ka);
     if (!early) loads_landed();
     __syncthreads();
     __builtin_amdgcn_s_setprio(1);
-    mfma_phase(std::true_type{}, std::true_type{}, i, pf, [&](int j) {
+    mfma_phase(std::true_type{}, std::true_type{}, va, ka, pf, [&](int j) {
       constexpr int TOTAL = (D / 32) * 4 + (D / 16) * 2;
 #pragma unroll
       for (int q = 0; q < NLOADS; ++q)
@@ -475,9 +483,11 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   {  // last sub-tile: nothing to prepare behind it
     frag pf[2][2];
     softmax_phase(cs.sb, pf);
+    unsigned va[D / 32], ka[D / 16];
+    operand_addresses(n - 1, va, ka);
     loads_landed();
     __syncthreads();
-    mfma_phase(std::true_type{}, std::false_type{}, n - 1, pf, [](int) {});
+    mfma_phase(std::true_type{}, std::false_type{}, va, ka, pf, [](int) {});
     __syncthreads();
   }
   if (NG > 1 && grp == 0) __syncthreads();  // matches group 1's leading barrier
@@ -793,14 +803,11 @@ hipError_t launch(K kernel, int threads, int smem, const FwdParams& p, hipStream
 // shared K/V buffers once that still leaves every CU at least two workgroups.
 template <typename T, int D>
 hipError_t launch16(FwdParams p, hipStream_t stream) {
-  static const int force = []() {
-    const char* e = getenv("SPA_FWD_GROUPS");
-    return e ? atoi(e) : 0;
-  }();
-  static const int force_share = []() {
-    const char* e = getenv("SPA_FWD_SHARE");
-    return e ? atoi(e) : -1;
-  }();
+  // overrides for experiments and tests, read at every launch: SPA_FWD_GROUPS=1|2, SPA_FWD_SHARE=0|1
+  const char* eg = getenv("SPA_FWD_GROUPS");
+  const char* es = getenv("SPA_FWD_SHARE");
+  const int force = eg ? atoi(eg) : 0;
+  const int force_share = es ? atoi(es) : -1;
   static const int cus = []() {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;

@@ -433,3 +433,36 @@ def test_ring_driver_modes_on_awkward_shapes(P, B, s, H, D, causal, fuse):
     out, lse = ops.ring_fwd(q.to(DEV), k.to(DEV), v.to(DEV), P, None, causal, fuse=fuse)
     check_out(out, want_out, torch.bfloat16)
     check_lse(lse, want_lse)
+
+
+@pytest.fixture
+def shared_buffer_variant(monkeypatch):
+    """Forces the 256-row forward variant whose wave groups share the K/V buffers (it is otherwise
+    chosen only for grids that fill the GPU twice over)."""
+    monkeypatch.setenv("SPA_FWD_SHARE", "1")
+    yield
+    monkeypatch.delenv("SPA_FWD_SHARE", raising=False)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,Sq,Sk,D,causal", [(1, 2, 256, 256, 128, True), (2, 3, 300, 300, 64, True), (1, 2, 130, 515, 128, False),
+                                                (1, 1, 77, 200, 64, True), (1, 2, 512, 129, 128, True), (1, 1, 1, 65, 128, False)])
+def test_shared_buffer_variant_block_forward(shared_buffer_variant, B, H, Sq, Sk, D, causal, dtype):
+    q = rand((B, H, Sq, D), 120, dtype)
+    k = rand((B, H, Sk, D), 121, dtype)
+    v = rand((B, H, Sk, D), 122, dtype)
+    want_out, want_lse = O.attn_block(q, k, v, None, causal)
+    out, lse = ops.flash_fwd(q.to(DEV), k.to(DEV), v.to(DEV), None, causal, layout="bhsd")
+    check_out(out, want_out, dtype)
+    check_lse(lse, want_lse)
+
+
+@pytest.mark.parametrize("fuse", ["step", "rank", "all"])
+@pytest.mark.parametrize("P,B,s,H,D,causal", [(3, 2, 200, 2, 64, True), (2, 1, 1024, 2, 128, True), (5, 1, 64, 1, 128, True),
+                                              (4, 1, 320, 2, 128, False)])
+def test_shared_buffer_variant_ring(shared_buffer_variant, P, B, s, H, D, causal, fuse):
+    q, k, v = rand_qkv((B, P * s, H, D), 123, torch.bfloat16)
+    want_out, want_lse = O.full_attention(q, k, v, None, causal)
+    out, lse = ops.ring_fwd(q.to(DEV), k.to(DEV), v.to(DEV), P, None, causal, fuse=fuse)
+    check_out(out, want_out, torch.bfloat16)
+    check_lse(lse, want_lse)
