@@ -466,7 +466,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     operand_addresses(i, va, ka);
     if (!early) loads_landed();
     __syncthreads();
-    __builtin_amdgcn_s_setprio(1);
+    __builtin_amdgcn_s_setprio(3);
     mfma_phase(std::true_type{}, std::true_type{}, va, ka, pf, [&](int j) {
       constexpr int TOTAL = (D / 32) * 4 + (D / 16) * 2;
 #pragma unroll
