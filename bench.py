@@ -226,6 +226,7 @@ def side_workload(torch, name, steps, warmup):
     for _ in range(warmup):
         fn()
     ms = time_region(torch, fn, steps)
+    cpu = side_cpu_baseline(torch, name)
     if bound == "hbm":
         achieved = units * unit_bytes / (ms * 1e-3) / 1e9
         peak, unit = HBM_PEAK_GBPS, "GB/s"
@@ -238,7 +239,47 @@ def side_workload(torch, name, steps, warmup):
         "data": "synthetic", "config": work,
         "roofline": {"bound": bound, "kernel": kernel, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
                      "frac": round(achieved / peak, 4), "traffic": None},
+        "cpu_baseline": cpu,
     }))
+
+
+def side_cpu_baseline(torch, name, budget_s=10.0):
+    """The reference's op sequence for the row on the host cores (oracle restatements, fp32 torch)."""
+    from oracle import attn_oracle as O
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(3)
+    if name == "relayout":
+        # the reference's reshape / transpose / contiguous chain around all_to_all_single
+        # (sp_aurora/intel_ulysses_attn.py:95-138) on the full config-4 tensor, both directions
+        x = torch.randn((8, 1, 2048, 32, 128), generator=g).to(torch.bfloat16)
+        xs = list(x)
+        fn = lambda: O.all_to_all_4d_h2s(O.all_to_all_4d_s2h(xs))
+        work, unit = 2 * 2 * x.numel() * 2 / 1e9, "GB/s"
+        sample = "config 4 tensor [8,1,2048,32,128] bf16, s2h then h2s, literal reshape/transpose/contiguous chains"
+    elif name == "merge":
+        acc = torch.randn((1, 32, 1024, 128), generator=g)
+        lse = torch.randn((1, 32, 1024, 1), generator=g)
+        blk = torch.randn((1, 32, 1024, 128), generator=g).to(torch.bfloat16)
+        bl = torch.randn((1, 32, 1024, 1), generator=g)
+        fn = lambda: O.merge(acc, lse, blk.float(), bl)
+        work, unit = (acc.numel() * 10 + lse.numel() * 12) / 1e9, "GB/s"
+        sample = "one config-3 chunk [1,32,1024,128]: sigmoid / logsigmoid merge of a bf16 block into fp32 (out, lse)"
+    else:
+        # one diagonal + one full block pair of config 5 through autograd of the closed form
+        q, k, v, do = (torch.randn((1, 2048, 16, 128), generator=g).to(torch.bfloat16) for _ in range(4))
+        fn = lambda: (O.attn_backward_autograd(q, k, v, do, None, True, compute_dtype=torch.float32),
+                      O.attn_backward_autograd(q, k, v, do, None, False, compute_dtype=torch.float32))
+        work, unit = 2.5 * 1.5 * 4.0 * 16 * 2048 * 2048 * 128 / 1e12, "TFLOP/s"
+        sample = "1 diagonal + 1 full block pair of config 5 ([1,16,2048,128] bf16 up-cast to fp32), torch CPU autograd of softmax(QK^T)V"
+    fn()  # warm-up
+    t0 = time.perf_counter()
+    n = 0
+    while time.perf_counter() - t0 < budget_s and n < 2000:
+        fn()
+        n += 1
+    dt = time.perf_counter() - t0
+    return {"value": work * n / dt, "unit": unit, "cores": cores, "kind": "port", "sample": f"{n} x ({sample}), {dt:.1f} s"}
 
 
 def main():

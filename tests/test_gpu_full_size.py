@@ -6,6 +6,8 @@ path runs at the full size and is checked
     (softmax(q k^T scale + mask) v, logsumexp) for a sample of (batch, head) slices, to the
     tolerances of BASELINE's north_star (bf16 out atol 2e-2 / rtol 1.6e-2, lse atol 1e-3,
     gradients 3e-2 of the gradient's scale), and
+  * against the float64 CPU oracle on a few dozen random query rows per config (which pins the
+    on-device fp32 evaluation itself), and
   * through size-independent properties: the three ring schedules and the step-by-step path
     agree, ring == one block call over the same keys, re-layout is a bit-exact permutation whose
     inverse restores the input, a value projection of all ones returns ones, lse of a ring equals
@@ -42,6 +44,23 @@ def ref_head(q, k, v, scale, causal, q_offset=0):
     return p @ v.float(), lse
 
 
+def spot_check_rows(out_h, lse_h, q_h, k_h, v_h, scale, causal, what, n_rows=24, seed=0, q_offset=0):
+    """Float64 CPU oracle on random query rows of one head: q_h [Sq,D], k_h, v_h [Sk,D],
+    out_h [Sq,D], lse_h [Sq]; query i sits at absolute position q_offset + i."""
+    from oracle import attn_oracle as O
+    g = torch.Generator().manual_seed(seed)
+    rows = torch.randperm(q_h.shape[0], generator=g)[:n_rows].tolist() + [0, q_h.shape[0] - 1]
+    kc, vc = k_h.cpu(), v_h.cpu()
+    for r in rows:
+        n_keys = min(q_offset + r + 1, kc.shape[0]) if causal else kc.shape[0]
+        # one query against the keys it sees: a non-causal block of the oracle, [B=1,H=1,1,D] x [1,1,n_keys,D]
+        want_o, want_l = O.attn_block(q_h[r].cpu()[None, None, None], kc[None, None, :n_keys], vc[None, None, :n_keys], scale, False)
+        got_o, got_l = out_h[r].cpu().double(), lse_h[r].cpu().double()
+        bad = (got_o - want_o[0, 0, 0]).abs() > OUT_ATOL + OUT_RTOL * want_o[0, 0, 0].abs()
+        assert not bad.any(), f"{what} row {r}: out max abs err {(got_o - want_o[0, 0, 0]).abs().max().item():.3e}"
+        assert abs(got_l.item() - want_l[0, 0, 0].item()) <= LSE_ATOL, f"{what} row {r}: lse err {abs(got_l.item() - want_l[0, 0, 0].item()):.3e}"
+
+
 def assert_out(got, want, what):
     got, want = got.float(), want.float()
     bad = (got - want).abs() > OUT_ATOL + OUT_RTOL * want.abs()
@@ -67,6 +86,8 @@ def test_config2_ring_rank2_of_4():
         want_o, want_l = ref_head(q_local[b, :, h], k[b, :(rank + 1) * s, h], v[b, :(rank + 1) * s, h], scale, True, rank * s)
         assert_out(out_a[b, :, h], want_o, f"stepwise b{b} h{h}")
         assert_lse(lse_a[b, h], want_l, f"stepwise b{b} h{h}")
+    spot_check_rows(out_a[1, :, 5], lse_a[1, 5], q_local[1, :, 5], k[1, :(rank + 1) * s, 5], v[1, :(rank + 1) * s, 5], scale, True,
+                    "cfg2 fp64", q_offset=rank * s)
     # the C driver in its three schedules writes rank 2's rows of the full tensors
     for fuse in ("step", "rank", "all"):
         out = torch.zeros_like(q)
@@ -94,6 +115,7 @@ def test_config3_ring_sweep_all_ranks():
         for f, (o, l) in res.items():
             assert_out(o[0, :, h], want_o, f"{f} h{h}")
             assert_lse(l[0, h], want_l, f"{f} h{h}")
+    spot_check_rows(res["all"][0][0, :, 7], res["all"][1][0, 7], q[0, :, 7], k[0, :, 7], v[0, :, 7], scale, True, "cfg3 fp64")
     # ring == the block operator on the undivided sequence (P = 1)
     o1, l1 = spa.ring.ring_flash_attn_forward(q, k, v, scale, True, 1)
     for f, (o, l) in res.items():
@@ -136,6 +158,7 @@ def test_config4_ulysses_relayout_and_attention():
         want_o, want_l = ref_head(qf[0, :, hd], kf[0, :, hd], vf[0, :, hd], scale, True)
         assert_out(of[0, :, hd], want_o, f"ulysses h{hd}")
         assert_lse(lse[hd // h, 0, hd % h], want_l, f"ulysses h{hd}")
+    spot_check_rows(of[0, :, 9], lse[9 // h, 0, 9 % h], qf[0, :, 9], kf[0, :, 9], vf[0, :, 9], scale, True, "cfg4 fp64", n_rows=12)
     assert torch.equal(spa.ulysses_flash_attn_func(q, k, v, causal=True), out)
 
 
@@ -155,6 +178,8 @@ def test_config5_qkvpacked_long_context_forward_backward():
         o1, l1 = ops.flash_fwd(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], scale, True)
         assert_out(out, o1, "ring vs P=1")
         assert_lse(lse, l1, "ring vs P=1")
+    with torch.no_grad():
+        spot_check_rows(out[0, :, 3], lse[0, 3], qkv[0, :, 0, 3], qkv[0, :, 1, 3], qkv[0, :, 2, 3], scale, True, "cfg5 fp64", n_rows=12)
     for h in (0, 15):
         qh, kh, vh = (qkv.detach()[0, :, i, h].float().requires_grad_(True) for i in range(3))
         want_o, want_l = ref_head(qh, kh, vh, scale, True)
