@@ -27,7 +27,7 @@ the host cores, on diagonal + full block pairs of the same workload.
 `--workload` selects the other measured rows of the path instead (one JSON line each, same keys,
 `metric` named after the row): `relayout` = the Ulysses re-layout of BASELINE config 4 (HBM
 bound), `merge` = update_out_and_lse on one config-3 chunk (HBM bound), `backward` = the ring
-backward of BASELINE config 5 (MFMA bound).
+backward of BASELINE config 5 (MFMA bound), `ulysses` = the whole Ulysses forward of config 4.
 
 Two helper modes for the HBM traffic figure (roofline.traffic):
   --traffic-leg          additionally runs a plain device copy of known size, so that a
@@ -193,6 +193,16 @@ def side_workload(torch, name, steps, warmup):
         units, unit_bytes = 2, 2 * x.numel() * 2   # two launches per step, each reads and writes the tensor once
         bound, kernel, metric = "hbm", "relayout_kernel<16>", "Ulysses re-layout GB/s, config 4 [8,1,2048,32,128] bf16, s2h + h2s"
         work = {"workload": "config 4 re-layout: [P=8,B=1,s=2048,H=32,D=128] bf16 -> [8,1,16384,4,128] and back", "bytes_per_launch": unit_bytes}
+    elif name == "ulysses":
+        Pn, Bn, sn, Hn, Dn = 8, 1, 2048, 32, 128
+        q, k, v = rnd((Pn, Bn, sn, Hn, Dn)), rnd((Pn, Bn, sn, Hn, Dn)), rnd((Pn, Bn, sn, Hn, Dn))
+        scale = Dn ** -0.5
+        fn = lambda: spa.intel_ulysses_flash_attn_forward(None, q, k, v, scale, causal=True)
+        unit_flops = 4.0 * Bn * Hn * (Pn * sn) ** 2 * Dn / 2
+        units = 1
+        bound, kernel, metric = "mfma", "relayout_kernel x4 + flash_fwd16_kernel<bf16,128,2>", "Ulysses forward TFLOP/s (causal-adjusted attention FLOPs over the whole step: 3 re-layouts in, attention, 1 out), config 4"
+        work = {"workload": "config 4: q,k,v [P=8,B=1,s=2048,H=32,D=128] bf16 -> head-sharded [8,1,16384,4,128], full causal attention "
+                            "per head group, inverse re-layout of out", "flops_per_step": unit_flops}
     elif name == "merge":
         Bn, sn, Hn, Dn = 1, 1024, 32, 128
         acc = torch.randn((Bn, sn, Hn, Dn), generator=g, dtype=torch.float32).to(dev)
@@ -226,7 +236,7 @@ def side_workload(torch, name, steps, warmup):
     for _ in range(warmup):
         fn()
     ms = time_region(torch, fn, steps)
-    cpu = side_cpu_baseline(torch, name)
+    cpu = side_cpu_baseline(torch, name) if name != "ulysses" else None
     if bound == "hbm":
         achieved = units * unit_bytes / (ms * 1e-3) / 1e9
         peak, unit = HBM_PEAK_GBPS, "GB/s"
@@ -292,7 +302,7 @@ def main():
     ap.add_argument("--only-all", action="store_true", help="skip the rank / step schedules (profiling runs)")
     ap.add_argument("--traffic-leg", action="store_true", help="also run the calibration copy (for --pmc runs)")
     ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"))
-    ap.add_argument("--workload", default="config3", choices=["config3", "relayout", "merge", "backward"])
+    ap.add_argument("--workload", default="config3", choices=["config3", "relayout", "merge", "backward", "ulysses"])
     args = ap.parse_args()
     if args.pmc_summary:
         pmc_summary(*args.pmc_summary)
@@ -310,8 +320,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.workload != "config3":
-        side_workload(torch, args.workload, args.steps if args.workload != "backward" else min(args.steps, 5),
-                      args.warmup if args.workload != "backward" else min(args.warmup, 2))
+        heavy = args.workload in ("backward", "ulysses")
+        side_workload(torch, args.workload, min(args.steps, 5) if heavy else args.steps, min(args.warmup, 2) if heavy else args.warmup)
         return
     q, k, v = make_inputs(torch, dev)
     scale = D ** -0.5

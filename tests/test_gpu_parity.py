@@ -466,3 +466,34 @@ def test_shared_buffer_variant_ring(shared_buffer_variant, P, B, s, H, D, causal
     out, lse = ops.ring_fwd(q.to(DEV), k.to(DEV), v.to(DEV), P, None, causal, fuse=fuse)
     check_out(out, want_out, torch.bfloat16)
     check_lse(lse, want_lse)
+
+
+@pytest.mark.parametrize("fuse", ["step", "all"])
+def test_ring_forward_replays_from_a_captured_graph(fuse):
+    """The library allocates nothing and never synchronises, so a ring forward can be captured in a
+    graph; every replay (with eager work and synchronisations in between) must equal the eager result."""
+    B, S, H, D, P = 1, 1024, 4, 128, 4
+    q, k, v = (t.to(DEV) for t in rand_qkv((B, S, H, D), 130, torch.bfloat16))
+    step = spa.ring.make_ring_forward_step(q, k, v, None, True, P, fuse=fuse)
+    eager_out, eager_lse = (t.clone() for t in step())
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()  # warm up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out, lse = step()
+    for rep in range(3):
+        out.fill_(7)
+        lse.fill_(7)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager_out) and torch.equal(lse, eager_lse), f"replay {rep} differs"
+        # eager work between replays, with new inputs of the same shape in the captured buffers
+        q.mul_(-1)
+        k.mul_(-1)
+        torch.cuda.synchronize()
+        q.mul_(-1)
+        k.mul_(-1)
