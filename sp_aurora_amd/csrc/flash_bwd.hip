@@ -567,6 +567,295 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// fp32 kernels: the same two-kernel scheme on v_mfma_f32_32x32x2_f32 (fp32 products and
+// accumulation, P and dS stay fp32).  Correctness path for fp32 inputs: tiles of 32 rows staged
+// through registers, no software pipeline.  The contraction index of the gradient products is the
+// row an accumulator register holds (8*(v/4) + 4*hh + v%4), so P and dS are used where they are.
+// ------------------------------------------------------------------------------------------
+constexpr int B32_ROWS = 32;
+
+template <int D>
+struct Bwd32Cfg {
+  static constexpr int PITCH = D + 4;              // floats per LDS row
+  static constexpr int TILE = B32_ROWS * PITCH;    // floats per tile
+  static constexpr int STAT = 2 * B32_ROWS;        // lse * log2 e and delta of a query tile
+  static constexpr int SMEM_DQ = 2 * 2 * TILE * 4;
+  static constexpr int SMEM_DKV = 2 * (2 * TILE + STAT) * 4;
+  static constexpr int CPR = D / 4;
+  static constexpr int RPP = BWD_THREADS / CPR;
+  static constexpr int PASS = (B32_ROWS + RPP - 1) / RPP;
+};
+
+// two row-major tiles of 32 rows (a, b) of tensors with the same row count, staged together
+template <int D>
+struct PairStage {
+  typedef Bwd32Cfg<D> C;
+  f32x4 ra[C::PASS], rb[C::PASS];
+  __device__ __forceinline__ void gload(const float* a, int64_t as, const float* b, int64_t bs, int row0, int nrows, int tid) {
+    const int cc = tid % C::CPR, cr = tid / C::CPR;
+#pragma unroll
+    for (int i = 0; i < C::PASS; ++i) {
+      const int lr = cr + i * C::RPP;
+      if (lr < B32_ROWS) {
+        int r = row0 + lr;
+        r = r < nrows ? r : nrows - 1;
+        ra[i] = *(const f32x4*)(a + (int64_t)r * as + cc * 4);
+        rb[i] = *(const f32x4*)(b + (int64_t)r * bs + cc * 4);
+      }
+    }
+  }
+  __device__ __forceinline__ void lstore(float* ta, float* tb, int tid) const {
+    const int cc = tid % C::CPR, cr = tid / C::CPR;
+#pragma unroll
+    for (int i = 0; i < C::PASS; ++i) {
+      const int lr = cr + i * C::RPP;
+      if (lr < B32_ROWS) {
+        *(f32x4*)(ta + lr * C::PITCH + cc * 4) = ra[i];
+        *(f32x4*)(tb + lr * C::PITCH + cc * 4) = rb[i];
+      }
+    }
+  }
+};
+
+template <int D>
+__global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dq_kernel(const BwdParams p) {
+  typedef Bwd32Cfg<D> C;
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* sm = (float*)smem;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, w = tid >> 6, ln = lane & 31, hh = lane >> 5;
+
+  int bid = blockIdx.x;
+  const int h = bid % p.H;
+  bid /= p.H;
+  const int qt = p.nqt - 1 - (bid % p.nqt);
+  const int b = bid / p.nqt;
+  const int q0 = qt * 128;
+  const int qw0 = q0 + w * 32;
+
+  const float* qp = (const float*)p.q + b * p.qs.b + h * p.qs.h;
+  const float* kp = (const float*)p.k + b * p.ks.b + h * p.ks.h;
+  const float* vp = (const float*)p.v + b * p.vs.b + h * p.vs.h;
+  const float* dop = (const float*)p.dout + b * p.dos.b + h * p.dos.h;
+
+  const int qrow = qw0 + ln;
+  const int qrow_c = qrow < p.Sq ? qrow : p.Sq - 1;
+  // contraction step of the first products: head dim 8*g + 4*hh + e
+  f32x4 qf[D / 8], dof[D / 8];
+#pragma unroll
+  for (int g = 0; g < D / 8; ++g) {
+    qf[g] = *(const f32x4*)(qp + (int64_t)qrow_c * p.qs.s + 8 * g + 4 * hh);
+    dof[g] = *(const f32x4*)(dop + (int64_t)qrow_c * p.dos.s + 8 * g + 4 * hh);
+  }
+  const int64_t li = ((int64_t)b * p.H + h) * p.Sq + qrow_c;
+  const float l2 = p.lse[li] * 1.4426950408889634f;
+  const float dl = p.delta[li];
+  const float c = p.scale_log2;
+  const int lim = p.causal ? (qrow < p.Sk - 1 ? qrow : p.Sk - 1) : p.Sk - 1;  // last visible key
+
+  const int kv_end = p.causal ? (q0 + 128 < p.Sk ? q0 + 128 : p.Sk) : p.Sk;
+  const int nt = (kv_end + B32_ROWS - 1) / B32_ROWS;
+
+  f32x16 dq[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i) zero16(dq[i]);
+
+  PairStage<D> st;
+  st.gload(kp, p.ks.s, vp, p.vs.s, 0, p.Sk, tid);
+  st.lstore(sm, sm + C::TILE, tid);
+  __syncthreads();
+
+  for (int it = 0; it < nt; ++it) {
+    const int cur = it & 1;
+    const int key0 = it * B32_ROWS;
+    const bool more = it + 1 < nt;
+    if (more) st.gload(kp, p.ks.s, vp, p.vs.s, key0 + B32_ROWS, p.Sk, tid);
+    if (!(p.causal && key0 > qw0 + 31)) {
+      const float* kb = sm + cur * 2 * C::TILE;
+      const float* vb = kb + C::TILE;
+      f32x16 s, dp;
+      zero16(s);
+      zero16(dp);
+#pragma unroll
+      for (int g = 0; g < D / 8; ++g) {
+        const f32x4 a = *(const f32x4*)(kb + ln * C::PITCH + 8 * g + 4 * hh);
+        const f32x4 a2 = *(const f32x4*)(vb + ln * C::PITCH + 8 * g + 4 * hh);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], qf[g][e], s, 0, 0, 0);
+          dp = __builtin_amdgcn_mfma_f32_32x32x2f32(a2[e], dof[g][e], dp, 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = key0 + 8 * (v >> 2) + 4 * hh + (v & 3);
+        const float pr = key > lim ? 0.f : fast_exp2(__builtin_fmaf(s[v], c, -l2));
+        s[v] = pr * (dp[v] - dl);
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int kl = 8 * (v >> 2) + 4 * hh + (v & 3);
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+          dq[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(kb[kl * C::PITCH + db * 32 + ln], s[v], dq[db], 0, 0, 0);
+      }
+    }
+    if (more) st.lstore(sm + (cur ^ 1) * 2 * C::TILE, sm + (cur ^ 1) * 2 * C::TILE + C::TILE, tid);
+    __syncthreads();
+  }
+
+  if (qrow < p.Sq) {
+    float* dqp = p.dq + b * p.dqs.b + h * p.dqs.h + (int64_t)qrow * p.dqs.s;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4* dst = (f32x4*)(dqp + db * 32 + 8 * g + 4 * hh);
+        f32x4 x = *dst;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] += dq[db][4 * g + e] * p.scale;
+        *dst = x;
+      }
+  }
+}
+
+template <int D>
+__global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dkdv_kernel(const BwdParams p) {
+  typedef Bwd32Cfg<D> C;
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* sm = (float*)smem;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, w = tid >> 6, ln = lane & 31, hh = lane >> 5;
+
+  int bid = blockIdx.x;
+  const int h = bid % p.H;
+  bid /= p.H;
+  const int kt = bid % p.nkt;
+  const int b = bid / p.nkt;
+  const int k0 = kt * 128;
+  const int kw0 = k0 + w * 32;
+
+  const float* qp = (const float*)p.q + b * p.qs.b + h * p.qs.h;
+  const float* kp = (const float*)p.k + b * p.ks.b + h * p.ks.h;
+  const float* vp = (const float*)p.v + b * p.vs.b + h * p.vs.h;
+  const float* dop = (const float*)p.dout + b * p.dos.b + h * p.dos.h;
+  const float* lsep = p.lse + ((int64_t)b * p.H + h) * p.Sq;
+  const float* delp = p.delta + ((int64_t)b * p.H + h) * p.Sq;
+
+  const int krow = kw0 + ln;
+  const int krow_c = krow < p.Sk ? krow : p.Sk - 1;
+  f32x4 kf[D / 8], vf[D / 8];
+#pragma unroll
+  for (int g = 0; g < D / 8; ++g) {
+    kf[g] = *(const f32x4*)(kp + (int64_t)krow_c * p.ks.s + 8 * g + 4 * hh);
+    vf[g] = *(const f32x4*)(vp + (int64_t)krow_c * p.vs.s + 8 * g + 4 * hh);
+  }
+  const float c = p.scale_log2;
+
+  const int it0 = p.causal ? k0 / B32_ROWS : 0;  // earlier query rows see none of these keys
+  const int nt = (p.Sq + B32_ROWS - 1) / B32_ROWS;
+  constexpr int STAGE = 2 * C::TILE + C::STAT;
+
+  f32x16 dk[D / 32], dv[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i) {
+    zero16(dk[i]);
+    zero16(dv[i]);
+  }
+
+  PairStage<D> st;
+  float st_l = 0.f, st_d = 0.f;
+  auto gload = [&](int it) {
+    st.gload(qp, p.qs.s, dop, p.dos.s, it * B32_ROWS, p.Sq, tid);
+    if (tid < B32_ROWS) {
+      int r = it * B32_ROWS + tid;
+      r = r < p.Sq ? r : p.Sq - 1;
+      st_l = lsep[r] * 1.4426950408889634f;
+      st_d = delp[r];
+    }
+  };
+  auto lstore = [&](int stage) {
+    float* sb = sm + stage * STAGE;
+    st.lstore(sb, sb + C::TILE, tid);
+    if (tid < B32_ROWS) {
+      sb[2 * C::TILE + tid] = st_l;
+      sb[2 * C::TILE + B32_ROWS + tid] = st_d;
+    }
+  };
+
+  if (it0 < nt) {
+    gload(it0);
+    lstore(it0 & 1);
+  }
+  __syncthreads();
+
+  for (int it = it0; it < nt; ++it) {
+    const int cur = it & 1;
+    const int r0 = it * B32_ROWS;
+    const bool more = it + 1 < nt;
+    if (more) gload(it + 1);
+    if (!(p.causal && r0 + B32_ROWS - 1 < kw0)) {
+      const float* qb = sm + cur * STAGE;
+      const float* dob = qb + C::TILE;
+      const float* stp = dob + C::TILE;
+      f32x16 s, dp;
+      zero16(s);
+      zero16(dp);
+#pragma unroll
+      for (int g = 0; g < D / 8; ++g) {
+        const f32x4 a = *(const f32x4*)(qb + ln * C::PITCH + 8 * g + 4 * hh);
+        const f32x4 a2 = *(const f32x4*)(dob + ln * C::PITCH + 8 * g + 4 * hh);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], kf[g][e], s, 0, 0, 0);
+          dp = __builtin_amdgcn_mfma_f32_32x32x2f32(a2[e], vf[g][e], dp, 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int ql = 8 * (v >> 2) + 4 * hh + (v & 3);
+        const int qi = r0 + ql;
+        const bool dead = qi >= p.Sq || (p.causal && krow > qi);
+        const float pr = dead ? 0.f : fast_exp2(__builtin_fmaf(s[v], c, -stp[ql]));
+        s[v] = pr;
+        dp[v] = pr * (dp[v] - stp[B32_ROWS + ql]);
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int ql = 8 * (v >> 2) + 4 * hh + (v & 3);
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db) {
+          dv[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(dob[ql * C::PITCH + db * 32 + ln], s[v], dv[db], 0, 0, 0);
+          dk[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(qb[ql * C::PITCH + db * 32 + ln], dp[v], dk[db], 0, 0, 0);
+        }
+      }
+    }
+    if (more) lstore(cur ^ 1);
+    __syncthreads();
+  }
+
+  if (krow < p.Sk) {
+    float* dkp = p.dk + b * p.dks.b + h * p.dks.h + (int64_t)krow * p.dks.s;
+    float* dvp = p.dv + b * p.dvs.b + h * p.dvs.h + (int64_t)krow * p.dvs.s;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4* d1 = (f32x4*)(dkp + db * 32 + 8 * g + 4 * hh);
+        f32x4* d2 = (f32x4*)(dvp + db * 32 + 8 * g + 4 * hh);
+        f32x4 x = *d1, y = *d2;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          x[e] += dk[db][4 * g + e] * p.scale;
+          y[e] += dv[db][4 * g + e];
+        }
+        *d1 = x;
+        *d2 = y;
+      }
+  }
+}
+
 template <typename K>
 hipError_t launch(K kernel, int smem, unsigned blocks, const BwdParams& p, hipStream_t stream) {
   hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -598,6 +887,17 @@ hipError_t spa_launch_flash_bwd(BwdParams p, int D, int dtype, hipStream_t strea
     if (D == 128) return launch_both<_Float16, 128>(p, stream);
     if (D == 64) return launch_both<_Float16, 64>(p, stream);
     if (D == 32) return launch_both<_Float16, 32>(p, stream);
+  } else if (dtype == 0) {
+    const unsigned qblocks = (unsigned)((int64_t)p.B * p.H * p.nqt);
+    const unsigned kblocks = (unsigned)((int64_t)p.B * p.H * p.nkt);
+    hipError_t e = hipErrorInvalidValue;
+    if (D == 128) e = launch(flash_bwd32_dq_kernel<128>, Bwd32Cfg<128>::SMEM_DQ, qblocks, p, stream);
+    if (D == 64) e = launch(flash_bwd32_dq_kernel<64>, Bwd32Cfg<64>::SMEM_DQ, qblocks, p, stream);
+    if (D == 32) e = launch(flash_bwd32_dq_kernel<32>, Bwd32Cfg<32>::SMEM_DQ, qblocks, p, stream);
+    if (e != hipSuccess) return e;
+    if (D == 128) return launch(flash_bwd32_dkdv_kernel<128>, Bwd32Cfg<128>::SMEM_DKV, kblocks, p, stream);
+    if (D == 64) return launch(flash_bwd32_dkdv_kernel<64>, Bwd32Cfg<64>::SMEM_DKV, kblocks, p, stream);
+    if (D == 32) return launch(flash_bwd32_dkdv_kernel<32>, Bwd32Cfg<32>::SMEM_DKV, kblocks, p, stream);
   }
   return hipErrorInvalidValue;
 }

@@ -321,6 +321,9 @@ int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout,
       !aligned16(dout, do_strides, esz) || !aligned16(dq_acc, dq_strides, 4) || !aligned16(dk_acc, dk_strides, 4) ||
       !aligned16(dv_acc, dv_strides, 4))
     return fail(SPA_EALIGN, "spa_flash_bwd: pointers and row strides must be 16-byte aligned");
+  if (!span_ok(Sq, q_strides[2], D, esz) || !span_ok(Sk, k_strides[2], D, esz) || !span_ok(Sk, v_strides[2], D, esz) ||
+      !span_ok(Sq, do_strides[2], D, esz))
+    return fail(SPA_EUNSUPPORTED, "spa_flash_bwd: a tensor of one (batch, head) spans more than 2 GiB");
   BwdParams p;
   p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta;
   p.dq = dq_acc; p.dk = dk_acc; p.dv = dv_acc;

@@ -63,7 +63,7 @@ def test_bad_arguments_return_codes_without_touching_a_device():
     assert lib.spa_relayout_s2h(p, ctypes.c_void_p(8192), 3, 1, 4, 8, 16, 1, 2, None) == -1
     assert lib.spa_relayout_s2h(p, p, 2, 1, 4, 8, 16, 1, 2, None) == -1
     assert lib.spa_relayout_h2s(p, ctypes.c_void_p(8192), 2, 1, 4, 8, 16, 4, 2, None) == -1
-    # backward: fp32 has no kernel
+    # backward: unknown dtype code
     f = ctypes.c_void_p(4096)
     args = [f] * 9 + [1, 1, 8, 8, 64] + [st] * 7
     assert lib.spa_flash_bwd(*args, 1.0, 0, 9, None) == -1
