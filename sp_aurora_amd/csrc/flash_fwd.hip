@@ -88,7 +88,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int w = wave & 3;     // which 32 query rows
-  const int grp = wave >> 2;  // which key sub-tiles
+  const int grp = wave >> 2;  // wave group: which key sub-tiles (or, with shared buffers, which 128 query rows)
   const int tg = SHARE ? tid : tid & (FWD_THREADS - 1);  // thread index among those filling one buffer
   const int ln = lane & 31;
   const int hh = lane >> 5;
@@ -220,17 +220,8 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const unsigned krow_b = (unsigned)(p.ks.s * (int64_t)sizeof(T));  // bytes per K row
   const unsigned vrow_b = (unsigned)(p.vs.s * (int64_t)sizeof(T));
   const int64_t rows_all = (int64_t)p.P * p.Sk;
-  auto descriptor = [&](const T* base, int64_t row_stride) {
-    const uint64_t a = (uint64_t)base;
-    u32x4 r;
-    r[0] = __builtin_amdgcn_readfirstlane((unsigned)a);
-    r[1] = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32) & 0xffffu);  // stride 0: raw buffer
-    r[2] = __builtin_amdgcn_readfirstlane((unsigned)(((rows_all - 1) * row_stride + D) * (int64_t)sizeof(T)));
-    r[3] = 0x00020000u;
-    return r;
-  };
-  const u32x4 krsrc = descriptor(kp, p.ks.s);
-  const u32x4 vrsrc = descriptor(vp, p.vs.s);
+  const u32x4 krsrc = buffer_descriptor(kp, (unsigned)(((rows_all - 1) * p.ks.s + D) * (int64_t)sizeof(T)));
+  const u32x4 vrsrc = buffer_descriptor(vp, (unsigned)(((rows_all - 1) * p.vs.s + D) * (int64_t)sizeof(T)));
   // LDS byte addresses of this group's buffers and of this wave's 1 KB share of a round
   const unsigned lds_group = (unsigned)(uintptr_t)(lds_u8*)smem + (SHARE ? 0 : grp * C::GROUP);
   const unsigned lds_wave = lds_group + (SHARE ? wave : w) * 1024;
