@@ -372,7 +372,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       mxd = fmaxf(fmaxf(mxd, s[1][v + 8]), s[1][v + 9]);
     }
     float mx = fmaxf(fmaxf(mxa, mxb), fmaxf(mxc, mxd));
-    mx = fmaxf(mx, xhalf(mx));
+    mx = halves_max(mx);
     // Lazy rescale: the reference max only moves when some row's max grew by more than
     // 2^8 in the exp2 domain; until then P <= 256, harmless in fp32 sums and bf16 operands.
     if (__builtin_amdgcn_ballot_w64((mx - m_run) * c > 8.f) != 0) {
@@ -494,7 +494,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   float* const ml = (float*)smem + NG * FWD_BM * TP;  // [NG][128](m, l), then lse_b[rows of the workgroup]
   float* const lsb = ml + NG * FWD_BM * 2;
   const int rloc = w * 32 + ln;
-  const float l_own = l_run + xhalf(l_run);
+  const float l_own = halves_sum(l_run);
   float scale, lse_b;
   if (NG > 1 && !SHARE) {
     if (hh == 0) {
@@ -724,7 +724,7 @@ __global__ void __launch_bounds__(FWD_THREADS, 1) flash_fwd32_kernel(const FwdPa
       float mx = s[0];
 #pragma unroll
       for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
-      mx = fmaxf(mx, xhalf(mx));
+      mx = halves_max(mx);
       const float m_new = fmaxf(m_run, mx);
       const float alpha = fast_exp2((m_run - m_new) * c);
       const float mc = m_new * c;
@@ -761,7 +761,7 @@ __global__ void __launch_bounds__(FWD_THREADS, 1) flash_fwd32_kernel(const FwdPa
     __syncthreads();
   }
 
-  const float l_tot = l_run + xhalf(l_run);
+  const float l_tot = halves_sum(l_run);
   const float inv = 1.f / l_tot;
   if (qrow < p.Sq) {
     float* op = (float*)p.out + b * p.os.b + h * p.os.h + (int64_t)qrow * p.os.s;

@@ -114,9 +114,27 @@ static __device__ __forceinline__ F as_frag(u32x4 x) {
   return __builtin_bit_cast(F, x);
 }
 
-// Exchange with the lane 32 away (the other half of the wavefront).
-static __device__ __forceinline__ float xhalf(float x) {
-  return __shfl_xor(x, 32, 64);
+// The two lanes 32 apart share a row of a 32x32 accumulator tile.  v_permlane32_swap hands every
+// lane both of them: the value of lane l % 32 and that of lane 32 + l % 32 (one VALU instruction,
+// no LDS round trip).  The second operand goes through an empty asm so that the compiler sees two
+// distinct registers.
+static __device__ __forceinline__ void both_halves(float x, float& lo, float& hi) {
+  float y = x;
+  asm volatile("" : "+v"(y));
+  const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x), __builtin_bit_cast(unsigned, y), false, false);
+  const unsigned u0 = r[0], u1 = r[1];
+  lo = __builtin_bit_cast(float, u0);
+  hi = __builtin_bit_cast(float, u1);
+}
+static __device__ __forceinline__ float halves_max(float x) {
+  float lo, hi;
+  both_halves(x, lo, hi);
+  return fmaxf(lo, hi);
+}
+static __device__ __forceinline__ float halves_sum(float x) {
+  float lo, hi;
+  both_halves(x, lo, hi);
+  return lo + hi;
 }
 
 // ---- LDS helpers shared by the attention kernels ----
