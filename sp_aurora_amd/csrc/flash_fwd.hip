@@ -433,7 +433,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   __syncthreads();
   if (NG > 1 && grp == 1) __syncthreads();  // group 1 runs one phase behind group 0
 
-  // One loop, no branch around an MFMA, the same two barriers per step for every wave.  A wave
+  // One loop, no branch around an MFMA, the same barriers per step for every wave of a group.  A wave
   // whose rows see none of a diagonal sub-tile's keys (at most the last two sub-tiles of the
   // diagonal chunk) simply gets P = 0 from the mask.
   // MFMA phase i reads V(i) and K(i+1); the other two buffers are free then and receive V(i+1)
@@ -441,8 +441,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // With shared buffers both groups load their share of the same two sub-tiles in the same
   // phase of the workgroup: group 0 during its MFMA phase, group 1 (one phase behind) at the start
   // of its VALU phase; each waits for its loads before the barrier two phases later.
-  constexpr bool LOAD_IN_VALU_PHASE_G1 = SHARE;
-  const bool early = LOAD_IN_VALU_PHASE_G1 && grp == 1;  // wave-uniform
+  const bool early = SHARE && grp == 1;  // wave-uniform
   Cursor cs = cursor_at(0), cv = cursor_at(1), ck = cursor_at(2);
   for (int i = 0; i + 1 < n; ++i) {
     frag pf[2][2];
@@ -455,8 +454,11 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     softmax_phase(cs.sb, pf);
     unsigned va[D / 32], ka[D / 16];
     operand_addresses(i, va, ka);
+    // Shared buffers need one barrier per step and group (after the wait for the loads: group 0
+    // at the end of its VALU phase, group 1 at the end of its MFMA phase, the same physical
+    // barrier); the other one only holds the two groups in step, and they drift little without it.
     if (!early) loads_landed();
-    __syncthreads();
+    if (!SHARE || !early) __syncthreads();
     __builtin_amdgcn_s_setprio(3);
     mfma_phase(std::true_type{}, std::true_type{}, va, ka, pf, [&](int j) {
       constexpr int TOTAL = (D / 32) * 4 + (D / 16) * 2;
@@ -469,7 +471,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     cursor_next(cv);
     cursor_next(ck);
     if (early) loads_landed();
-    __syncthreads();
+    if (!SHARE || early) __syncthreads();
   }
   {  // last sub-tile: nothing to prepare behind it
     frag pf[2][2];
@@ -477,9 +479,9 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     unsigned va[D / 32], ka[D / 16];
     operand_addresses(n - 1, va, ka);
     loads_landed();
-    __syncthreads();
+    if (!SHARE || !early) __syncthreads();
     mfma_phase(std::true_type{}, std::false_type{}, va, ka, pf, [](int) {});
-    __syncthreads();
+    if (!SHARE || early) __syncthreads();
   }
   if (NG > 1 && grp == 0) __syncthreads();  // matches group 1's leading barrier
 
