@@ -193,3 +193,40 @@ def test_config5_qkvpacked_long_context_forward_backward():
             assert not bad.any(), f"{name} h{h}: {int(bad.sum())} out of tolerance, max err {(got - ref).abs().max().item():.3e} (scale {ref.abs().max().item():.3e})"
         del qh, kh, vh, want_o, want_l
         torch.cuda.empty_cache()
+
+
+# ------------------------------------------------------------------ beyond the configs: a long sequence
+def test_long_sequence_131072_forward_backward_spot_checks():
+    """bf16, B=1, S=131072, H=2, D=128, causal (a score matrix no reference can materialise):
+    forward rows and gradient rows / columns against float64 evaluations of the defining sums."""
+    B, S, H, D = 1, 131072, 2, 128
+    scale = D ** -0.5
+    q, k, v, dout = (randn((B, S, H, D), 50 + i, torch.bfloat16) for i in range(4))
+    out, lse = spa.ring.ring_flash_attn_forward(q, k, v, scale, True, 8, fuse="all")
+    o1, l1 = ops.flash_fwd(q, k, v, scale, True)
+    assert_out(out, o1, "ring of 8 vs one block call")
+    assert_lse(lse, l1, "ring of 8 vs one block call")
+    h = 1
+    spot_check_rows(out[0, :, h], lse[0, h], q[0, :, h], k[0, :, h], v[0, :, h], scale, True, "S=131072 fp64", n_rows=6)
+    dq, dk, dv = spa.ring.ring_flash_attn_backward(dout, q, k, v, out, lse, scale, True, 8, fuse="all")
+    # float64 on the CPU, one head
+    qc, kc, vc, doc, oc = (t[0, :, h].cpu().double() for t in (q, k, v, dout, out))
+    lc = lse[0, h].cpu().double()
+    delta = (doc * oc).sum(-1)
+    g = torch.Generator().manual_seed(1)
+    for i in torch.randint(0, S, (4,), generator=g).tolist() + [0, S - 1]:
+        # dq_i = scale * sum_{j<=i} P_ij (dO_i . v_j - delta_i) k_j
+        p = torch.exp(kc[:i + 1] @ qc[i] * scale - lc[i])
+        ds = p * (vc[:i + 1] @ doc[i] - delta[i])
+        want = scale * (ds @ kc[:i + 1])
+        err = (dq[0, i, h].cpu().double() - want).abs().max().item()
+        assert err <= 3e-2 * max(want.abs().max().item(), 1e-2), f"dq row {i}: err {err:.3e} scale {want.abs().max().item():.3e}"
+    for j in torch.randint(0, S, (4,), generator=g).tolist() + [0, S - 1]:
+        # dv_j = sum_{i>=j} P_ij dO_i ;  dk_j = scale * sum_{i>=j} P_ij (dO_i . v_j - delta_i) q_i
+        p = torch.exp(qc[j:] @ kc[j] * scale - lc[j:])
+        want_dv = p @ doc[j:]
+        ds = p * (doc[j:] @ vc[j] - delta[j:])
+        want_dk = scale * (ds @ qc[j:])
+        for name, got, want in (("dv", dv, want_dv), ("dk", dk, want_dk)):
+            err = (got[0, j, h].cpu().double() - want).abs().max().item()
+            assert err <= 3e-2 * max(want.abs().max().item(), 1e-2), f"{name} row {j}: err {err:.3e} scale {want.abs().max().item():.3e}"
