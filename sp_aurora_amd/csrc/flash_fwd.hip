@@ -361,17 +361,27 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         }
     }
 
-    // four independent chains instead of one 32-long dependent one
-    float mxa = fmaxf(s[0][0], s[0][1]), mxb = fmaxf(s[0][8], s[0][9]);
-    float mxc = fmaxf(s[1][0], s[1][1]), mxd = fmaxf(s[1][8], s[1][9]);
-#pragma unroll
-    for (int v = 2; v < 8; v += 2) {
-      mxa = fmaxf(fmaxf(mxa, s[0][v]), s[0][v + 1]);
-      mxb = fmaxf(fmaxf(mxb, s[0][v + 8]), s[0][v + 9]);
-      mxc = fmaxf(fmaxf(mxc, s[1][v]), s[1][v + 1]);
-      mxd = fmaxf(fmaxf(mxd, s[1][v + 8]), s[1][v + 9]);
-    }
-    float mx = fmaxf(fmaxf(mxa, mxb), fmaxf(mxc, mxd));
+    // row max of the lane's 32 scores: 3-input maxima in four independent chains.  (Through the
+    // instruction itself: fmaxf() makes the compiler quiet possible signalling NaNs first, one
+    // extra instruction per MFMA result; the scores are finite or -inf here.)
+    auto max3 = [](float a, float b, float c3) {
+      float r;
+      asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c3));
+      return r;
+    };
+    float mxa = max3(s[0][0], s[0][1], s[0][2]), mxb = max3(s[0][8], s[0][9], s[0][10]);
+    float mxc = max3(s[1][0], s[1][1], s[1][2]), mxd = max3(s[1][8], s[1][9], s[1][10]);
+    mxa = max3(mxa, s[0][3], s[0][4]);
+    mxb = max3(mxb, s[0][11], s[0][12]);
+    mxc = max3(mxc, s[1][3], s[1][4]);
+    mxd = max3(mxd, s[1][11], s[1][12]);
+    mxa = max3(mxa, s[0][5], s[0][6]);
+    mxb = max3(mxb, s[0][13], s[0][14]);
+    mxc = max3(mxc, s[1][5], s[1][6]);
+    mxd = max3(mxd, s[1][13], s[1][14]);
+    mxa = max3(mxa, s[0][7], mxb);
+    mxc = max3(mxc, s[1][7], mxd);
+    float mx = max3(mxa, mxc, fmaxf(s[0][15], s[1][15]));
     mx = halves_max(mx);
     // Lazy rescale: the reference max only moves when some row's max grew by more than
     // 2^8 in the exp2 domain; until then P <= 256, harmless in fp32 sums and bf16 operands.
