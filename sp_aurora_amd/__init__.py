@@ -17,6 +17,7 @@ from .flash_attn import (  # noqa: F401
     intel_flash_attn_forward,
     is_available,
 )
+from .layers import AttnType, LongContextAttention, UlyssesAttention, select_flash_attn_impl  # noqa: F401
 from .ring import (  # noqa: F401
     IntelRingFlashAttnFunc,
     RingFlashAttnFunc,
