@@ -178,6 +178,49 @@ int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout,
                   const int64_t dv_strides[3],
                   float scale, int mask_mode, int dtype, void* stream);
 
+/*
+ * Block attention over a batch of sequences of different lengths packed back
+ * to back (no padding): q / out are [total_q, H, D], k / v [total_k, H, D];
+ * sequence b owns query rows cu_seqlens_q[b] .. cu_seqlens_q[b+1] and key rows
+ * cu_seqlens_k[b] .. cu_seqlens_k[b+1] and attends to nothing else.
+ * cu_seqlens_*: int32[nseq + 1] in DEVICE memory, non-decreasing, first 0,
+ * last = total_*; max_sq / max_sk >= the longest sequence (they size the grid:
+ * rows past max_sq of a longer sequence would be left unwritten).  The library
+ * cannot read the arrays on the host, the caller vouches for them.
+ * lse: fp32 [H, total_q].  A sequence with queries but no keys gets out = 0,
+ * lse = -inf.  mask_mode causal is aligned top-left within each sequence.
+ * *_strides = element strides of (head, row); head-dim stride is 1.
+ * This is the call the reference's variable-length entry points are written
+ * against: sp_aurora_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k,
+ * max_seqlen, ...) in test/flash_attention/test_intel_ring_flash_attn_varlen.py:23-26,66-74
+ * (the function itself is missing from the reference), and the packed lse
+ * layout of flatten_varlen_lse (sp_aurora/utils.py:150-157).
+ */
+int spa_flash_fwd_varlen(const void* q, const void* k, const void* v, void* out, float* lse,
+                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                         int nseq, int H, int total_q, int total_k, int max_sq, int max_sk, int D,
+                         const int64_t q_strides[2], const int64_t k_strides[2],
+                         const int64_t v_strides[2], const int64_t o_strides[2],
+                         float scale, int mask_mode, int dtype, void* stream);
+
+/*
+ * Backward of spa_flash_fwd_varlen, same packing.  lse and delta: fp32
+ * [H, total_q] (delta from spa_bwd_delta with B = 1, Sq = total_q);
+ * dq_acc [total_q, H, D], dk_acc / dv_acc [total_k, H, D]: fp32, ACCUMULATED
+ * into, strides (head, row) as given.  What out.backward() of the reference's
+ * variable-length test needs (test_intel_ring_flash_attn_varlen.py:85-91).
+ */
+int spa_flash_bwd_varlen(const void* q, const void* k, const void* v, const void* dout,
+                         const float* lse, const float* delta,
+                         float* dq_acc, float* dk_acc, float* dv_acc,
+                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                         int nseq, int H, int total_q, int total_k, int max_sq, int max_sk, int D,
+                         const int64_t q_strides[2], const int64_t k_strides[2],
+                         const int64_t v_strides[2], const int64_t do_strides[2],
+                         const int64_t dq_strides[2], const int64_t dk_strides[2],
+                         const int64_t dv_strides[2],
+                         float scale, int mask_mode, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -49,6 +49,7 @@ from .ulysses import (  # noqa: F401
     ulysses_flash_attn_kvpacked_func,
     ulysses_flash_attn_qkvpacked_func,
 )
-from .utils import update_out_and_lse  # noqa: F401
+from .utils import flatten_varlen_lse, unflatten_varlen_lse, update_out_and_lse  # noqa: F401
+from .varlen import VarlenFlashAttnFunc, ring_flash_attn_varlen_func, sp_aurora_varlen_func  # noqa: F401
 
 __version__ = "0.1.0"

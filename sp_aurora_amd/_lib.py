@@ -33,6 +33,8 @@ SIGNATURES = {
     "spa_relayout_h2s": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "spa_bwd_delta": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _s3, _s3, _i, _vp]),
     "spa_flash_bwd": (_i, [_vp] * 9 + [_i] * 5 + [_s3] * 7 + [_f, _i, _i, _vp]),
+    "spa_flash_fwd_varlen": (_i, [_vp] * 7 + [_i] * 7 + [_s3] * 4 + [_f, _i, _i, _vp]),
+    "spa_flash_bwd_varlen": (_i, [_vp] * 11 + [_i] * 7 + [_s3] * 7 + [_f, _i, _i, _vp]),
 }
 
 _lib = None
@@ -69,6 +71,10 @@ def load():
 
 def strides3(vals):
     return _I64x3(*[int(v) for v in vals])
+
+
+def strides2(vals):
+    return (ctypes.c_int64 * 2)(*[int(v) for v in vals])
 
 
 def check(code):

@@ -133,8 +133,30 @@ struct DqCfg {
   static constexpr int NL = 2 * C::NDMA;      // loads per thread and stage
 };
 
+// Variable-length batch: sequence b owns rows cu_q[b] .. cu_q[b+1] of the query-side tensors and
+// cu_k[b] .. cu_k[b+1] of the key-side ones; the kernel then works on that sequence as on batch 0
+// of a batch whose bases and sizes are the sequence's.
+template <typename T>
+__device__ __forceinline__ void select_sequence(BwdParams& p, int& b) {
+  if (!p.cu_q) return;
+  const int q_lo = p.cu_q[b], k_lo = p.cu_k[b];
+  p.Sq = p.cu_q[b + 1] - q_lo;
+  p.Sk = p.cu_k[b + 1] - k_lo;
+  p.q = (const T*)p.q + (int64_t)q_lo * p.qs.s;
+  p.dout = (const T*)p.dout + (int64_t)q_lo * p.dos.s;
+  p.k = (const T*)p.k + (int64_t)k_lo * p.ks.s;
+  p.v = (const T*)p.v + (int64_t)k_lo * p.vs.s;
+  p.dq += (int64_t)q_lo * p.dqs.s;
+  p.dk += (int64_t)k_lo * p.dks.s;
+  p.dv += (int64_t)k_lo * p.dvs.s;
+  p.lse += q_lo;
+  p.delta += q_lo;
+  b = 0;
+}
+
 template <typename T, int D>
-__global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dq_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dq_kernel(const BwdParams pk) {
+  BwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
   typedef BwdCfg<D> C;
   typedef DqCfg<D> G;
   typedef Mma16<T> M;
@@ -149,9 +171,11 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dq_kernel(const BwdP
   const int h = bid % p.H;
   bid /= p.H;
   const int qt = p.nqt - 1 - (bid % p.nqt);
-  const int b = bid / p.nqt;
+  int b = bid / p.nqt;
   const int q0 = qt * 128;
   const int qw0 = q0 + w * 32;
+  select_sequence<T>(p, b);
+  if (q0 >= p.Sq || p.Sk <= 0) return;  // (variable-length batches only) nothing to add to dq
 
   const T* qp = (const T*)p.q + b * p.qs.b + h * p.qs.h;
   const T* kp = (const T*)p.k + b * p.ks.b + h * p.ks.h;
@@ -167,7 +191,7 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dq_kernel(const BwdP
     qf[ks] = as_frag<frag>(*(const u32x4*)(qp + (int64_t)qrow_c * p.qs.s + ks * 16 + hh * 8));
     dof[ks] = as_frag<frag>(*(const u32x4*)(dop + (int64_t)qrow_c * p.dos.s + ks * 16 + hh * 8));
   }
-  const int64_t li = ((int64_t)b * p.H + h) * p.Sq + qrow_c;
+  const int64_t li = ((int64_t)b * p.H + h) * p.lse_bh + qrow_c;
   const float l2 = p.lse[li] * 1.4426950408889634f;
   const float dl = p.delta[li];
   const float c = p.scale_log2;
@@ -340,7 +364,8 @@ struct DkvCfg {
 };
 
 template <typename T, int D>
-__global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const BwdParams pk) {
+  BwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
   typedef BwdCfg<D> C;
   typedef DkvCfg<D> G;
   typedef Mma16<T> M;
@@ -355,16 +380,18 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
   const int h = bid % p.H;
   bid /= p.H;
   const int kt = bid % p.nkt;  // causal: low key tiles see the most query tiles, they go first
-  const int b = bid / p.nkt;
+  int b = bid / p.nkt;
   const int k0 = kt * 128;
   const int kw0 = k0 + w * 32;
+  select_sequence<T>(p, b);
+  if (k0 >= p.Sk || p.Sq <= 0 || (p.causal && k0 >= p.Sq)) return;  // no query sees these keys: nothing to add to dk, dv
 
   const T* qp = (const T*)p.q + b * p.qs.b + h * p.qs.h;
   const T* kp = (const T*)p.k + b * p.ks.b + h * p.ks.h;
   const T* vp = (const T*)p.v + b * p.vs.b + h * p.vs.h;
   const T* dop = (const T*)p.dout + b * p.dos.b + h * p.dos.h;
-  const float* lsep = p.lse + ((int64_t)b * p.H + h) * p.Sq;
-  const float* delp = p.delta + ((int64_t)b * p.H + h) * p.Sq;
+  const float* lsep = p.lse + ((int64_t)b * p.H + h) * p.lse_bh;
+  const float* delp = p.delta + ((int64_t)b * p.H + h) * p.lse_bh;
 
   const int krow = kw0 + ln;
   const int krow_c = krow < p.Sk ? krow : p.Sk - 1;
@@ -619,7 +646,8 @@ struct PairStage {
 };
 
 template <int D>
-__global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dq_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dq_kernel(const BwdParams pk) {
+  BwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
   typedef Bwd32Cfg<D> C;
   extern __shared__ __align__(16) unsigned char smem[];
   float* sm = (float*)smem;
@@ -630,9 +658,11 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dq_kernel(const Bw
   const int h = bid % p.H;
   bid /= p.H;
   const int qt = p.nqt - 1 - (bid % p.nqt);
-  const int b = bid / p.nqt;
+  int b = bid / p.nqt;
   const int q0 = qt * 128;
   const int qw0 = q0 + w * 32;
+  select_sequence<float>(p, b);
+  if (q0 >= p.Sq || p.Sk <= 0) return;  // (variable-length batches only) nothing to add to dq
 
   const float* qp = (const float*)p.q + b * p.qs.b + h * p.qs.h;
   const float* kp = (const float*)p.k + b * p.ks.b + h * p.ks.h;
@@ -648,7 +678,7 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dq_kernel(const Bw
     qf[g] = *(const f32x4*)(qp + (int64_t)qrow_c * p.qs.s + 8 * g + 4 * hh);
     dof[g] = *(const f32x4*)(dop + (int64_t)qrow_c * p.dos.s + 8 * g + 4 * hh);
   }
-  const int64_t li = ((int64_t)b * p.H + h) * p.Sq + qrow_c;
+  const int64_t li = ((int64_t)b * p.H + h) * p.lse_bh + qrow_c;
   const float l2 = p.lse[li] * 1.4426950408889634f;
   const float dl = p.delta[li];
   const float c = p.scale_log2;
@@ -721,7 +751,8 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dq_kernel(const Bw
 }
 
 template <int D>
-__global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dkdv_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dkdv_kernel(const BwdParams pk) {
+  BwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
   typedef Bwd32Cfg<D> C;
   extern __shared__ __align__(16) unsigned char smem[];
   float* sm = (float*)smem;
@@ -732,16 +763,18 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dkdv_kernel(const 
   const int h = bid % p.H;
   bid /= p.H;
   const int kt = bid % p.nkt;
-  const int b = bid / p.nkt;
+  int b = bid / p.nkt;
   const int k0 = kt * 128;
   const int kw0 = k0 + w * 32;
+  select_sequence<float>(p, b);
+  if (k0 >= p.Sk || p.Sq <= 0 || (p.causal && k0 >= p.Sq)) return;  // no query sees these keys: nothing to add to dk, dv
 
   const float* qp = (const float*)p.q + b * p.qs.b + h * p.qs.h;
   const float* kp = (const float*)p.k + b * p.ks.b + h * p.ks.h;
   const float* vp = (const float*)p.v + b * p.vs.b + h * p.vs.h;
   const float* dop = (const float*)p.dout + b * p.dos.b + h * p.dos.h;
-  const float* lsep = p.lse + ((int64_t)b * p.H + h) * p.Sq;
-  const float* delp = p.delta + ((int64_t)b * p.H + h) * p.Sq;
+  const float* lsep = p.lse + ((int64_t)b * p.H + h) * p.lse_bh;
+  const float* delp = p.delta + ((int64_t)b * p.H + h) * p.lse_bh;
 
   const int krow = kw0 + ln;
   const int krow_c = krow < p.Sk ? krow : p.Sk - 1;

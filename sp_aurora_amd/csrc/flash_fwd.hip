@@ -78,8 +78,9 @@ __device__ __forceinline__ int v_swizzle(int row) {
 }
 
 template <typename T, int D, int NG, bool SHARE>
-__global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams p) {
+__global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams pk) {
   typedef Fwd16Cfg<D, NG, SHARE> C;
+  FwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
   typedef Mma16<T> M;
   typedef typename M::frag frag;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -101,9 +102,32 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   bid /= p.H;
   const int qt = p.nqt - 1 - (bid % p.nqt);
   bid /= p.nqt;
-  const int b = bid % p.B;
+  int b = bid % p.B;
   const int rank = p.rank0 + p.nranks - 1 - bid / p.B;
   const int q0 = qt * C::BMW;
+  if (p.cu_q) {
+    const int q_lo = p.cu_q[b], k_lo = p.cu_k[b];
+    p.Sq = p.cu_q[b + 1] - q_lo;
+    p.Sk = p.cu_k[b + 1] - k_lo;
+    p.q = (const T*)p.q + (int64_t)q_lo * p.qs.s;
+    p.k = (const T*)p.k + (int64_t)k_lo * p.ks.s;
+    p.v = (const T*)p.v + (int64_t)k_lo * p.vs.s;
+    p.out = (T*)p.out + (int64_t)q_lo * p.os.s;
+    p.lse += q_lo;
+    b = 0;
+    if (q0 >= p.Sq) return;  // this sequence is shorter than the longest one
+    if (p.Sk <= 0) {
+      // no keys: the empty sum, out = 0 and lse = -inf
+      for (int idx = tid; idx < C::BMW * (D / 8); idx += FWD_THREADS * NG) {
+        const int grow = q0 + idx / (D / 8), ch = idx % (D / 8);
+        if (grow >= p.Sq) break;
+        u32x4 z = {0u, 0u, 0u, 0u};
+        *(u32x4*)((T*)p.out + h * p.os.h + (int64_t)grow * p.os.s + ch * 8) = z;
+        if (ch == 0) p.lse[(int64_t)h * p.lse_bh + grow] = -INFINITY;
+      }
+      return;
+    }
+  }
   const int qw0 = q0 + (SHARE ? grp * FWD_BM : 0) + w * 32;
   const int64_t qoff = (int64_t)rank * p.Sq;  // first row of this rank's query chunk
 
@@ -621,8 +645,9 @@ struct Fwd32Cfg {
 };
 
 template <int D>
-__global__ void __launch_bounds__(FWD_THREADS, 1) flash_fwd32_kernel(const FwdParams p) {
+__global__ void __launch_bounds__(FWD_THREADS, 1) flash_fwd32_kernel(const FwdParams pk) {
   typedef Fwd32Cfg<D> C;
+  FwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
   extern __shared__ __align__(16) unsigned char smem[];
   float* sm = (float*)smem;
 
@@ -636,9 +661,31 @@ __global__ void __launch_bounds__(FWD_THREADS, 1) flash_fwd32_kernel(const FwdPa
   const int h = bid % p.H;
   bid /= p.H;
   const int qt = p.nqt - 1 - (bid % p.nqt);
-  const int b = bid / p.nqt;
+  int b = bid / p.nqt;
   const int q0 = qt * FWD_BM;
   const int qw0 = q0 + w * 32;
+  if (p.cu_q) {
+    const int q_lo = p.cu_q[b], k_lo = p.cu_k[b];
+    p.Sq = p.cu_q[b + 1] - q_lo;
+    p.Sk = p.cu_k[b + 1] - k_lo;
+    p.q = (const float*)p.q + (int64_t)q_lo * p.qs.s;
+    p.k = (const float*)p.k + (int64_t)k_lo * p.ks.s;
+    p.v = (const float*)p.v + (int64_t)k_lo * p.vs.s;
+    p.out = (float*)p.out + (int64_t)q_lo * p.os.s;
+    p.lse += q_lo;
+    b = 0;
+    if (q0 >= p.Sq) return;
+    if (p.Sk <= 0) {
+      for (int idx = tid; idx < FWD_BM * (D / 4); idx += FWD_THREADS) {
+        const int grow = q0 + idx / (D / 4), ch = idx % (D / 4);
+        if (grow >= p.Sq) break;
+        f32x4 z = {0.f, 0.f, 0.f, 0.f};
+        *(f32x4*)((float*)p.out + h * p.os.h + (int64_t)grow * p.os.s + ch * 4) = z;
+        if (ch == 0) p.lse[(int64_t)h * p.lse_bh + grow] = -INFINITY;
+      }
+      return;
+    }
+  }
 
   const float* qp = (const float*)p.q + b * p.qs.b + h * p.qs.h;
   const float* kp = (const float*)p.k + b * p.ks.b + h * p.ks.h;

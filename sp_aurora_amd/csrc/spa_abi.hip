@@ -118,6 +118,7 @@ int spa_flash_fwd(const void* q, const void* k, const void* v, void* out, float*
   p.as = S3(o_strides);
   p.epi = SPA_EPI_PLAIN;
   p.P = 1; p.rank0 = 0; p.nranks = 1; p.t_begin = 0; p.t_count = -1;
+  p.cu_q = nullptr; p.cu_k = nullptr;
   return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), "spa_flash_fwd");
 }
 
@@ -197,6 +198,7 @@ int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* 
   p.as = as;
   p.P = P;
   p.epi = SPA_EPI_PLAIN;
+  p.cu_q = nullptr; p.cu_k = nullptr;
 
   if (fuse == SPA_RING_ALL_RANKS) {  // one launch: every requested rank, every step
     p.rank0 = r_lo; p.nranks = r_hi - r_lo; p.t_begin = 0; p.t_count = -1;
@@ -335,7 +337,107 @@ int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout,
   p.causal = mask_mode == SPA_MASK_CAUSAL;
   p.nqt = 0;
   p.nkt = 0;
+  p.lse_bh = Sq;
+  p.cu_q = nullptr; p.cu_k = nullptr;
   return launch_result(spa_launch_flash_bwd(p, D, dtype, (hipStream_t)stream), "spa_flash_bwd");
+}
+
+namespace {
+// Strides of a packed [rows, H, D] tensor come as (head, row); the batch stride is unused.
+Strides3 S2(const int64_t* s) {
+  Strides3 r;
+  r.b = 0; r.h = s[0]; r.s = s[1];
+  return r;
+}
+bool aligned16v(const void* p, const int64_t* s, int esz) {
+  return ((uintptr_t)p & 15) == 0 && (s[0] * esz) % 16 == 0 && (s[1] * esz) % 16 == 0;
+}
+int varlen_sizes_ok(const char* what, const void* cu_q, const void* cu_k, int nseq, int H, int total_q, int total_k,
+                    int max_sq, int max_sk, int D, int dtype, int mask_mode, float scale) {
+  if (!cu_q || !cu_k) return fail(SPA_EINVAL, "%s: null cu_seqlens", what);
+  if ((((uintptr_t)cu_q | (uintptr_t)cu_k) & 3) != 0) return fail(SPA_EALIGN, "%s: cu_seqlens must be 4-byte aligned", what);
+  if (nseq <= 0 || H <= 0 || total_q <= 0 || total_k <= 0 || max_sq <= 0 || max_sk <= 0 || max_sq > total_q || max_sk > total_k)
+    return fail(SPA_EINVAL, "%s: sizes must be positive and the longest sequence no longer than the total (nseq=%d H=%d total_q=%d total_k=%d max_sq=%d max_sk=%d)",
+                what, nseq, H, total_q, total_k, max_sq, max_sk);
+  if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "%s: bad dtype %d", what, dtype);
+  if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "%s: bad mask_mode %d", what, mask_mode);
+  if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "%s: softmax scale must be positive and finite", what);
+  if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "%s: head dim %d not in {32,64,128}", what, D);
+  if ((int64_t)nseq * H * ((max_sq + 127) / 128) > 0x7fffffffLL || (int64_t)nseq * H * ((max_sk + 127) / 128) > 0x7fffffffLL)
+    return fail(SPA_EINVAL, "%s: grid too large", what);
+  return SPA_OK;
+}
+}  // namespace
+
+int spa_flash_fwd_varlen(const void* q, const void* k, const void* v, void* out, float* lse,
+                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int nseq, int H, int total_q,
+                         int total_k, int max_sq, int max_sk, int D, const int64_t q_strides[2],
+                         const int64_t k_strides[2], const int64_t v_strides[2], const int64_t o_strides[2],
+                         float scale, int mask_mode, int dtype, void* stream) {
+  if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "spa_flash_fwd_varlen: null pointer");
+  if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(SPA_EINVAL, "spa_flash_fwd_varlen: null strides");
+  const int rc = varlen_sizes_ok("spa_flash_fwd_varlen", cu_seqlens_q, cu_seqlens_k, nseq, H, total_q, total_k, max_sq,
+                                 max_sk, D, dtype, mask_mode, scale);
+  if (rc != SPA_OK) return rc;
+  const int esz = elem_size(dtype);
+  if (!aligned16v(q, q_strides, esz) || !aligned16v(k, k_strides, esz) || !aligned16v(v, v_strides, esz) ||
+      !aligned16v(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0)
+    return fail(SPA_EALIGN, "spa_flash_fwd_varlen: pointers and row strides must be 16-byte aligned");
+  if (!span_ok(max_sk, k_strides[1], D, esz) || !span_ok(max_sk, v_strides[1], D, esz))
+    return fail(SPA_EUNSUPPORTED, "spa_flash_fwd_varlen: K/V of one (sequence, head) span more than 2 GiB");
+  FwdParams p;
+  p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
+  p.B = nseq; p.H = H; p.Sq = max_sq; p.Sk = max_sk;
+  p.qs = S2(q_strides); p.ks = S2(k_strides); p.vs = S2(v_strides); p.os = S2(o_strides);
+  p.scale = scale;
+  p.scale_log2 = scale * 1.4426950408889634f;
+  p.causal = mask_mode == SPA_MASK_CAUSAL;
+  p.nqt = 0;
+  p.lse_bh = total_q;
+  p.acc = nullptr;
+  p.as = S2(o_strides);
+  p.epi = SPA_EPI_PLAIN;
+  p.P = 1; p.rank0 = 0; p.nranks = 1; p.t_begin = 0; p.t_count = -1;
+  p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
+  return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), "spa_flash_fwd_varlen");
+}
+
+int spa_flash_bwd_varlen(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                         const float* delta, float* dq_acc, float* dk_acc, float* dv_acc,
+                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int nseq, int H, int total_q,
+                         int total_k, int max_sq, int max_sk, int D, const int64_t q_strides[2],
+                         const int64_t k_strides[2], const int64_t v_strides[2], const int64_t do_strides[2],
+                         const int64_t dq_strides[2], const int64_t dk_strides[2], const int64_t dv_strides[2],
+                         float scale, int mask_mode, int dtype, void* stream) {
+  if (!q || !k || !v || !dout || !lse || !delta || !dq_acc || !dk_acc || !dv_acc)
+    return fail(SPA_EINVAL, "spa_flash_bwd_varlen: null pointer");
+  if (!q_strides || !k_strides || !v_strides || !do_strides || !dq_strides || !dk_strides || !dv_strides)
+    return fail(SPA_EINVAL, "spa_flash_bwd_varlen: null strides");
+  const int rc = varlen_sizes_ok("spa_flash_bwd_varlen", cu_seqlens_q, cu_seqlens_k, nseq, H, total_q, total_k, max_sq,
+                                 max_sk, D, dtype, mask_mode, scale);
+  if (rc != SPA_OK) return rc;
+  const int esz = elem_size(dtype);
+  if (!aligned16v(q, q_strides, esz) || !aligned16v(k, k_strides, esz) || !aligned16v(v, v_strides, esz) ||
+      !aligned16v(dout, do_strides, esz) || !aligned16v(dq_acc, dq_strides, 4) || !aligned16v(dk_acc, dk_strides, 4) ||
+      !aligned16v(dv_acc, dv_strides, 4) || (((uintptr_t)lse | (uintptr_t)delta) & 3) != 0)
+    return fail(SPA_EALIGN, "spa_flash_bwd_varlen: pointers and row strides must be 16-byte aligned");
+  if (!span_ok(max_sq, q_strides[1], D, esz) || !span_ok(max_sk, k_strides[1], D, esz) ||
+      !span_ok(max_sk, v_strides[1], D, esz) || !span_ok(max_sq, do_strides[1], D, esz))
+    return fail(SPA_EUNSUPPORTED, "spa_flash_bwd_varlen: a tensor of one (sequence, head) spans more than 2 GiB");
+  BwdParams p;
+  p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta;
+  p.dq = dq_acc; p.dk = dk_acc; p.dv = dv_acc;
+  p.B = nseq; p.H = H; p.Sq = max_sq; p.Sk = max_sk;
+  p.qs = S2(q_strides); p.ks = S2(k_strides); p.vs = S2(v_strides); p.dos = S2(do_strides);
+  p.dqs = S2(dq_strides); p.dks = S2(dk_strides); p.dvs = S2(dv_strides);
+  p.scale = scale;
+  p.scale_log2 = scale * 1.4426950408889634f;
+  p.causal = mask_mode == SPA_MASK_CAUSAL;
+  p.nqt = 0;
+  p.nkt = 0;
+  p.lse_bh = total_q;
+  p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
+  return launch_result(spa_launch_flash_bwd(p, D, dtype, (hipStream_t)stream), "spa_flash_bwd_varlen");
 }
 
 }  // extern "C"

@@ -35,6 +35,11 @@ struct FwdParams {
   float* acc;        // fp32 running output, [B,H,Sq,D] by `as` (SPA_EPI_INIT/MERGE/FINAL)
   Strides3 as;
   int epi;
+  // variable-length batch (null: every sequence has Sq queries and Sk keys): sequence b owns rows
+  // cu_q[b] .. cu_q[b+1] of q/out/lse and cu_k[b] .. cu_k[b+1] of k/v, batch strides are unused,
+  // Sq and Sk are the longest sequence's sizes (they shape the grid) and lse is [H][lse_bh]
+  const int* cu_q;
+  const int* cu_k;
 };
 
 enum {
@@ -61,6 +66,11 @@ struct BwdParams {
   int causal;
   int nqt;  // number of query tiles per (batch, head)
   int nkt;  // number of key tiles per (batch, head)
+  int64_t lse_bh;  // elements between consecutive (batch, head) rows of lse and delta
+  // variable-length batch, as in FwdParams: rows cu_q[b] .. cu_q[b+1] of q/dout/dq/lse/delta and
+  // cu_k[b] .. cu_k[b+1] of k/v/dk/dv belong to sequence b; lse and delta are [H][lse_bh]
+  const int* cu_q;
+  const int* cu_k;
 };
 
 // 16-bit element traits: MFMA 32x32x16 with 8 elements per lane per operand.

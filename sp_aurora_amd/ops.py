@@ -243,3 +243,83 @@ def flash_bwd(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, softmax_scale=N
             float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE,
             _dtype_code(q), _stream()))
     return dq_acc, dk_acc, dv_acc
+
+
+# ------------------------------------------------------------------ variable-length batches
+def _thd(t, what):
+    """(rows, H, D) sizes and (head, row) element strides of a packed 3-D tensor."""
+    if t.dim() != 3:
+        raise ValueError(f"{what}: expected a packed [total, H, D] tensor, got {tuple(t.shape)}")
+    return tuple(t.shape), (t.stride(1), t.stride(0))
+
+
+def _cu(cu, device, what):
+    if cu.dim() != 1 or cu.numel() < 2:
+        raise ValueError(f"{what} must be a 1-D tensor of nseq + 1 offsets, got {tuple(cu.shape)}")
+    if cu.dtype != torch.int32 or cu.device != device or not cu.is_contiguous():
+        cu = cu.to(device=device, dtype=torch.int32).contiguous()
+    return cu
+
+
+def flash_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale=None,
+                     causal=False, out=None, lse=None):
+    """Attention inside each sequence of a packed batch: q [total_q,H,D], k,v [total_k,H,D],
+    cu_seqlens_* int32 [nseq+1] on the device.  Returns (out like q, lse fp32 [H,total_q]).
+    Calls spa_flash_fwd_varlen."""
+    lib = _lib.load()
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise TypeError("q, k, v must share a dtype")
+    (Tq, H, D), qs = _thd(q, "q")
+    (Tk, Hk, Dk), ks = _thd(k, "k")
+    shp_v, vs = _thd(v, "v")
+    if (Hk, Dk) != (H, D) or shp_v != (Tk, Hk, Dk):
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    cu_q, cu_k = _cu(cu_seqlens_q, q.device, "cu_seqlens_q"), _cu(cu_seqlens_k, q.device, "cu_seqlens_k")
+    if cu_q.numel() != cu_k.numel():
+        raise ValueError("cu_seqlens_q and cu_seqlens_k must describe the same number of sequences")
+    if softmax_scale is None:
+        softmax_scale = D ** (-0.5)
+    if out is None:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    if lse is None:
+        lse = torch.empty((H, Tq), dtype=torch.float32, device=q.device)
+    _, os_ = _thd(out, "out")
+    with torch.cuda.device(q.device):
+        _lib.check(lib.spa_flash_fwd_varlen(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(),
+            cu_q.numel() - 1, H, Tq, Tk, int(max_seqlen_q), int(max_seqlen_k), D,
+            _lib.strides2(qs), _lib.strides2(ks), _lib.strides2(vs), _lib.strides2(os_),
+            float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(q), _stream()))
+    return out, lse
+
+
+def flash_bwd_varlen(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
+                     max_seqlen_k, softmax_scale=None, causal=False):
+    """Backward of flash_fwd_varlen; adds into the fp32 accumulators dq [total_q,H,D], dk, dv
+    [total_k,H,D].  lse, delta: fp32 [H,total_q].  Calls spa_flash_bwd_varlen."""
+    lib = _lib.load()
+    q, k, v, dout = _prep(q), _prep(k), _prep(v), _prep(dout)
+    (Tq, H, D), qs = _thd(q, "q")
+    (Tk, _, _), ks = _thd(k, "k")
+    _, vs = _thd(v, "v")
+    _, dos = _thd(dout, "dout")
+    _, dqs = _thd(dq_acc, "dq_acc")
+    _, dks = _thd(dk_acc, "dk_acc")
+    _, dvs = _thd(dv_acc, "dv_acc")
+    for t in (dq_acc, dk_acc, dv_acc, lse, delta):
+        if t.dtype != torch.float32:
+            raise TypeError("accumulators, lse and delta must be float32")
+    if tuple(lse.shape) != (H, Tq) or tuple(delta.shape) != (H, Tq) or not lse.is_contiguous() or not delta.is_contiguous():
+        raise ValueError("lse and delta must be contiguous [H, total_q]")
+    cu_q, cu_k = _cu(cu_seqlens_q, q.device, "cu_seqlens_q"), _cu(cu_seqlens_k, q.device, "cu_seqlens_k")
+    if softmax_scale is None:
+        softmax_scale = D ** (-0.5)
+    with torch.cuda.device(q.device):
+        _lib.check(lib.spa_flash_bwd_varlen(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            dq_acc.data_ptr(), dk_acc.data_ptr(), dv_acc.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(),
+            cu_q.numel() - 1, H, Tq, Tk, int(max_seqlen_q), int(max_seqlen_k), D,
+            _lib.strides2(qs), _lib.strides2(ks), _lib.strides2(vs), _lib.strides2(dos), _lib.strides2(dqs),
+            _lib.strides2(dks), _lib.strides2(dvs),
+            float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(q), _stream()))

@@ -1,0 +1,68 @@
+"""Attention over packed variable-length batches (`cu_seqlens`), on one GPU.
+
+The reference's tests and adapter are written against sp_aurora_varlen_func(q, k, v,
+cu_seqlens_q, cu_seqlens_k, max_seqlen=..., dropout_p=..., causal=...)
+(test/flash_attention/test_intel_ring_flash_attn_varlen.py:23-26,66-74,85-91) but the
+reference does not ship the function; only the lse helpers exist (sp_aurora/utils.py:150-169).
+Here it is the block attention kernels run once over the packed batch, every sequence
+attending to itself only, with a backward pass.  A ring over packed batches (every rank
+holding a slice of every sequence) is not built: with one GPU a ring of one is the whole
+computation.
+"""
+import torch
+
+from . import ops
+from .flash_attn import _check_unsupported
+from .ring import _no_multi_gpu
+
+__all__ = ["sp_aurora_varlen_func", "ring_flash_attn_varlen_func", "VarlenFlashAttnFunc"]
+
+
+class VarlenFlashAttnFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, causal,
+                return_softmax):
+        if softmax_scale is None:
+            softmax_scale = q.shape[-1] ** (-0.5)
+        out, lse = ops.flash_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                                        softmax_scale, causal)
+        ctx.save_for_backward(q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k)
+        ctx.args = (int(max_seqlen_q), int(max_seqlen_k), softmax_scale, causal)
+        ctx.mark_non_differentiable(lse)
+        return out if not return_softmax else (out, lse, None)
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        q, k, v, out, lse, cu_q, cu_k = ctx.saved_tensors
+        max_q, max_k, scale, causal = ctx.args
+        # delta = rowsum(dout * out) per (row, head): the packed tensors are one batch of total_q rows
+        delta = ops.bwd_delta(out.unsqueeze(0), dout.unsqueeze(0), layout="bshd")[0]
+        dq = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
+        dk = torch.zeros(k.shape, dtype=torch.float32, device=q.device)
+        dv = torch.zeros(v.shape, dtype=torch.float32, device=q.device)
+        ops.flash_bwd_varlen(q, k, v, dout, lse, delta, dq, dk, dv, cu_q, cu_k, max_q, max_k, scale, causal)
+        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None, None, None, None, None
+
+
+def sp_aurora_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k=None, max_seqlen=None, dropout_p=0.0,
+                          softmax_scale=None, causal=False, window_size=(-1, -1), alibi_slopes=None,
+                          deterministic=False, return_attn_probs=False, group=None, *, max_seqlen_k=None):
+    """q [total_q,H,D], k,v [total_k,H,D] packed without padding; sequence b owns rows
+    cu_seqlens_q[b]..cu_seqlens_q[b+1] of q and cu_seqlens_k[b]..cu_seqlens_k[b+1] of k, v
+    (cu_seqlens_k defaults to cu_seqlens_q).  max_seqlen: the longest sequence (of the queries;
+    max_seqlen_k for the keys if different); computed from cu_seqlens (one device-to-host
+    read) when omitted.  Returns out [total_q,H,D], or (out, lse fp32 [H,total_q], None) with
+    return_attn_probs."""
+    _check_unsupported(dropout_p, window_size, alibi_slopes)
+    _no_multi_gpu(group)
+    if cu_seqlens_k is None:
+        cu_seqlens_k = cu_seqlens_q
+    if max_seqlen is None:
+        max_seqlen = int((cu_seqlens_q[1:] - cu_seqlens_q[:-1]).max())
+    if max_seqlen_k is None:
+        max_seqlen_k = max_seqlen if cu_seqlens_k is cu_seqlens_q else int((cu_seqlens_k[1:] - cu_seqlens_k[:-1]).max())
+    return VarlenFlashAttnFunc.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen, max_seqlen_k, softmax_scale,
+                                     causal, return_attn_probs)
+
+
+ring_flash_attn_varlen_func = sp_aurora_varlen_func

@@ -67,6 +67,24 @@ def test_bad_arguments_return_codes_without_touching_a_device():
     f = ctypes.c_void_p(4096)
     args = [f] * 9 + [1, 1, 8, 8, 64] + [st] * 7
     assert lib.spa_flash_bwd(*args, 1.0, 0, 9, None) == -1
+    # variable-length batches: (head, row) strides; the cu_seqlens arrays are never read on the host
+    s2 = _lib.strides2((64, 64))
+    ok = [p] * 7 + [2, 1, 16, 16, 8, 8, 64, s2, s2, s2, s2, 1.0, 1, 1, None]
+    bad = list(ok); bad[5] = None  # cu_seqlens_q
+    assert lib.spa_flash_fwd_varlen(*bad) == -1 and b"cu_seqlens" in lib.spa_last_error()
+    bad = list(ok); bad[11] = 32  # longest sequence longer than the total
+    assert lib.spa_flash_fwd_varlen(*bad) == -1
+    bad = list(ok); bad[13] = 48  # head dim
+    assert lib.spa_flash_fwd_varlen(*bad) == -2
+    bad = list(ok); bad[5] = ctypes.c_void_p(4098)  # cu_seqlens alignment
+    assert lib.spa_flash_fwd_varlen(*bad) == -3
+    bad = list(ok); bad[14] = _lib.strides2((64, 63))  # row stride
+    assert lib.spa_flash_fwd_varlen(*bad) == -3
+    okb = [p] * 11 + [2, 1, 16, 16, 8, 8, 64] + [s2] * 7 + [1.0, 1, 1, None]
+    bad = list(okb); bad[11] = 0  # no sequences
+    assert lib.spa_flash_bwd_varlen(*bad) == -1
+    bad = list(okb); bad[-2] = 9  # dtype
+    assert lib.spa_flash_bwd_varlen(*bad) == -1
 
 
 def test_python_wrappers_refuse_cpu_tensors():
@@ -115,3 +133,8 @@ def test_unsupported_features_raise_before_any_launch():
         spa.ring_flash_attn_func(q, q, q, alibi_slopes=torch.zeros(1))
     with pytest.raises(NotImplementedError):
         spa.ring_flash_attn_func(q, q, q, group=object())
+    cu = torch.tensor([0, 8], dtype=torch.int32)
+    with pytest.raises(NotImplementedError):
+        spa.sp_aurora_varlen_func(q[0], q[0], q[0], cu, cu, max_seqlen=8, dropout_p=0.1)
+    with pytest.raises(ValueError, match="HIP device"):
+        spa.sp_aurora_varlen_func(q[0], q[0], q[0], cu, cu, max_seqlen=8)

@@ -1,0 +1,143 @@
+"""GPU parity of attention over packed variable-length batches: every sequence of the packed
+batch must come out as the oracle's attention of that sequence alone (forward, lse, gradients).
+The sequence-length patterns of the reference's own test come first
+(test/flash_attention/test_intel_ring_flash_attn_varlen.py:42-48,146)."""
+import pytest
+import torch
+
+from conftest import rand
+from oracle import attn_oracle as O
+import sp_aurora_amd as spa
+from sp_aurora_amd import ops
+from test_gpu_parity import DEV, check_grad, check_lse, check_out
+
+pytestmark = pytest.mark.gpu
+
+
+def cu_of(lengths):
+    return torch.tensor([0] + list(torch.tensor(lengths).cumsum(0)), dtype=torch.int32)
+
+
+def per_sequence(q, k, v, lens_q, lens_k, causal):
+    """Oracle attention of each sequence alone -> packed out [Tq,H,D], lse [H,Tq]."""
+    outs, lses = [], []
+    q0 = k0 = 0
+    for lq, lk in zip(lens_q, lens_k):
+        if lq == 0:
+            k0 += lk
+            continue
+        if lk == 0:
+            outs.append(torch.zeros(lq, q.shape[1], q.shape[2], dtype=torch.float64))
+            lses.append(torch.full((q.shape[1], lq), float("-inf"), dtype=torch.float64))
+        else:
+            o, l = O.full_attention(q[None, q0:q0 + lq], k[None, k0:k0 + lk], v[None, k0:k0 + lk], None, causal)
+            outs.append(o[0])
+            lses.append(l[0])
+        q0 += lq
+        k0 += lk
+    return torch.cat(outs, 0), torch.cat(lses, 1)
+
+
+SELF_CASES = [
+    # lengths, H, D, dtype, causal
+    ([128, 256, 128], 8, 64, torch.float16, True),        # "Mixed lengths"
+    ([100, 100, 100, 100], 8, 64, torch.float16, True),   # "Equal lengths"
+    ([512], 8, 64, torch.float16, True),                  # "Single sequence"
+    ([64, 128, 256, 512], 8, 64, torch.float16, True),    # "Increasing lengths"
+    ([128, 256, 128, 192], 8, 64, torch.float16, True),   # the distributed test's batch
+    ([1, 77, 300, 5, 129], 3, 128, torch.bfloat16, False),
+    ([1, 77, 300, 5, 129], 3, 128, torch.bfloat16, True),
+    ([33, 1, 64, 200], 2, 32, torch.bfloat16, True),
+    ([40, 130, 7], 2, 64, torch.float32, True),
+    ([40, 130, 7], 2, 128, torch.float32, False),
+]
+
+
+@pytest.mark.parametrize("lengths,H,D,dtype,causal", SELF_CASES)
+def test_varlen_forward_and_backward_match_per_sequence_attention(lengths, H, D, dtype, causal):
+    T = sum(lengths)
+    q, k, v, dout = (rand((T, H, D), 400 + i, dtype) for i in range(4))
+    want_out, want_lse = per_sequence(q, k, v, lengths, lengths, causal)
+    cu = cu_of(lengths).to(DEV)
+    xs = [t.to(DEV).requires_grad_(True) for t in (q, k, v)]
+    out, lse, _ = spa.sp_aurora_varlen_func(*xs, cu, cu, max_seqlen=max(lengths), dropout_p=0.0, causal=causal,
+                                            return_attn_probs=True)
+    assert out.shape == (T, H, D) and out.dtype == dtype and lse.shape == (H, T)
+    check_out(out, want_out, dtype)
+    check_lse(lse, want_lse)
+    out.backward(dout.to(DEV))
+    s0 = 0
+    for n in lengths:
+        sl = slice(s0, s0 + n)
+        want = O.attn_backward_autograd(q[None, sl], k[None, sl], v[None, sl], dout[None, sl], None, causal)
+        for x, w, name in zip(xs, want, "qkv"):
+            if n == 1 and name in "qk":
+                # a single key: the softmax is constant, dq = dk = 0 exactly; rounding of P - 1 remains
+                assert w.abs().max() < 1e-12 and x.grad[sl].abs().max() < 1e-5
+                continue
+            check_grad(x.grad[sl], w[0], dtype, f"d{name} of the sequence at {s0}")
+        s0 += n
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_varlen_with_different_query_and_key_lengths_and_empty_sequences(causal):
+    lens_q = [50, 0, 130, 20, 64]
+    lens_k = [70, 40, 0, 300, 10]
+    H, D, dtype = 2, 64, torch.bfloat16
+    q = rand((sum(lens_q), H, D), 410, dtype)
+    k, v = rand((sum(lens_k), H, D), 411, dtype), rand((sum(lens_k), H, D), 412, dtype)
+    dout = rand((sum(lens_q), H, D), 413, dtype)
+    want_out, want_lse = per_sequence(q, k, v, lens_q, lens_k, causal)
+    xs = [t.to(DEV).requires_grad_(True) for t in (q, k, v)]
+    out, lse, _ = spa.sp_aurora_varlen_func(*xs, cu_of(lens_q).to(DEV), cu_of(lens_k).to(DEV), causal=causal,
+                                            return_attn_probs=True)
+    check_out(out, want_out, dtype)
+    got_lse = lse.cpu().double()
+    finite = torch.isfinite(want_lse)
+    assert torch.equal(torch.isneginf(got_lse), torch.isneginf(want_lse))
+    assert (got_lse[finite] - want_lse[finite]).abs().max() <= 1e-3
+    out.backward(dout.to(DEV))
+    q0 = k0 = 0
+    for lq, lk in zip(lens_q, lens_k):
+        qs, ks = slice(q0, q0 + lq), slice(k0, k0 + lk)
+        if lq and lk:
+            want = O.attn_backward_autograd(q[None, qs], k[None, ks], v[None, ks], dout[None, qs], None, causal)
+            check_grad(xs[0].grad[qs], want[0][0], dtype, "dq")
+            check_grad(xs[1].grad[ks], want[1][0], dtype, "dk")
+            check_grad(xs[2].grad[ks], want[2][0], dtype, "dv")
+        else:  # nothing attends, or nothing is attended to
+            assert not xs[0].grad[qs].any() and not xs[1].grad[ks].any() and not xs[2].grad[ks].any()
+        q0 += lq
+        k0 += lk
+
+
+def test_varlen_large_batch_matches_the_fixed_length_kernels():
+    """Enough workgroups for the shared-buffer forward variant; equal lengths make the padded
+    batch call a second opinion, the ragged tail a check that short sequences leave their
+    neighbours' rows alone."""
+    H, D, dtype = 16, 128, torch.bfloat16
+    lengths = [1024] * 8 + [1000, 24]
+    T = sum(lengths)
+    q, k, v = (rand((T, H, D), 420 + i, dtype).to(DEV) for i in range(3))
+    cu = cu_of(lengths).to(DEV)
+    out, lse = ops.flash_fwd_varlen(q, k, v, cu, cu, 1024, 1024, None, True)
+    ref_out, ref_lse = ops.flash_fwd(q[:8192].view(8, 1024, H, D), k[:8192].view(8, 1024, H, D),
+                                     v[:8192].view(8, 1024, H, D), None, True)
+    assert torch.equal(out[:8192].view(8, 1024, H, D), ref_out)
+    assert torch.equal(lse[:, :8192].view(H, 8, 1024).transpose(0, 1), ref_lse)
+    for s0, n in ((8192, 1000), (9192, 24)):
+        o, l = ops.flash_fwd(q[None, s0:s0 + n], k[None, s0:s0 + n], v[None, s0:s0 + n], None, True)
+        check_out(out[s0:s0 + n], o[0].cpu(), dtype)
+        assert (lse[:, s0:s0 + n] - l[0]).abs().max() <= 1e-3
+
+
+def test_varlen_lse_helpers_round_trip():
+    """flatten_varlen_lse / unflatten_varlen_lse (sp_aurora/utils.py:150-169) against the packed lse."""
+    lengths, H, D = [30, 64, 7], 2, 64
+    T = sum(lengths)
+    q, k, v = (rand((T, H, D), 430 + i, torch.bfloat16).to(DEV) for i in range(3))
+    cu = cu_of(lengths).to(DEV)
+    _, lse, _ = spa.sp_aurora_varlen_func(q, k, v, cu, cu, max_seqlen=64, causal=True, return_attn_probs=True)
+    padded = spa.unflatten_varlen_lse(lse.t().unsqueeze(-1), cu, 64)     # [nseq, H, max]
+    assert padded.shape == (3, H, 64)
+    assert torch.equal(spa.flatten_varlen_lse(padded, cu), lse)
