@@ -5,7 +5,7 @@
 // (sp_aurora/intel_ring_flash_attn.py:192-258), which re-runs autograd on each block.
 //
 // Two kernels, no atomics, every output row has one owner (deterministic):
-//   dq kernel   : workgroup = 128 query rows (4 waves x 32), walks key tiles of 64.
+//   dq kernel   : workgroup = 128 or 256 query rows (4 or 8 waves x 32), walks key tiles of 64.
 //                 S^T = K Q^T and dP^T = V dO^T land with a lane owning one query row,
 //                 so lse/delta are per-lane scalars and dS^T is, register for register,
 //                 the B operand of dQ^T = K^T dS^T.
@@ -19,13 +19,15 @@
 // contractions) and, through the transposing read, columns (A operands K^T, Q^T, dO^T of the
 // gradient contractions).  No transposed copies exist.
 //
-// One wave per SIMD, software-pipelined inside the wave at half-tile (32 rows) granularity:
+// One wave per SIMD (the 8-wave dq kernel: two, which also halves the K/V traffic per query row),
+// software-pipelined inside the wave at half-tile (32 rows) granularity:
 // the MFMAs that produce S and dP of half-tile g+1 are interleaved, one to one, with the
 // element-wise work (exp, dS) on half-tile g, followed by the gradient MFMAs of half-tile g.
 // MFMA operands come from LDS through a rolling window that runs ahead of the MFMAs and is
 // carried across loop iterations; one workgroup barrier per 64-row tile.
 // Accumulators are fp32 in HBM and are ADDED to (read-modify-write by the owning lane).
 #include "spa_common.h"
+#include <stdlib.h>
 
 namespace {
 
@@ -35,13 +37,14 @@ constexpr int BWD_STAGES = 4;   // tiles resident or on their way
 constexpr int BWD_LOOK_MAX = 8; // operands are fetched from LDS up to this many MFMAs ahead
 constexpr unsigned OFF_NONE = 0x80000000u;  // a buffer offset beyond any tensor: the load stores zeros
 
-template <int D>
+template <int D, int THREADS = BWD_THREADS>
 struct BwdCfg {
   static constexpr int ROWB = D * 2;             // bytes per tile row
   static constexpr int TILEB = BWD_ROWS * ROWB;  // one tile
   static constexpr int CPR = D / 8;              // 16-byte chunks per row
-  static constexpr int NDMA = TILEB / (BWD_THREADS * 16);  // direct loads per thread and tile
-  static constexpr int RPD = BWD_THREADS / CPR;  // rows one round of the workgroup's loads covers
+  static constexpr int NDMA = TILEB / (THREADS * 16);  // direct loads per thread and tile
+  static_assert(NDMA >= 1, "a tile must give every thread at least one 16-byte slot");
+  static constexpr int RPD = THREADS / CPR;  // rows one round of the workgroup's loads covers
 };
 
 // Chunk permutation of a tile row, good for both read patterns: 16 consecutive rows at one chunk
@@ -78,13 +81,13 @@ struct TileReads {
 
 // Global side of the direct loads: thread tid owns 16-byte slot tid of every round of 256 slots;
 // round j covers rows j * RPD + tid / CPR.  Slot (row, pos) receives chunk pos ^ swizzle(row).
-template <typename T, int D>
+template <typename T, int D, int THREADS = BWD_THREADS>
 struct TileLoader {
   u32x4 rsrc;
   unsigned lane_off;  // bytes
   unsigned row_b;     // bytes per tensor row
   __device__ __forceinline__ void init(const T* base, int64_t row_stride, int rows, int tid) {
-    typedef BwdCfg<D> C;
+    typedef BwdCfg<D, THREADS> C;
     rsrc = buffer_descriptor(base, (unsigned)((((int64_t)rows - 1) * row_stride + D) * (int64_t)sizeof(T)));
     const int drow = tid / C::CPR, dpos = tid % C::CPR;
     lane_off = (unsigned)((drow * row_stride + ((dpos ^ tile_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(T));
@@ -92,9 +95,9 @@ struct TileLoader {
   }
   // round q of the tile whose first tensor row is row0 (on = false: store zeros) into LDS at lds_wave
   __device__ __forceinline__ void load(int q, bool on, int row0, unsigned lds_wave) const {
-    typedef BwdCfg<D> C;
+    typedef BwdCfg<D, THREADS> C;
     const unsigned u = on ? (unsigned)(row0 + q * C::RPD) * row_b : OFF_NONE;
-    load_to_lds_b128(rsrc, lane_off + u, lds_wave + q * (BWD_THREADS * 16));
+    load_to_lds_b128(rsrc, lane_off + u, lds_wave + q * (THREADS * 16));
   }
 };
 
@@ -125,9 +128,9 @@ __device__ __forceinline__ void wait_loads_but() {  // until at most N of this w
 // ------------------------------------------------------------------------------------------
 // dQ kernel
 // ------------------------------------------------------------------------------------------
-template <int D>
+template <int D, int NW = 4>
 struct DqCfg {
-  typedef BwdCfg<D> C;
+  typedef BwdCfg<D, NW * 64> C;
   static constexpr int STAGE = 2 * C::TILEB;  // K tile, V tile
   static constexpr int SMEM = BWD_STAGES * STAGE;
   static constexpr int NL = 2 * C::NDMA;      // loads per thread and stage
@@ -154,11 +157,11 @@ __device__ __forceinline__ void select_sequence(BwdParams& p, int& b) {
   b = 0;
 }
 
-template <typename T, int D>
-__global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dq_kernel(const BwdParams pk) {
+template <typename T, int D, int NW>
+__global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParams pk) {
   BwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
-  typedef BwdCfg<D> C;
-  typedef DqCfg<D> G;
+  typedef BwdCfg<D, NW * 64> C;
+  typedef DqCfg<D, NW> G;
   typedef Mma16<T> M;
   typedef typename M::frag frag;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -172,7 +175,7 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dq_kernel(const BwdP
   bid /= p.H;
   const int qt = p.nqt - 1 - (bid % p.nqt);
   int b = bid / p.nqt;
-  const int q0 = qt * 128;
+  const int q0 = qt * (NW * 32);
   const int qw0 = q0 + w * 32;
   select_sequence<T>(p, b);
   if (q0 >= p.Sq || p.Sk <= 0) return;  // (variable-length batches only) nothing to add to dq
@@ -197,10 +200,10 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dq_kernel(const BwdP
   const float c = p.scale_log2;
   const int lim = p.causal ? (qrow < p.Sk - 1 ? qrow : p.Sk - 1) : p.Sk - 1;  // last visible key
 
-  const int kv_end = p.causal ? (q0 + 128 < p.Sk ? q0 + 128 : p.Sk) : p.Sk;
+  const int kv_end = p.causal ? (q0 + NW * 32 < p.Sk ? q0 + NW * 32 : p.Sk) : p.Sk;
   const int nt = (kv_end + BWD_ROWS - 1) / BWD_ROWS;  // key tiles this workgroup visits
 
-  TileLoader<T, D> kld, vld;
+  TileLoader<T, D, NW * 64> kld, vld;
   kld.init(kp, p.ks.s, p.Sk, tid);
   vld.init(vp, p.vs.s, p.Sk, tid);
   TileReads<D> rd;
@@ -224,7 +227,8 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dq_kernel(const BwdP
   //   list 2i+1: S^T, dP^T of half 2i+2 (tile i+1, rows 0..31)  | dS^T of half 2i+1 | dQ of half 2i+1
   // NA MFMAs produce, the element-wise work rides between them, NB MFMAs consume.
   constexpr int NA = 2 * (D / 16), NB = 2 * (D / 32), NLIST = NA + NB, NBODY = 2 * NLIST;
-  constexpr int BWD_LOOK = NA < BWD_LOOK_MAX ? NA : BWD_LOOK_MAX;
+  constexpr int LOOK_CAP = NW == 8 ? 4 : BWD_LOOK_MAX;  // two waves per SIMD: 256 registers each, and the other wave covers LDS latency
+  constexpr int BWD_LOOK = NA < LOOK_CAP ? NA : LOOK_CAP;
   static_assert(NBODY % BWD_LOOK == 0 && BWD_LOOK <= NA, "the operand window must tile the loop body");
 
   issue_tile(0);
@@ -890,18 +894,37 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dkdv_kernel(const 
 }
 
 template <typename K>
-hipError_t launch(K kernel, int smem, unsigned blocks, const BwdParams& p, hipStream_t stream) {
+hipError_t launch(K kernel, int smem, unsigned blocks, const BwdParams& p, hipStream_t stream, int threads = BWD_THREADS) {
   hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(BWD_THREADS), smem, stream, p);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(threads), smem, stream, p);
   return hipGetLastError();
 }
 
 template <typename T, int D>
 hipError_t launch_both(const BwdParams& p, hipStream_t stream) {
-  const unsigned qblocks = (unsigned)((int64_t)p.B * p.H * p.nqt);
   const unsigned kblocks = (unsigned)((int64_t)p.B * p.H * p.nkt);
-  hipError_t e = launch(flash_bwd_dq_kernel<T, D>, DqCfg<D>::SMEM, qblocks, p, stream);
+  // dq kernel: 256-row workgroups (two waves per SIMD, the K/V stream shared by twice the rows) once
+  // there are enough of them to occupy every CU; SPA_BWD_DQ_WAVES=4|8 overrides (experiments, tests)
+  static const int cus = []() {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    return n;
+  }();
+  const int nqt8 = (p.Sq + 255) / 256;
+  const char* env = getenv("SPA_BWD_DQ_WAVES");
+  const int forced = env ? atoi(env) : 0;
+  hipError_t e = hipErrorInvalidValue;
+  bool wide = false;
+  if constexpr (D >= 64) {  // a D = 32 tile has fewer 16-byte slots than 512 threads
+    wide = forced ? forced == 8 : (int64_t)p.B * p.H * nqt8 >= cus;
+    if (wide) {
+      BwdParams p8 = p;
+      p8.nqt = nqt8;
+      e = launch(flash_bwd_dq_kernel<T, D, 8>, DqCfg<D, 8>::SMEM, (unsigned)((int64_t)p.B * p.H * nqt8), p8, stream, 512);
+    }
+  }
+  if (!wide) e = launch(flash_bwd_dq_kernel<T, D, 4>, DqCfg<D, 4>::SMEM, (unsigned)((int64_t)p.B * p.H * p.nqt), p, stream);
   if (e != hipSuccess) return e;
   return launch(flash_bwd_dkdv_kernel<T, D>, DkvCfg<D>::SMEM, kblocks, p, stream);
 }

@@ -366,6 +366,26 @@ def test_ring_backward_schedules_agree(causal):
         spa.ring.ring_flash_attn_backward(dd, qd, kd, vd, out, lse, None, causal, P, fuse="rank")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,S,H,D,causal", [(1, 300, 2, 128, True), (2, 515, 2, 64, True), (1, 256, 3, 32, False),
+                                            (1, 1000, 2, 128, False), (1, 77, 1, 128, True)])
+def test_dq_kernel_workgroup_sizes_agree(monkeypatch, B, S, H, D, causal, dtype):
+    """The dq kernel runs 128-row or 256-row workgroups depending on the grid; both orders of
+    accumulation are the same per row, so the gradients must be identical, and right."""
+    q, k, v, dout = rand_qkv((B, S, H, D), 140, dtype, n=4)
+    want = O.attn_backward_autograd(q, k, v, dout, None, causal)
+    got = {}
+    for waves in ("4", "8"):
+        monkeypatch.setenv("SPA_BWD_DQ_WAVES", waves)
+        xs = [t.to(DEV).requires_grad_(True) for t in (q, k, v)]
+        spa.ring_flash_attn_func(*xs, causal=causal).backward(dout.to(DEV))
+        got[waves] = [x.grad for x in xs]
+        for g, w, name in zip(got[waves], want, "qkv"):
+            check_grad(g, w, dtype, f"d{name} with {waves} waves")
+    for a, b in zip(got["4"], got["8"]):
+        assert torch.equal(a, b)
+
+
 def test_backward_packed_and_operator_entry():
     B, S, H, D = 1, 256, 2, 128
     qkv = rand((B, S, 3, H, D), 101, torch.bfloat16)
