@@ -26,6 +26,8 @@
 // MFMA operands come from LDS through a rolling window that runs ahead of the MFMAs and is
 // carried across loop iterations; one workgroup barrier per 64-row tile.
 // Accumulators are fp32 in HBM and are ADDED to (read-modify-write by the owning lane).
+// In the one-wave-per-SIMD kernels the MFMAs are written with their register files spelled out
+// (gradient accumulators in AGPRs, S / dP tiles in VGPRs), see MmaAsm.
 #include "spa_common.h"
 #include <stdlib.h>
 
@@ -125,6 +127,42 @@ __device__ __forceinline__ void wait_loads_but() {  // until at most N of this w
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
+// MFMAs with the accumulator's register file spelled out.  The compiler gives every MFMA of a
+// function the same form; the one-wave-per-SIMD kernels want both: the gradient accumulators
+// (touched by MFMAs only) in AGPRs, the S / dP tiles, which the VALU works on, in VGPRs, so that
+// no v_accvgpr_read / v_accvgpr_write copies are needed between the matrix pipe and the VALU.
+// The compiler does not see these as MFMAs: the code keeps the distances the hardware needs
+// (a VALU read of a tile comes at least 16 MFMAs after the tile's last MFMA; srcC is the
+// destination itself or the literal 0, never a register a VALU instruction has just written).
+template <typename T>
+struct MmaAsm;
+template <>
+struct MmaAsm<__bf16> {
+  typedef bf16x8 frag;
+  static __device__ __forceinline__ void first_v(f32x16& c, frag a, frag b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void acc_v(f32x16& c, frag a, frag b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void acc_a(f32x16& c, frag a, frag b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+};
+template <>
+struct MmaAsm<_Float16> {
+  typedef f16x8 frag;
+  static __device__ __forceinline__ void first_v(f32x16& c, frag a, frag b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void acc_v(f32x16& c, frag a, frag b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void acc_a(f32x16& c, frag a, frag b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+};
+
 // ------------------------------------------------------------------------------------------
 // dQ kernel
 // ------------------------------------------------------------------------------------------
@@ -163,6 +201,11 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
   typedef BwdCfg<D, NW * 64> C;
   typedef DqCfg<D, NW> G;
   typedef Mma16<T> M;
+  typedef MmaAsm<T> MA;
+  // one wave per SIMD: AGPRs are there for the dq accumulators.  D = 128 only: its 8 gradient
+  // MFMAs (with their operand reads) between a tile's last MFMA and the first VALU read of the
+  // tile give the matrix pipe the time it needs; the shorter lists of smaller D would not.
+  constexpr bool MIXED = NW == 4 && D == 128;
   typedef typename M::frag frag;
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -239,13 +282,27 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
 
   f32x16 sc, dc, sn, dn;  // S^T, dP^T of the current / next half-tile
   {
-    zero16(sc);
-    zero16(dc);
+    if (!MIXED) {
+      zero16(sc);
+      zero16(dc);
+    }
     const unsigned kb = stage_of(0);
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks) {
-      sc = M::run(as_frag<frag>(lds_read_b128(kb + rd.row[ks])), qf[ks], sc);
-      dc = M::run(as_frag<frag>(lds_read_b128(kb + C::TILEB + rd.row[ks])), dof[ks], dc);
+      const frag a0 = as_frag<frag>(lds_read_b128(kb + rd.row[ks]));
+      const frag a1 = as_frag<frag>(lds_read_b128(kb + C::TILEB + rd.row[ks]));
+      if (MIXED) {
+        if (ks == 0) {
+          MA::first_v(sc, a0, qf[0]);
+          MA::first_v(dc, a1, dof[0]);
+        } else {
+          MA::acc_v(sc, a0, qf[ks]);
+          MA::acc_v(dc, a1, dof[ks]);
+        }
+      } else {
+        sc = M::run(a0, qf[ks], sc);
+        dc = M::run(a1, dof[ks], dc);
+      }
     }
   }
 
@@ -300,8 +357,10 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
         for (int v = 0; v < 16; ++v)
           if (key0 + 8 * (v >> 2) + 4 * hh + (v & 3) > lim) sc[v] = -INFINITY;
       }
-      zero16(sn);
-      zero16(dn);
+      if (!MIXED) {
+        zero16(sn);
+        zero16(dn);
+      }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < NLIST; ++j) {
@@ -311,10 +370,17 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
         __builtin_amdgcn_sched_barrier(0);
         if (j < NA) {
           const int ks = j >> 1;
-          if (j & 1)
+          if (MIXED) {
+            if (j & 1) {
+              if (ks == 0) MA::first_v(dn, a, dof[0]); else MA::acc_v(dn, a, dof[ks]);
+            } else {
+              if (ks == 0) MA::first_v(sn, a, qf[0]); else MA::acc_v(sn, a, qf[ks]);
+            }
+          } else if (j & 1) {
             dn = M::run(a, dof[ks], dn);
-          else
+          } else {
             sn = M::run(a, qf[ks], sn);
+          }
           // element-wise work on the current half-tile, spread over the producing MFMAs
 #pragma unroll
           for (int v = 0; v < 16; ++v)
@@ -328,7 +394,10 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
         } else {
           const int jb = j - NA;
           const int db = jb % (D / 32), u = jb / (D / 32);
-          dq[db] = M::run(a, dsf[u], dq[db]);
+          if (MIXED)
+            MA::acc_a(dq[db], a, dsf[u]);
+          else
+            dq[db] = M::run(a, dsf[u], dq[db]);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -337,6 +406,7 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
     }
   }
   wait_loads_but<0>();  // nothing may still be writing LDS when the workgroup ends
+  if (MIXED) asm volatile("s_nop 15\n s_nop 15" ::: "memory");  // the last MFMAs must have written dq before it is read
 
   if (qrow < p.Sq) {
     float* dqp = p.dq + b * p.dqs.b + h * p.dqs.h + (int64_t)qrow * p.dqs.s;
@@ -373,6 +443,8 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
   typedef BwdCfg<D> C;
   typedef DkvCfg<D> G;
   typedef Mma16<T> M;
+  typedef MmaAsm<T> MA;
+  constexpr bool MIXED = D == 128;  // see the dq kernel; here 16 gradient MFMAs separate a tile's MFMAs from its VALU reads
   typedef typename M::frag frag;
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -456,13 +528,25 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
 
     f32x16 sc, dc, sn, dn;
     {
-      zero16(sc);
-      zero16(dc);
       const unsigned qb = stage_of(it0);
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks) {
-        sc = M::run(as_frag<frag>(lds_read_b128(qb + rd.row[ks])), kf[ks], sc);
-        dc = M::run(as_frag<frag>(lds_read_b128(qb + C::TILEB + rd.row[ks])), vf[ks], dc);
+        const frag a0 = as_frag<frag>(lds_read_b128(qb + rd.row[ks]));
+        const frag a1 = as_frag<frag>(lds_read_b128(qb + C::TILEB + rd.row[ks]));
+        if (!MIXED) {
+          if (ks == 0) {
+            zero16(sc);
+            zero16(dc);
+          }
+          sc = M::run(a0, kf[ks], sc);
+          dc = M::run(a1, vf[ks], dc);
+        } else if (ks == 0) {
+          MA::first_v(sc, a0, kf[0]);
+          MA::first_v(dc, a1, vf[0]);
+        } else {
+          MA::acc_v(sc, a0, kf[ks]);
+          MA::acc_v(dc, a1, vf[ks]);
+        }
       }
     }
 
@@ -530,8 +614,10 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
             de[4 * g4 + e] = d4[e];
           }
         }
-        zero16(sn);
-        zero16(dn);
+        if (!MIXED) {
+          zero16(sn);
+          zero16(dn);
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < NLIST; ++j) {
@@ -541,10 +627,16 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
           __builtin_amdgcn_sched_barrier(0);
           if (j < NA) {
             const int ks = j >> 1;
-            if (j & 1)
-              dn = M::run(a, vf[ks], dn);
-            else
-              sn = M::run(a, kf[ks], sn);
+            if (!MIXED) {
+              if (j & 1)
+                dn = M::run(a, vf[ks], dn);
+              else
+                sn = M::run(a, kf[ks], sn);
+            } else if (j & 1) {
+              if (ks == 0) MA::first_v(dn, a, vf[0]); else MA::acc_v(dn, a, vf[ks]);
+            } else {
+              if (ks == 0) MA::first_v(sn, a, kf[0]); else MA::acc_v(sn, a, kf[ks]);
+            }
 #pragma unroll
             for (int v = 0; v < 16; ++v)
               if (v * NA / 16 == j) {
@@ -563,10 +655,16 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
           } else {
             const int jb = j - NA;
             const int which = jb & 1, db = (jb >> 1) % (D / 32), u = (jb >> 1) / (D / 32);
-            if (which)
-              dk[db] = M::run(a, dsf[u], dk[db]);
-            else
-              dv[db] = M::run(a, pf[u], dv[db]);
+            if (!MIXED) {
+              if (which)
+                dk[db] = M::run(a, dsf[u], dk[db]);
+              else
+                dv[db] = M::run(a, pf[u], dv[db]);
+            } else if (which) {
+              MA::acc_a(dk[db], a, dsf[u]);
+            } else {
+              MA::acc_a(dv[db], a, pf[u]);
+            }
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -576,6 +674,8 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
     }
     wait_loads_but<0>();
   }
+  // the last MFMAs must have written dk / dv before they are read
+  if (MIXED) asm volatile("s_nop 15\n s_nop 15" ::: "memory");
 
   if (krow < p.Sk) {
     float* dkp = p.dk + b * p.dks.b + h * p.dks.h + (int64_t)krow * p.dks.s;
