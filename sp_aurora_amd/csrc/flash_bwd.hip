@@ -214,10 +214,10 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   int bid = blockIdx.x;
-  const int h = bid % p.H;
-  bid /= p.H;
-  const int qt = p.nqt - 1 - (bid % p.nqt);
-  int b = bid / p.nqt;
+  const int bh = bid % (p.B * p.H);  // (batch, head) pairs first: each keeps to one XCD also when H < 8
+  const int h = bh % p.H;
+  int b = bh / p.H;
+  const int qt = p.nqt - 1 - bid / (p.B * p.H);
   const int q0 = qt * (NW * 32);
   const int qw0 = q0 + w * 32;
   select_sequence<T>(p, b);
@@ -453,10 +453,10 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   int bid = blockIdx.x;
-  const int h = bid % p.H;
-  bid /= p.H;
-  const int kt = bid % p.nkt;  // causal: low key tiles see the most query tiles, they go first
-  int b = bid / p.nkt;
+  const int bh = bid % (p.B * p.H);  // (batch, head) pairs first: each keeps to one XCD also when H < 8
+  const int h = bh % p.H;
+  int b = bh / p.H;
+  const int kt = bid / (p.B * p.H);  // causal: low key tiles see the most query tiles, they go first
   const int k0 = kt * 128;
   const int kw0 = k0 + w * 32;
   select_sequence<T>(p, b);
@@ -759,10 +759,10 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dq_kernel(const Bw
   const int lane = tid & 63, w = tid >> 6, ln = lane & 31, hh = lane >> 5;
 
   int bid = blockIdx.x;
-  const int h = bid % p.H;
-  bid /= p.H;
-  const int qt = p.nqt - 1 - (bid % p.nqt);
-  int b = bid / p.nqt;
+  const int bh = bid % (p.B * p.H);  // (batch, head) pairs first: each keeps to one XCD also when H < 8
+  const int h = bh % p.H;
+  int b = bh / p.H;
+  const int qt = p.nqt - 1 - bid / (p.B * p.H);
   const int q0 = qt * 128;
   const int qw0 = q0 + w * 32;
   select_sequence<float>(p, b);
@@ -864,10 +864,10 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dkdv_kernel(const 
   const int lane = tid & 63, w = tid >> 6, ln = lane & 31, hh = lane >> 5;
 
   int bid = blockIdx.x;
-  const int h = bid % p.H;
-  bid /= p.H;
-  const int kt = bid % p.nkt;
-  int b = bid / p.nkt;
+  const int bh = bid % (p.B * p.H);  // (batch, head) pairs first: each keeps to one XCD also when H < 8
+  const int h = bh % p.H;
+  int b = bh / p.H;
+  const int kt = bid / (p.B * p.H);
   const int k0 = kt * 128;
   const int kw0 = k0 + w * 32;
   select_sequence<float>(p, b);

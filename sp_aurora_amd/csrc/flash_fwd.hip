@@ -94,16 +94,16 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const int ln = lane & 31;
   const int hh = lane >> 5;
 
-  // Consecutive workgroup ids walk the heads first: with round-robin placement of
+  // Consecutive workgroup ids walk the (batch, head) pairs first: with round-robin placement of
   // workgroups on the 8 XCDs, all query tiles of a head share one XCD's L2 for K/V.
   // Then query tiles and ranks, heaviest first.
   int bid = blockIdx.x;
-  const int h = bid % p.H;
-  bid /= p.H;
+  const int bh = bid % (p.B * p.H);  // (batch, head) pairs first: each keeps to one XCD also when H < 8
+  bid /= p.B * p.H;
+  const int h = bh % p.H;
+  int b = bh / p.H;
   const int qt = p.nqt - 1 - (bid % p.nqt);
-  bid /= p.nqt;
-  int b = bid % p.B;
-  const int rank = p.rank0 + p.nranks - 1 - bid / p.B;
+  const int rank = p.rank0 + p.nranks - 1 - bid / p.nqt;
   const int q0 = qt * C::BMW;
   if (p.cu_q) {
     const int q_lo = p.cu_q[b], k_lo = p.cu_k[b];
