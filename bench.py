@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ring-step attention hot path on one MI355X.
 
-Workload = BASELINE config 3: bf16, B=1, S=8192 in P=8 chunks of 1024, H=32, D=128, causal;
+Workload = benchmark config 3: bf16, B=1, S=8192 in P=8 chunks of 1024, H=32, D=128, causal;
 every rank's Q chunk against its prefix of KV chunks in ring order (8 diagonal + 28 full block
 pairs), partial results merged per step, cast at the end.  One "step" is that whole 36-pair
 sweep; inputs are resident in HBM before the timed region.  value = causal-adjusted TFLOP/s of
@@ -25,9 +25,9 @@ out + a second q k^T / logsumexp for lse, sp_aurora/intel_flash_attn_optimized.p
 the host cores, on diagonal + full block pairs of the same workload.
 
 `--workload` selects the other measured rows of the path instead (one JSON line each, same keys,
-`metric` named after the row): `relayout` = the Ulysses re-layout of BASELINE config 4 (HBM
+`metric` named after the row): `relayout` = the Ulysses re-layout of benchmark config 4 (HBM
 bound), `merge` = update_out_and_lse on one config-3 chunk (HBM bound), `backward` = the ring
-backward of BASELINE config 5 (MFMA bound), `ulysses` = the whole Ulysses forward of config 4.
+backward of benchmark config 5 (MFMA bound), `ulysses` = the whole Ulysses forward of config 4.
 
 Two helper modes for the HBM traffic figure (roofline.traffic):
   --traffic-leg          additionally runs a plain device copy of known size, so that a

@@ -33,7 +33,7 @@ def digest(*tensors):
 
 # name -> (seed, dtype, shape [B,S,H,D], input scale, causal, ring size, softmax scale)
 CASES = {
-    # BASELINE config 1: the reference's CPU-runnable case
+    # benchmark config 1: the reference's CPU-runnable case
     "cfg1_fp32_b1_s512_h8_d64": (0, torch.float32, (1, 512, 8, 64), 1.0, False, 1, 1.0 / 8.0),
     # known-answer procedure of test/flash_attention/test_flash_attention_simple.py:74-137
     "simple_fp32_b1_s64_h2_d32_causal": (42, torch.float32, (1, 64, 2, 32), 1.0, True, 1, None),

@@ -1,10 +1,10 @@
-"""GPU parity at BASELINE's full sizes (configs 2-5).
+"""GPU parity at the full sizes of benchmark configs 2-5.
 
 The float64 CPU oracle covers these shapes at reduced sizes in test_gpu_parity.py; here the HIP
 path runs at the full size and is checked
   * against a plain fp32 PyTorch evaluation on the same GPU of the same mathematics
     (softmax(q k^T scale + mask) v, logsumexp) for a sample of (batch, head) slices, to the
-    tolerances of BASELINE's north_star (bf16 out atol 2e-2 / rtol 1.6e-2, lse atol 1e-3,
+    stated tolerances (bf16 out atol 2e-2 / rtol 1.6e-2, lse atol 1e-3,
     gradients 3e-2 of the gradient's scale), and
   * against the float64 CPU oracle on a few dozen random query rows per config (which pins the
     on-device fp32 evaluation itself), and

@@ -1,6 +1,6 @@
 """GPU parity: the HIP path (through the C ABI) against the CPU oracle on the same seeded inputs.
 
-Tolerances (BASELINE north_star): fp32 out atol 1e-5; bf16 out atol 2e-2 / rtol 1.6e-2;
+Tolerances: fp32 out atol 1e-5; bf16 out atol 2e-2 / rtol 1.6e-2;
 lse atol 1e-3; re-layout bit-exact.  fp16 uses the bf16 bound (it is tighter in practice).
 The oracle computes in float64 from the inputs at their storage precision.
 """
@@ -142,7 +142,7 @@ GOLDEN_CASES = {
 
 @pytest.mark.parametrize("name", sorted(GOLDEN_CASES))
 def test_golden_fixture(name):
-    """Committed vectors (tests/golden/make_golden.py); cfg1_* is BASELINE config 1."""
+    """Committed vectors (tests/golden/make_golden.py); cfg1_* is benchmark config 1."""
     seed, dtype, shape, causal, P, scale = GOLDEN_CASES[name]
     fx = np.load(os.path.join(GOLDEN, name + ".npz"))
     q, k, v = rand_qkv(shape, seed, dtype)
@@ -223,7 +223,7 @@ def test_ring_equals_full_attention(P, causal, dtype):
 
 
 def test_ring_rank_follows_the_oracle_schedule():
-    """One rank's chunk against its KV chunks in ring order, as BASELINE config 2 (scaled down)."""
+    """One rank's chunk against its KV chunks in ring order, as benchmark config 2 (scaled down)."""
     P, B, s, H, D, rank = 4, 2, 96, 4, 64, 2
     q, k, v = rand_qkv((B, P * s, H, D), 71, torch.bfloat16)
     ks, vs = list(k.chunk(P, 1)), list(v.chunk(P, 1))
@@ -418,7 +418,7 @@ def test_delta_kernel():
 def test_ring_driver_matches_stepwise_path_and_oracle(causal, dtype):
     """spa_ring_fwd (merge fused into the kernel epilogue) against the step-by-step path through
     spa_flash_fwd + spa_merge + spa_finalize, and against the oracle's ring schedule; also a single
-    rank, as BASELINE config 2 runs it."""
+    rank, as benchmark config 2 runs it."""
     P, B, s, H, D = 4, 2, 160, 3, 64
     q, k, v = rand_qkv((B, P * s, H, D), 110, dtype)
     dq, dk, dv = q.to(DEV), k.to(DEV), v.to(DEV)
