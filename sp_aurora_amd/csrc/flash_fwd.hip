@@ -525,6 +525,37 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // waves walk the 128 x D tile row-major, add the groups' partials and write full rows:
   // 16-byte coalesced stores instead of 8-byte pieces scattered over 32 rows per wave.
   // A ring step's merge with the running (acc, lse) happens in the same pass (p.epi).
+  if (SHARE && p.epi == SPA_EPI_PLAIN) {
+    // A wave's rows are complete and nothing is merged: straight from the registers.  A lane holds
+    // 4 consecutive head dims per register group and its partner 32 lanes on the next 4; one
+    // v_permlane32_swap per dword pairs them up so that every lane stores 16-byte pieces, the two
+    // lanes of a row side by side.  No LDS round trip, no barrier.
+    const float l_tot = halves_sum(l_run);
+    const float inv = 1.f / l_tot;
+    if (hh == 0 && qrow < p.Sq)
+      p.lse[((int64_t)b * p.H + h) * p.lse_bh + qoff + qrow] = (m_run * c + fast_log2(l_tot)) * 0.6931471805599453f;
+    T* const orow = (T*)p.out + b * p.os.b + h * p.os.h + (qoff + qrow_c) * p.os.s;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int gp = 0; gp < 2; ++gp) {
+        unsigned x[2], y[2];  // this lane's 4 dims of the even and of the odd group, as two packed pairs each
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+          x[k] = M::pack2(o[db][8 * gp + 2 * k] * inv, o[db][8 * gp + 2 * k + 1] * inv);
+          y[k] = M::pack2(o[db][8 * gp + 4 + 2 * k] * inv, o[db][8 * gp + 4 + 2 * k + 1] * inv);
+        }
+        u32x4 st;
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+          const auto r = __builtin_amdgcn_permlane32_swap(x[k], y[k], false, false);
+          st[k] = r[0];      // lanes 0-31: own dims 0-3 of the even group; lanes 32-63: partner's dims 0-3 of the odd group
+          st[2 + k] = r[1];  // lanes 0-31: partner's dims 4-7 of the even group; lanes 32-63: own dims 4-7 of the odd group
+        }
+        if (qrow < p.Sq) *(u32x4*)(orow + db * 32 + 8 * (2 * gp + hh)) = st;
+      }
+    return;
+  }
   constexpr int TP = D + 4;  // floats per staged row
   float* const tile = (float*)smem + grp * (FWD_BM * TP);
   float* const ml = (float*)smem + NG * FWD_BM * TP;  // [NG][128](m, l), then lse_b[rows of the workgroup]
