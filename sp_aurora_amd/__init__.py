@@ -17,7 +17,19 @@ from .flash_attn import (  # noqa: F401
     intel_flash_attn_forward,
     is_available,
 )
-from .layers import AttnType, LongContextAttention, UlyssesAttention, select_flash_attn_impl  # noqa: F401
+from .layers import (  # noqa: F401
+    HAS_FLASH_ATTN,
+    HAS_LONG_CTX_ATTN,
+    HAS_SPARSE_SAGE_ATTENTION,
+    AttnType,
+    LongContextAttention,
+    UlyssesAttention,
+    pytorch_attn_forward,
+    pytorch_attn_func,
+    ring_pytorch_attn_forward,
+    ring_pytorch_attn_func,
+    select_flash_attn_impl,
+)
 from .ring import (  # noqa: F401
     IntelRingFlashAttnFunc,
     RingFlashAttnFunc,
@@ -51,5 +63,7 @@ from .ulysses import (  # noqa: F401
 )
 from .utils import flatten_varlen_lse, unflatten_varlen_lse, update_out_and_lse  # noqa: F401
 from .varlen import VarlenFlashAttnFunc, ring_flash_attn_varlen_func, sp_aurora_varlen_func  # noqa: F401
+
+SeqAllToAll4D_v2 = SeqAllToAll4D  # sp_aurora/__init__.py:77
 
 __version__ = "0.1.0"

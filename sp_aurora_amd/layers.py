@@ -20,7 +20,14 @@ from .flash_attn import _check_unsupported
 from .ring import _no_multi_gpu, ring_flash_attn_func
 from .ulysses import SeqAllToAll4D, ulysses_flash_attn_func
 
-__all__ = ["AttnType", "select_flash_attn_impl", "UlyssesAttention", "LongContextAttention"]
+__all__ = ["AttnType", "select_flash_attn_impl", "UlyssesAttention", "LongContextAttention", "pytorch_attn_forward",
+           "pytorch_attn_func", "ring_pytorch_attn_func", "ring_pytorch_attn_forward", "HAS_LONG_CTX_ATTN",
+           "HAS_FLASH_ATTN", "HAS_SPARSE_SAGE_ATTENTION"]
+
+# sp_aurora/globals.py:171-173
+HAS_LONG_CTX_ATTN = True
+HAS_FLASH_ATTN = True
+HAS_SPARSE_SAGE_ATTENTION = False
 
 
 class AttnType(str, Enum):
@@ -41,6 +48,43 @@ def _local_attention(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, w
     res = ring_flash_attn_func(q, k, v, dropout_p, softmax_scale, causal, window_size, alibi_slopes,
                                deterministic, return_attn_probs, None, ring_size=1)
     return res[:2] if return_attn_probs else res
+
+
+def pytorch_attn_forward(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, window_size=(-1, -1), softcap=0.0,
+                         alibi_slopes=None, deterministic=False, return_attn_probs=False):
+    """sp_aurora/kernels/attention.py:12-86 with its documented layout (batch, seq_len, num_heads,
+    head_dim): -> (out, None).  The reference's second value is the materialised S x S probability
+    matrix, which these kernels never form: return_attn_probs raises."""
+    if return_attn_probs:
+        raise NotImplementedError("the attention probabilities are not materialised")
+    return _local_attention(q, k, v, dropout_p, softmax_scale, causal, window_size, softcap, alibi_slopes,
+                            deterministic, False), None
+
+
+def pytorch_attn_func(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, window_size=(-1, -1), softcap=0.0,
+                      alibi_slopes=None, deterministic=False, return_attn_probs=False):
+    """sp_aurora/kernels/attention.py:89-117: the output of pytorch_attn_forward."""
+    return pytorch_attn_forward(q, k, v, dropout_p, softmax_scale, causal, window_size, softcap, alibi_slopes,
+                                deterministic, return_attn_probs)[0]
+
+
+def ring_pytorch_attn_func(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, window_size=(-1, -1),
+                           alibi_slopes=None, deterministic=False, return_attn_probs=False, group=None, *, ring_size=1):
+    """sp_aurora/ring_pytorch_attn.py:20-197, the reference's second ring implementation: the same
+    result as ring_flash_attn_func, through the same kernels."""
+    out = ring_flash_attn_func(q, k, v, dropout_p, softmax_scale, causal, window_size, alibi_slopes, deterministic,
+                               return_attn_probs, group, ring_size=ring_size)
+    return out[:2] if return_attn_probs else out
+
+
+def ring_pytorch_attn_forward(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, window_size=(-1, -1),
+                              alibi_slopes=None, deterministic=False, return_attn_probs=False, group=None, *,
+                              ring_size=1):
+    """sp_aurora/ring_pytorch_attn.py:200-226: -> (out, lse); the reference returns None for the lse
+    unless return_attn_probs, this returns the fp32 [B,H,S] lse either way."""
+    out, lse, _ = ring_flash_attn_func(q, k, v, dropout_p, softmax_scale, causal, window_size, alibi_slopes,
+                                       deterministic, True, group, ring_size=ring_size)
+    return out, lse
 
 
 def select_flash_attn_impl(attn_type):

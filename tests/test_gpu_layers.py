@@ -91,3 +91,23 @@ def test_layer_argument_contract():
     with pytest.raises(ValueError):
         spa.LongContextAttention(sp_ulysses_degree=8, sp_ring_degree=1)(
             torch.zeros(8, 1, 8, 4, 64, device=DEV, dtype=torch.bfloat16), q, q)  # 4 heads over 8 ranks
+
+
+def test_second_implementation_names_reach_the_same_kernels():
+    """pytorch_attn_* (sp_aurora/kernels/attention.py) and ring_pytorch_attn_* (sp_aurora/ring_pytorch_attn.py)."""
+    B, S, H, D = 2, 96, 4, 64
+    q, k, v = rand_qkv((B, S, H, D), 330, torch.bfloat16)
+    want, want_lse = O.full_attention(q, k, v, None, True)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    out, probs = spa.pytorch_attn_forward(qd, kd, vd, causal=True)
+    assert probs is None
+    check_out(out, want, torch.bfloat16)
+    assert torch.equal(spa.pytorch_attn_func(qd, kd, vd, causal=True), out)
+    out2, lse2 = spa.ring_pytorch_attn_forward(qd, kd, vd, causal=True, ring_size=3)
+    check_out(out2, want, torch.bfloat16)
+    assert (lse2.cpu().double() - want_lse).abs().max() <= 1e-3
+    assert torch.equal(spa.ring_pytorch_attn_func(qd, kd, vd, causal=True, ring_size=3), out2)
+    with pytest.raises(NotImplementedError):
+        spa.pytorch_attn_forward(qd, kd, vd, return_attn_probs=True)
+    assert spa.HAS_LONG_CTX_ATTN and spa.HAS_FLASH_ATTN and not spa.HAS_SPARSE_SAGE_ATTENTION
+    assert spa.SeqAllToAll4D_v2 is spa.SeqAllToAll4D
