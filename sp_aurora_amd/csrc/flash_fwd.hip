@@ -477,17 +477,23 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // of its VALU phase; each waits for its loads before the barrier two phases later.
   const bool early = SHARE && grp == 1;  // wave-uniform
   Cursor cs = cursor_at(0), cv = cursor_at(1), ck = cursor_at(2);
-  for (int i = 0; i + 1 < n; ++i) {
+  // The loop body comes in two copies, one per buffer parity of the step, so that every LDS address of
+  // the MFMA phase is a per-lane constant plus an immediate offset (no address arithmetic per step).
+  auto body = [&](auto parity, int i) __attribute__((always_inline)) {
+    constexpr int PAR = decltype(parity)::value;  // == i & 1
     frag pf[2][2];
     const bool kon = ck.i < n, von = cv.i < n;
-    const unsigned kb = k_lds(i), vb = v_lds(i + 1);
+    constexpr unsigned kb = (unsigned)(PAR * C::TILEB), vb = (unsigned)(2 * C::TILEB + (PAR ^ 1) * C::TILEB);  // k_lds(i), v_lds(i + 1)
     if (early) {
 #pragma unroll
       for (int q = 0; q < NLOADS; ++q) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb);
     }
     softmax_phase(cs.sb, pf);
     unsigned va[D / 32], ka[D / 16];
-    operand_addresses(i, va, ka);
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db) va[db] = vra[db] + (unsigned)(2 * C::TILEB + PAR * C::TILEB);  // v_lds(i)
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) ka[ks] = kra[ks] + (unsigned)((PAR ^ 1) * C::TILEB);            // k_lds(i + 1)
     // Shared buffers need one barrier per step and group (after the wait for the loads: group 0
     // at the end of its VALU phase, group 1 at the end of its MFMA phase, the same physical
     // barrier); the other one only holds the two groups in step, and they drift little without it.
@@ -506,6 +512,14 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     cursor_next(ck);
     if (early) loads_landed();
     if (!SHARE || early) __syncthreads();
+  };
+  {
+    int i = 0;
+    for (; i + 2 < n; i += 2) {
+      body(std::integral_constant<int, 0>{}, i);
+      body(std::integral_constant<int, 1>{}, i + 1);
+    }
+    if (i + 1 < n) body(std::integral_constant<int, 0>{}, i);
   }
   {  // last sub-tile: nothing to prepare behind it
     frag pf[2][2];
