@@ -16,18 +16,15 @@ FLAGS = [
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     # packed fp32 VALU ops are kept off on purpose (scalar fp32 code only)
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+# per-file additions: the forward kernels' softmax phase gains 1-3 % from the scheduler that
+# maximises instruction-level parallelism; the backward kernels lose 2 % with it
+EXTRA = {"flash_fwd.hip": ["-mllvm", "-amdgpu-sched-strategy=max-ilp"]}
 
 
-def build(verbose: bool = True) -> str:
-    """Compile every HIP source into sp_aurora_amd/libsp_aurora_hip.so and return its path."""
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    if not os.path.exists(hipcc):
-        hipcc = "hipcc"
-    cmd = [hipcc] + FLAGS + ["-o", LIB_PATH] + [os.path.join(CSRC, s) for s in SOURCES]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -36,6 +33,21 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out:
         print(out)
+
+
+def build(verbose: bool = True) -> str:
+    """Compile every HIP source into sp_aurora_amd/libsp_aurora_hip.so and return its path."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    if not os.path.exists(hipcc):
+        hipcc = "hipcc"
+    objdir = os.path.join(HERE, "_obj")
+    os.makedirs(objdir, exist_ok=True)
+    objs = []
+    for src in SOURCES:
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        _run([hipcc] + FLAGS + EXTRA.get(src, []) + ["-c", "-o", obj, os.path.join(CSRC, src)], verbose)
+        objs.append(obj)
+    _run([hipcc, "--offload-arch=gfx950", "-fPIC", "-shared", "-o", LIB_PATH] + objs, verbose)
     return LIB_PATH
 
 
