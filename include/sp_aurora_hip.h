@@ -110,10 +110,13 @@ int spa_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* 
  *                       accumulators in registers and walks the rank's KV chunks in ring order,
  *                       so the merge is the online softmax itself and no accumulator leaves the CU.
  *   SPA_RING_ALL_RANKS  one launch for all requested ranks (heaviest first).
- * fp32 always runs per step.  No collectives: the "ring" is the order in which chunks are visited.
+ * fp32 always runs per step, whatever `fuse` says.  No collectives: the "ring" is the order in
+ * which chunks are visited.
  * workspace: device scratch of spa_ring_fwd_workspace_bytes() bytes (16-byte aligned), owned
- * by the caller; it holds the fp32 running output of one rank between separate step launches
- * (may be NULL for the fused modes).
+ * by the caller; it holds the fp32 running output of one rank between separate step launches.
+ * It may be NULL only when no launch needs it: 16-bit types in the fused modes, or a schedule in
+ * which no rank visits more than one block (P = 1; causal rank 0).  fp32 inputs with more than
+ * one block per rank always need it (SPA_EINVAL otherwise).
  */
 enum { SPA_RING_PER_STEP = 0, SPA_RING_PER_RANK = 1, SPA_RING_ALL_RANKS = 2 };
 int64_t spa_ring_fwd_workspace_bytes(int B, int H, int S, int D, int P, int dtype);
@@ -220,6 +223,18 @@ int spa_flash_bwd_varlen(const void* q, const void* k, const void* v, const void
                          const int64_t dq_strides[2], const int64_t dk_strides[2],
                          const int64_t dv_strides[2],
                          float scale, int mask_mode, int dtype, void* stream);
+
+/*
+ * Kernel-variant override for experiments and tests; no counterpart in the reference and not
+ * needed in production (value 0 restores the library's own choice).  Process-wide.
+ *   SPA_TUNE_FWD_GROUPS    1 | 2   wave groups per forward workgroup
+ *   SPA_TUNE_FWD_SHARE     1 | 2   1 = 128-row workgroups, private K/V buffers per wave group;
+ *                                  2 = 256-row workgroups sharing one set of buffers
+ *   SPA_TUNE_BWD_DQ_WAVES  4 | 8   waves per workgroup of the backward's dq kernel
+ *   SPA_TUNE_BWD_DKDV_FORM 1       compiler-scheduled MFMAs in the D = 128 dk/dv kernel
+ */
+enum { SPA_TUNE_FWD_GROUPS = 0, SPA_TUNE_FWD_SHARE = 1, SPA_TUNE_BWD_DQ_WAVES = 2, SPA_TUNE_BWD_DKDV_FORM = 3 };
+int spa_tune(int knob, int value);
 
 #ifdef __cplusplus
 }

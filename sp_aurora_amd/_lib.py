@@ -27,6 +27,7 @@ SIGNATURES = {
     "spa_flash_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _vp]),
     "spa_ring_fwd_workspace_bytes": (ctypes.c_int64, [_i, _i, _i, _i, _i, _i]),
     "spa_ring_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _i, _vp]),
+    "spa_tune": (_i, [_i, _i]),
     "spa_merge": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _s3, _s3, _i, _i, _vp]),
     "spa_finalize": (_i, [_vp, _vp, _i, _i, _i, _i, _s3, _s3, _i, _vp]),
     "spa_relayout_s2h": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
@@ -80,6 +81,14 @@ def strides2(vals):
 def check(code):
     if code != 0:
         raise SpaError(code, load().spa_last_error().decode("utf-8", "replace"))
+
+
+TUNE_KNOBS = {"fwd_groups": 0, "fwd_share": 1, "bwd_dq_waves": 2, "bwd_dkdv_form": 3}
+
+
+def tune(knob, value):
+    """Kernel-variant override for experiments and tests (spa_tune); value 0 = the library's choice."""
+    check(load().spa_tune(TUNE_KNOBS[knob], int(value)))
 
 
 def device_info():

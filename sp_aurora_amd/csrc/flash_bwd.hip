@@ -29,6 +29,7 @@
 // In the one-wave-per-SIMD kernels the MFMAs are written with their register files spelled out
 // (gradient accumulators in AGPRs, S / dP tiles in VGPRs), see MmaAsm.
 #include "spa_common.h"
+#include "spa_host.h"
 #include <stdlib.h>
 
 namespace {
@@ -993,9 +994,9 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dkdv_kernel(const 
   }
 }
 
-template <typename K>
-hipError_t launch(K kernel, int smem, unsigned blocks, const BwdParams& p, hipStream_t stream, int threads = BWD_THREADS) {
-  hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+template <auto kernel>
+hipError_t launch(int smem, unsigned blocks, const BwdParams& p, hipStream_t stream, int threads = BWD_THREADS) {
+  const hipError_t e = spa_allow_dynamic_lds<kernel>(smem);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(threads), smem, stream, p);
   return hipGetLastError();
@@ -1005,28 +1006,22 @@ template <typename T, int D>
 hipError_t launch_both(const BwdParams& p, hipStream_t stream) {
   const unsigned kblocks = (unsigned)((int64_t)p.B * p.H * p.nkt);
   // dq kernel: 256-row workgroups (two waves per SIMD, the K/V stream shared by twice the rows) once
-  // there are enough of them to occupy every CU; SPA_BWD_DQ_WAVES=4|8 overrides (experiments, tests)
-  static const int cus = []() {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    return n;
-  }();
+  // there are enough of them to occupy every CU; spa_tune() can force 4 or 8 waves (experiments, tests)
   const int nqt8 = (p.Sq + 255) / 256;
-  const char* env = getenv("SPA_BWD_DQ_WAVES");
-  const int forced = env ? atoi(env) : 0;
+  const int forced = spa_knob(SPA_KNOB_BWD_DQ_WAVES);
   hipError_t e = hipErrorInvalidValue;
   bool wide = false;
   if constexpr (D >= 64) {  // a D = 32 tile has fewer 16-byte slots than 512 threads
-    wide = forced ? forced == 8 : (int64_t)p.B * p.H * nqt8 >= cus;
+    wide = forced ? forced == 8 : (int64_t)p.B * p.H * nqt8 >= spa_device_cus();
     if (wide) {
       BwdParams p8 = p;
       p8.nqt = nqt8;
-      e = launch(flash_bwd_dq_kernel<T, D, 8>, DqCfg<D, 8>::SMEM, (unsigned)((int64_t)p.B * p.H * nqt8), p8, stream, 512);
+      e = launch<flash_bwd_dq_kernel<T, D, 8>>(DqCfg<D, 8>::SMEM, (unsigned)((int64_t)p.B * p.H * nqt8), p8, stream, 512);
     }
   }
-  if (!wide) e = launch(flash_bwd_dq_kernel<T, D, 4>, DqCfg<D, 4>::SMEM, (unsigned)((int64_t)p.B * p.H * p.nqt), p, stream);
+  if (!wide) e = launch<flash_bwd_dq_kernel<T, D, 4>>(DqCfg<D, 4>::SMEM, (unsigned)((int64_t)p.B * p.H * p.nqt), p, stream);
   if (e != hipSuccess) return e;
-  return launch(flash_bwd_dkdv_kernel<T, D>, DkvCfg<D>::SMEM, kblocks, p, stream);
+  return launch<flash_bwd_dkdv_kernel<T, D>>(DkvCfg<D>::SMEM, kblocks, p, stream);
 }
 
 }  // namespace
@@ -1047,13 +1042,13 @@ hipError_t spa_launch_flash_bwd(BwdParams p, int D, int dtype, hipStream_t strea
     const unsigned qblocks = (unsigned)((int64_t)p.B * p.H * p.nqt);
     const unsigned kblocks = (unsigned)((int64_t)p.B * p.H * p.nkt);
     hipError_t e = hipErrorInvalidValue;
-    if (D == 128) e = launch(flash_bwd32_dq_kernel<128>, Bwd32Cfg<128>::SMEM_DQ, qblocks, p, stream);
-    if (D == 64) e = launch(flash_bwd32_dq_kernel<64>, Bwd32Cfg<64>::SMEM_DQ, qblocks, p, stream);
-    if (D == 32) e = launch(flash_bwd32_dq_kernel<32>, Bwd32Cfg<32>::SMEM_DQ, qblocks, p, stream);
+    if (D == 128) e = launch<flash_bwd32_dq_kernel<128>>(Bwd32Cfg<128>::SMEM_DQ, qblocks, p, stream);
+    if (D == 64) e = launch<flash_bwd32_dq_kernel<64>>(Bwd32Cfg<64>::SMEM_DQ, qblocks, p, stream);
+    if (D == 32) e = launch<flash_bwd32_dq_kernel<32>>(Bwd32Cfg<32>::SMEM_DQ, qblocks, p, stream);
     if (e != hipSuccess) return e;
-    if (D == 128) return launch(flash_bwd32_dkdv_kernel<128>, Bwd32Cfg<128>::SMEM_DKV, kblocks, p, stream);
-    if (D == 64) return launch(flash_bwd32_dkdv_kernel<64>, Bwd32Cfg<64>::SMEM_DKV, kblocks, p, stream);
-    if (D == 32) return launch(flash_bwd32_dkdv_kernel<32>, Bwd32Cfg<32>::SMEM_DKV, kblocks, p, stream);
+    if (D == 128) return launch<flash_bwd32_dkdv_kernel<128>>(Bwd32Cfg<128>::SMEM_DKV, kblocks, p, stream);
+    if (D == 64) return launch<flash_bwd32_dkdv_kernel<64>>(Bwd32Cfg<64>::SMEM_DKV, kblocks, p, stream);
+    if (D == 32) return launch<flash_bwd32_dkdv_kernel<32>>(Bwd32Cfg<32>::SMEM_DKV, kblocks, p, stream);
   }
   return hipErrorInvalidValue;
 }

@@ -30,11 +30,10 @@
 //   separated by workgroup barriers, and group 1 runs one barrier behind group 0, so at
 //   any time one wave of a SIMD is in its MFMA phase while its neighbour is in its VALU
 //   phase (ping-pong).  The groups' partial (O, m, l) are combined through LDS at the end.
-#include <stdlib.h>
-
 #include <type_traits>
 
 #include "spa_common.h"
+#include "spa_host.h"
 
 namespace {
 
@@ -885,9 +884,9 @@ __global__ void __launch_bounds__(FWD_THREADS, 1) flash_fwd32_kernel(const FwdPa
   }
 }
 
-template <typename K>
-hipError_t launch(K kernel, int threads, int smem, const FwdParams& p, hipStream_t stream) {
-  hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+template <auto kernel>
+hipError_t launch(int threads, int smem, const FwdParams& p, hipStream_t stream) {
+  const hipError_t e = spa_allow_dynamic_lds<kernel>(smem);
   if (e != hipSuccess) return e;
   const dim3 grid((unsigned)((int64_t)p.B * p.H * p.nqt * p.nranks));
   hipLaunchKernelGGL(kernel, grid, dim3(threads), smem, stream, p);
@@ -895,31 +894,24 @@ hipError_t launch(K kernel, int threads, int smem, const FwdParams& p, hipStream
 }
 
 // Two wave groups once there are at least two 64-key sub-tiles to split; 256-row workgroups with
-// shared K/V buffers once that still leaves every CU at least two workgroups.
+// shared K/V buffers once that still leaves every CU at least two workgroups.  spa_tune() can
+// force either choice (experiments and tests).
 template <typename T, int D>
 hipError_t launch16(FwdParams p, hipStream_t stream) {
-  // overrides for experiments and tests, read at every launch: SPA_FWD_GROUPS=1|2, SPA_FWD_SHARE=0|1
-  const char* eg = getenv("SPA_FWD_GROUPS");
-  const char* es = getenv("SPA_FWD_SHARE");
-  const int force = eg ? atoi(eg) : 0;
-  const int force_share = es ? atoi(es) : -1;
-  static const int cus = []() {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    return n;
-  }();
+  const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
+  const int force_share = spa_knob(SPA_KNOB_FWD_SHARE);
   const bool two = force ? force == 2 : p.Sk > FWD_BN;
   if (two && D >= 64) {
     const int nqt2 = (p.Sq + 2 * FWD_BM - 1) / (2 * FWD_BM);
     const int64_t wgs = (int64_t)p.B * p.H * nqt2 * p.nranks;
-    const bool share = force_share >= 0 ? force_share != 0 : wgs >= 2 * (int64_t)cus;
+    const bool share = force_share ? force_share == 2 : wgs >= 2 * (int64_t)spa_device_cus();
     if (share) {
       p.nqt = nqt2;
-      return launch(flash_fwd16_kernel<T, D, 2, (D >= 64)>, 2 * FWD_THREADS, Fwd16Cfg<D, 2, (D >= 64)>::SMEM, p, stream);
+      return launch<flash_fwd16_kernel<T, D, 2, (D >= 64)>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, (D >= 64)>::SMEM, p, stream);
     }
   }
-  if (two) return launch(flash_fwd16_kernel<T, D, 2, false>, 2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
-  return launch(flash_fwd16_kernel<T, D, 1, false>, FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+  if (two) return launch<flash_fwd16_kernel<T, D, 2, false>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+  return launch<flash_fwd16_kernel<T, D, 1, false>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
 }
 
 }  // namespace
@@ -937,9 +929,9 @@ hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t strea
     if (D == 32) return launch16<_Float16, 32>(p, stream);
   } else if (dtype == 0) {
     if (p.epi != SPA_EPI_PLAIN) return hipErrorInvalidValue;  // fp32 ring steps merge with the separate kernel
-    if (D == 128) return launch(flash_fwd32_kernel<128>, FWD_THREADS, Fwd32Cfg<128>::SMEM, p, stream);
-    if (D == 64) return launch(flash_fwd32_kernel<64>, FWD_THREADS, Fwd32Cfg<64>::SMEM, p, stream);
-    if (D == 32) return launch(flash_fwd32_kernel<32>, FWD_THREADS, Fwd32Cfg<32>::SMEM, p, stream);
+    if (D == 128) return launch<flash_fwd32_kernel<128>>(FWD_THREADS, Fwd32Cfg<128>::SMEM, p, stream);
+    if (D == 64) return launch<flash_fwd32_kernel<64>>(FWD_THREADS, Fwd32Cfg<64>::SMEM, p, stream);
+    if (D == 32) return launch<flash_fwd32_kernel<32>>(FWD_THREADS, Fwd32Cfg<32>::SMEM, p, stream);
   }
   return hipErrorInvalidValue;
 }

@@ -7,6 +7,9 @@
 
 #include "../../include/sp_aurora_hip.h"
 #include "spa_common.h"
+#include "spa_host.h"
+
+std::atomic<int> g_spa_knob[SPA_KNOB_COUNT];
 
 hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream);
 hipError_t spa_launch_flash_bwd(BwdParams p, int D, int dtype, hipStream_t stream);
@@ -147,34 +150,42 @@ int64_t spa_ring_fwd_workspace_bytes(int B, int H, int S, int D, int P, int dtyp
   return 2 * acc + (int64_t)B * H * s * 4;
 }
 
-int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace, int B,
-                 int H, int S, int D, int P, int rank, const int64_t q_strides[3], const int64_t k_strides[3],
-                 const int64_t v_strides[3], const int64_t o_strides[3], float scale, int mask_mode, int dtype,
-                 int fuse, void* stream) {
-  if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "spa_ring_fwd: null pointer");
-  if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(SPA_EINVAL, "spa_ring_fwd: null strides");
-  if (!dims_ok(B, H, S, D)) return fail(SPA_EINVAL, "spa_ring_fwd: sizes must be positive");
-  if (P <= 0 || S % P != 0) return fail(SPA_EINVAL, "spa_ring_fwd: ring size %d must divide the sequence length %d", P, S);
-  if (rank < -1 || rank >= P) return fail(SPA_EINVAL, "spa_ring_fwd: rank %d outside [-1, %d)", rank, P);
-  if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "spa_ring_fwd: bad dtype %d", dtype);
-  if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "spa_ring_fwd: bad mask_mode %d", mask_mode);
-  if (fuse < SPA_RING_PER_STEP || fuse > SPA_RING_ALL_RANKS) return fail(SPA_EINVAL, "spa_ring_fwd: bad fuse mode %d", fuse);
-  if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "spa_ring_fwd: softmax scale must be positive and finite");
-  if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "spa_ring_fwd: head dim %d not in {32,64,128}", D);
+}  // extern "C"
+
+namespace {
+
+// `what` names the entry point in messages; `ws_bytes` < 0: the caller vouches for the workspace size.
+int ring_fwd(const char* what, const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
+             int64_t ws_bytes, int B, int H, int S, int D, int P, int rank, const int64_t q_strides[3],
+             const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3], float scale,
+             int mask_mode, int dtype, int fuse, void* stream) {
+  if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "%s: null pointer", what);
+  if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(SPA_EINVAL, "%s: null strides", what);
+  if (!dims_ok(B, H, S, D)) return fail(SPA_EINVAL, "%s: sizes must be positive", what);
+  if (P <= 0 || S % P != 0) return fail(SPA_EINVAL, "%s: ring size %d must divide the sequence length %d", what, P, S);
+  if (rank < -1 || rank >= P) return fail(SPA_EINVAL, "%s: rank %d outside [-1, %d)", what, rank, P);
+  if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "%s: bad dtype %d", what, dtype);
+  if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "%s: bad mask_mode %d", what, mask_mode);
+  if (fuse < SPA_RING_PER_STEP || fuse > SPA_RING_ALL_RANKS) return fail(SPA_EINVAL, "%s: bad fuse mode %d", what, fuse);
+  if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "%s: softmax scale must be positive and finite", what);
+  if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "%s: head dim %d not in {32,64,128}", what, D);
   const int esz = elem_size(dtype);
   if (!aligned16(q, q_strides, esz) || !aligned16(k, k_strides, esz) || !aligned16(v, v_strides, esz) ||
       !aligned16(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0 || ((uintptr_t)workspace & 15) != 0)
-    return fail(SPA_EALIGN, "spa_ring_fwd: pointers and row strides must be 16-byte aligned");
+    return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned", what);
   if (!span_ok(S, k_strides[2], D, esz) || !span_ok(S, v_strides[2], D, esz))
-    return fail(SPA_EUNSUPPORTED, "spa_ring_fwd: K/V of one (batch, head) span more than 2 GiB");
+    return fail(SPA_EUNSUPPORTED, "%s: K/V of one (batch, head) span more than 2 GiB", what);
   const bool causal = mask_mode == SPA_MASK_CAUSAL;
   const int s = S / P;
   if (dtype == SPA_F32) fuse = SPA_RING_PER_STEP;  // the fp32 kernel handles one block pair per launch
   const bool multi = P > 1 && (!causal || rank != 0);  // does some rank visit more than one block?
   if (fuse == SPA_RING_PER_STEP && multi && !workspace)
-    return fail(SPA_EINVAL, "spa_ring_fwd: workspace required when steps are separate launches");
+    return fail(SPA_EINVAL, "%s: workspace required when steps are separate launches", what);
+  if (fuse == SPA_RING_PER_STEP && multi && ws_bytes >= 0 && spa_ring_fwd_workspace_bytes(B, H, S, D, P, dtype) > ws_bytes)
+    return fail(SPA_EINVAL, "%s: these sizes need %lld bytes of scratch, the built-in buffer holds %lld", what,
+                (long long)spa_ring_fwd_workspace_bytes(B, H, S, D, P, dtype), (long long)ws_bytes);
   const int r_lo = rank < 0 ? 0 : rank, r_hi = rank < 0 ? P : rank + 1;
-  if ((int64_t)B * H * ((s + 127) / 128) * (r_hi - r_lo) > 0x7fffffffLL) return fail(SPA_EINVAL, "spa_ring_fwd: grid too large");
+  if ((int64_t)B * H * ((s + 127) / 128) * (r_hi - r_lo) > 0x7fffffffLL) return fail(SPA_EINVAL, "%s: grid too large", what);
   hipStream_t st = (hipStream_t)stream;
 
   // workspace carve-up; the running output of one rank is laid out [B, s, H, D]
@@ -202,14 +213,14 @@ int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* 
 
   if (fuse == SPA_RING_ALL_RANKS) {  // one launch: every requested rank, every step
     p.rank0 = r_lo; p.nranks = r_hi - r_lo; p.t_begin = 0; p.t_count = -1;
-    return launch_result(spa_launch_flash_fwd(p, D, dtype, st), "spa_ring_fwd");
+    return launch_result(spa_launch_flash_fwd(p, D, dtype, st), what);
   }
   for (int r = r_lo; r < r_hi; ++r) {
     p.rank0 = r; p.nranks = 1;
     if (fuse == SPA_RING_PER_RANK) {  // one launch per rank: the workgroup walks the rank's chunks
       p.t_begin = 0; p.t_count = -1;
       hipError_t e = spa_launch_flash_fwd(p, D, dtype, st);
-      if (e != hipSuccess) return launch_result(e, "spa_ring_fwd");
+      if (e != hipSuccess) return launch_result(e, what);
       continue;
     }
     const int nsteps = causal ? r + 1 : P;
@@ -248,9 +259,27 @@ int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* 
             e = spa_launch_finalize(outr, acc, B, H, s, D, p.os, as, SPA_F32, st);
         }
       }
-      if (e != hipSuccess) return launch_result(e, "spa_ring_fwd");
+      if (e != hipSuccess) return launch_result(e, what);
     }
   }
+  return SPA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace, int B,
+                 int H, int S, int D, int P, int rank, const int64_t q_strides[3], const int64_t k_strides[3],
+                 const int64_t v_strides[3], const int64_t o_strides[3], float scale, int mask_mode, int dtype,
+                 int fuse, void* stream) {
+  return ring_fwd("spa_ring_fwd", q, k, v, out, lse, workspace, -1, B, H, S, D, P, rank, q_strides, k_strides,
+                  v_strides, o_strides, scale, mask_mode, dtype, fuse, stream);
+}
+
+int spa_tune(int knob, int value) {
+  if (knob < 0 || knob >= SPA_KNOB_COUNT) return fail(SPA_EINVAL, "spa_tune: unknown knob %d", knob);
+  g_spa_knob[knob].store(value, std::memory_order_relaxed);
   return SPA_OK;
 }
 
@@ -299,6 +328,7 @@ int spa_bwd_delta(const void* out, const void* dout, float* delta, int B, int H,
   const int esz = elem_size(dtype);
   if (!aligned16(out, o_strides, esz) || !aligned16(dout, do_strides, esz))
     return fail(SPA_EALIGN, "spa_bwd_delta: pointers and row strides must be 16-byte aligned");
+  if ((int64_t)B * H * Sq * (D / 8) / 256 > 0x7ffffff0LL) return fail(SPA_EINVAL, "spa_bwd_delta: grid too large");
   return launch_result(spa_launch_delta(out, dout, delta, B, H, Sq, D, S3(o_strides), S3(do_strides), dtype,
                                         (hipStream_t)stream),
                        "spa_bwd_delta");
@@ -326,6 +356,8 @@ int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout,
   if (!span_ok(Sq, q_strides[2], D, esz) || !span_ok(Sk, k_strides[2], D, esz) || !span_ok(Sk, v_strides[2], D, esz) ||
       !span_ok(Sq, do_strides[2], D, esz))
     return fail(SPA_EUNSUPPORTED, "spa_flash_bwd: a tensor of one (batch, head) spans more than 2 GiB");
+  if ((int64_t)B * H * ((Sq + 127) / 128) > 0x7fffffffLL || (int64_t)B * H * ((Sk + 127) / 128) > 0x7fffffffLL)
+    return fail(SPA_EINVAL, "spa_flash_bwd: grid too large");
   BwdParams p;
   p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta;
   p.dq = dq_acc; p.dk = dk_acc; p.dv = dv_acc;

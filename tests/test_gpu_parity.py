@@ -14,7 +14,7 @@ import torch
 from conftest import rand, rand_qkv
 from oracle import attn_oracle as O
 import sp_aurora_amd as spa
-from sp_aurora_amd import ops
+from sp_aurora_amd import _lib, ops
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -369,20 +369,23 @@ def test_ring_backward_schedules_agree(causal):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,S,H,D,causal", [(1, 300, 2, 128, True), (2, 515, 2, 64, True), (1, 256, 3, 32, False),
                                             (1, 1000, 2, 128, False), (1, 77, 1, 128, True)])
-def test_dq_kernel_workgroup_sizes_agree(monkeypatch, B, S, H, D, causal, dtype):
+def test_dq_kernel_workgroup_sizes_agree(B, S, H, D, causal, dtype):
     """The dq kernel runs 128-row or 256-row workgroups depending on the grid; both orders of
     accumulation are the same per row, so the gradients must be identical, and right."""
     q, k, v, dout = rand_qkv((B, S, H, D), 140, dtype, n=4)
     want = O.attn_backward_autograd(q, k, v, dout, None, causal)
     got = {}
-    for waves in ("4", "8"):
-        monkeypatch.setenv("SPA_BWD_DQ_WAVES", waves)
-        xs = [t.to(DEV).requires_grad_(True) for t in (q, k, v)]
-        spa.ring_flash_attn_func(*xs, causal=causal).backward(dout.to(DEV))
-        got[waves] = [x.grad for x in xs]
-        for g, w, name in zip(got[waves], want, "qkv"):
-            check_grad(g, w, dtype, f"d{name} with {waves} waves")
-    for a, b in zip(got["4"], got["8"]):
+    try:
+        for waves in (4, 8):
+            _lib.tune("bwd_dq_waves", waves)
+            xs = [t.to(DEV).requires_grad_(True) for t in (q, k, v)]
+            spa.ring_flash_attn_func(*xs, causal=causal).backward(dout.to(DEV))
+            got[waves] = [x.grad for x in xs]
+            for g, w, name in zip(got[waves], want, "qkv"):
+                check_grad(g, w, dtype, f"d{name} with {waves} waves")
+    finally:
+        _lib.tune("bwd_dq_waves", 0)
+    for a, b in zip(got[4], got[8]):
         assert torch.equal(a, b)
 
 
@@ -457,12 +460,12 @@ def test_ring_driver_modes_on_awkward_shapes(P, B, s, H, D, causal, fuse):
 
 
 @pytest.fixture
-def shared_buffer_variant(monkeypatch):
+def shared_buffer_variant():
     """Forces the 256-row forward variant whose wave groups share the K/V buffers (it is otherwise
     chosen only for grids that fill the GPU twice over)."""
-    monkeypatch.setenv("SPA_FWD_SHARE", "1")
+    _lib.tune("fwd_share", 2)
     yield
-    monkeypatch.delenv("SPA_FWD_SHARE", raising=False)
+    _lib.tune("fwd_share", 0)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
