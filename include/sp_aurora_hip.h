@@ -126,6 +126,25 @@ int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* 
                  const int64_t v_strides[3], const int64_t o_strides[3],
                  float scale, int mask_mode, int dtype, int fuse, void* stream);
 
+/*
+ * spa_ring_fwd for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the same call without the workspace
+ * argument.  The scratch is a fixed buffer of SPA_STATIC_SCRATCH_BYTES inside the library's
+ * code object (every device the library is loaded on holds its own copy until the process
+ * ends); the call allocates and frees nothing.  Sizes whose spa_ring_fwd_workspace_bytes()
+ * exceed the buffer are rejected with SPA_EINVAL when the schedule needs the scratch.  All calls
+ * on one device share that device's buffer: calls that overlap in time on one device (two
+ * streams, two threads) race; serialise them.  Same kernels, same results as spa_ring_fwd.
+ * This entry point has no counterpart in the reference.
+ */
+#define SPA_STATIC_SCRATCH_BYTES (32 << 20)
+int64_t spa_static_scratch_bytes(void);
+int spa_ring_fwd_static(const void* q, const void* k, const void* v, void* out, float* lse,
+                        int B, int H, int S, int D, int P, int rank,
+                        const int64_t q_strides[3], const int64_t k_strides[3],
+                        const int64_t v_strides[3], const int64_t o_strides[3],
+                        float scale, int mask_mode, int dtype, int fuse, void* stream);
+
 /* out = cast(out_acc) — the `out.to(q.dtype)` that closes a ring forward
  * (sp_aurora/intel_ring_flash_attn.py:141-143). */
 int spa_finalize(void* out, const float* out_acc,

@@ -27,6 +27,8 @@ SIGNATURES = {
     "spa_flash_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _vp]),
     "spa_ring_fwd_workspace_bytes": (ctypes.c_int64, [_i, _i, _i, _i, _i, _i]),
     "spa_ring_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _i, _vp]),
+    "spa_static_scratch_bytes": (ctypes.c_int64, []),
+    "spa_ring_fwd_static": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _i, _vp]),
     "spa_tune": (_i, [_i, _i]),
     "spa_merge": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _s3, _s3, _i, _i, _vp]),
     "spa_finalize": (_i, [_vp, _vp, _i, _i, _i, _i, _s3, _s3, _i, _vp]),

@@ -11,6 +11,11 @@
 
 std::atomic<int> g_spa_knob[SPA_KNOB_COUNT];
 
+// Scratch of spa_ring_fwd_static: lives in the code object, one copy per device the library is
+// loaded on, from load to process end.  The name below is a host-side handle only; kernels and
+// copies get the device address hipGetSymbolAddress returns for the current device.
+static __device__ __align__(256) unsigned char scratch[SPA_STATIC_SCRATCH_BYTES];
+
 hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream);
 hipError_t spa_launch_flash_bwd(BwdParams p, int D, int dtype, hipStream_t stream);
 hipError_t spa_launch_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* blk_lse, int B,
@@ -154,6 +159,21 @@ int64_t spa_ring_fwd_workspace_bytes(int B, int H, int S, int D, int P, int dtyp
 
 namespace {
 
+// Device address of `scratch` on the current device, looked up once per device.
+int static_scratch(void** ptr) {
+  static std::atomic<void*> addr[SPA_MAX_DEVICES];
+  const int dev = spa_current_device();
+  if (dev < 0 || dev >= SPA_MAX_DEVICES) return fail(SPA_ELAUNCH, "spa_ring_fwd_static: no current device (or index >= %d)", SPA_MAX_DEVICES);
+  void* a = addr[dev].load(std::memory_order_acquire);
+  if (!a) {
+    const hipError_t e = hipGetSymbolAddress(&a, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !a) return fail(SPA_ELAUNCH, "spa_ring_fwd_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    addr[dev].store(a, std::memory_order_release);
+  }
+  *ptr = a;
+  return SPA_OK;
+}
+
 // `what` names the entry point in messages; `ws_bytes` < 0: the caller vouches for the workspace size.
 int ring_fwd(const char* what, const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
              int64_t ws_bytes, int B, int H, int S, int D, int P, int rank, const int64_t q_strides[3],
@@ -275,6 +295,19 @@ int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* 
                  int fuse, void* stream) {
   return ring_fwd("spa_ring_fwd", q, k, v, out, lse, workspace, -1, B, H, S, D, P, rank, q_strides, k_strides,
                   v_strides, o_strides, scale, mask_mode, dtype, fuse, stream);
+}
+
+int64_t spa_static_scratch_bytes(void) { return (int64_t)SPA_STATIC_SCRATCH_BYTES; }
+
+int spa_ring_fwd_static(const void* q, const void* k, const void* v, void* out, float* lse, int B, int H, int S,
+                        int D, int P, int rank, const int64_t q_strides[3], const int64_t k_strides[3],
+                        const int64_t v_strides[3], const int64_t o_strides[3], float scale, int mask_mode,
+                        int dtype, int fuse, void* stream) {
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc != SPA_OK) return rc;
+  return ring_fwd("spa_ring_fwd_static", q, k, v, out, lse, ws, (int64_t)SPA_STATIC_SCRATCH_BYTES, B, H, S, D, P,
+                  rank, q_strides, k_strides, v_strides, o_strides, scale, mask_mode, dtype, fuse, stream);
 }
 
 int spa_tune(int knob, int value) {
