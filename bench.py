@@ -1,34 +1,40 @@
 #!/usr/bin/env python3
-"""Benchmark of the ring-step attention hot path on one MI355X.
+"""Benchmark of the ring-step attention hot path on one MI355X.  Prints ONE JSON line.
 
-Workload = benchmark config 3: bf16, B=1, S=8192 in P=8 chunks of 1024, H=32, D=128, causal;
-every rank's Q chunk against its prefix of KV chunks in ring order (8 diagonal + 28 full block
-pairs), partial results merged per step, cast at the end.  One "step" is that whole 36-pair
-sweep; inputs are resident in HBM before the timed region.  value = causal-adjusted TFLOP/s of
-the whole sweep (549.76 GFLOP / step time).
+Headline workload = benchmark config 3: bf16, B=1, S=8192 in P=8 chunks of 1024, H=32, D=128,
+causal; every rank's Q chunk against its prefix of KV chunks in ring order (8 diagonal + 28 full
+block pairs), cast at the end.  One "step" is that whole 36-pair sweep; inputs are resident in
+HBM before the timed region.  value = causal-adjusted TFLOP/s of the sweep (549.76 GFLOP / step).
 
-The sweep is run through the C entry point spa_ring_fwd in its three schedules, all producing
-the same (out, lse):
-  all   one launch for the whole sweep: a workgroup keeps its query tile and accumulators in
-        registers and walks its rank's KV chunks in ring order (the step merge is the online
-        softmax).  This is `value`.
-  rank  one launch per rank (what one GPU of a real ring would run when its KV is resident).
-  step  one launch per (rank, ring step), running accumulators in HBM, the merge in the
-        kernel's epilogue (what a rank runs when each chunk arrives over the wire).
-The other two are reported beside it.
+The sweep runs through the C entry point spa_ring_fwd in three schedules, same (out, lse):
+  all   ONE launch for the sweep: every rank's workgroups are in one grid; a workgroup keeps its
+        query tile and accumulators in registers and walks its rank's KV chunks in ring order, so
+        the merge of ring steps is the online softmax itself.  A one-GPU fusion (the eight ranks of
+        a real ring are eight GPUs).  This is `value`.
+  rank  one launch per rank: what one GPU of a ring runs when its KV chunks are resident.
+  step  one launch per (rank, ring step), the running (out, lse) in HBM, the update_out_and_lse
+        merge in the kernel's epilogue: what a rank runs while chunks arrive over the wire.
+`other_schedules` holds rank and step; `ring_step` repeats the step figure as the per-ring-step
+number.
 
-Prints ONE JSON line.  `roofline` is for the dominant kernel, the block attention forward:
-algorithmic FLOPs per launch / average launch duration, the latter measured here with events on
-the launch stream over the timed region (in the `all` schedule the sweep is one launch of that
-kernel).  `cpu_baseline` times the oracle's restatement of the reference's op sequence (SDPA for
-out + a second q k^T / logsumexp for lse, sp_aurora/intel_flash_attn_optimized.py:156-193) on
-the host cores, on diagonal + full block pairs of the same workload.
+Timing protocol.  (1) settle: the same launch repeated until 10 consecutive launches agree within
+2 % or 0.3 s have passed (after an idle period the first ~40 launches run 5-25 % slower while the
+power management answers the load step; reported as `settle_launches`, `settle_ms`,
+`cold_ms_per_step` = mean of the first 5 launches).  (2) `--warmup` untimed steps.  (3) the timed
+region: blocks of exactly `--steps` steps, each block bracketed by events on the launch stream and
+a synchronize, repeated until >= 0.2 s are covered; `ms_per_step` is the MEDIAN block
+(`timed_blocks`, `block_ms_min`, `block_ms_max` beside it).
 
-`--workload` selects the other measured rows of the path instead (one JSON line each, same keys,
-`metric` named after the row): `relayout` = the Ulysses re-layout of benchmark config 4 (HBM
-bound), `merge` = update_out_and_lse on one config-3 chunk (HBM bound), `backward` = the ring
-backward of benchmark config 5 (MFMA bound), `ulysses` = the whole Ulysses forward of config 4.
+`roofline` is for the dominant kernel, the block attention forward: algorithmic FLOPs per launch
+/ its average launch duration, measured here with events over the timed region (in the `all`
+schedule a step is one launch of that kernel and nothing else).  `rows` carries the other rows of
+the path (configs 1, 2, 4, 5, merge), each with its own roofline and cpu_baseline.
+`cpu_baseline` legs time the oracle's restatement of the reference's op sequence (SDPA for out +
+a second q k^T / logsumexp for lse, sp_aurora/intel_flash_attn_optimized.py:156-193; sigmoid /
+logsigmoid merge, sp_aurora/utils.py:103-104; reshape / transpose / contiguous re-layout,
+sp_aurora/intel_ulysses_attn.py:95-138) on the host cores: 2 warm-up + 5 timed, median.
 
+`--workload` prints a single row instead (profiling runs: one kernel family per trace).
 Two helper modes for the HBM traffic figure (roofline.traffic):
   --traffic-leg          additionally runs a plain device copy of known size, so that a
                          `rocprofv3 --pmc FETCH_SIZE` (or WRITE_SIZE) run of this script holds
@@ -41,6 +47,7 @@ import csv
 import glob
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -48,6 +55,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+MFMA_F32_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBPS = 8000.0
 
 B, S, H, D, P = 1, 8192, 32, 128, 8
@@ -55,6 +63,8 @@ SEED = 2
 INPUT_SCALE = 0.5
 COPY_BYTES = 1 << 30  # calibration copy of the traffic leg: reads and writes this many bytes
 TRAFFIC_JSON = os.path.join(ROOT, "profiles", "flash_fwd_traffic.json")
+MIN_TIMED_S = 0.2
+MAX_BLOCKS = 200
 
 
 def sweep_flops():
@@ -72,15 +82,19 @@ def algorithmic_bytes():
     return n_pairs * 2 * chunk + P * chunk + P * chunk + B * H * S * 4
 
 
-def make_inputs(torch, device):
-    g = torch.Generator().manual_seed(SEED)
-    mk = lambda: (torch.randn((B, S, H, D), generator=g, dtype=torch.float32) * INPUT_SCALE).to(torch.bfloat16)
-    q, k, v = mk(), mk(), mk()
-    return q.to(device), k.to(device), v.to(device)
+def rand_tensors(torch, shape, seed, n, scale=1.0, dtype=None, device=None):
+    g = torch.Generator().manual_seed(seed)
+    out = []
+    for _ in range(n):
+        t = torch.randn(shape, generator=g, dtype=torch.float32) * scale
+        t = t.to(dtype or torch.bfloat16)
+        out.append(t.to(device) if device is not None else t)
+    return out
 
 
-def time_region(torch, fn, iters):
-    """ms per call of fn(), events on the current (= launch) stream."""
+# ------------------------------------------------------------------------------------ GPU timing
+def timed_block(torch, fn, iters):
+    """ms per call over exactly `iters` calls, events on the current (= launch) stream."""
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
@@ -92,44 +106,346 @@ def time_region(torch, fn, iters):
     return start.elapsed_time(end) / iters
 
 
-def cpu_baseline(torch, budget_s=15.0):
-    """The reference's op sequence on the host cores, on a bounded sample of the same workload."""
-    from oracle import attn_oracle as O
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16)
-    torch.set_num_threads(cores)
-    s = S // P
-    g = torch.Generator().manual_seed(SEED)
-    mk = lambda: (torch.randn((B, H, s, D), generator=g, dtype=torch.float32) * INPUT_SCALE).to(torch.bfloat16)
-    q, k, v = mk(), mk(), mk()
-    _, _, full = sweep_flops()
-
-    def pair(causal):
-        # bf16 inputs up-cast to fp32 on the host (no fast bf16 GEMM assumed); fp32 math
-        return O.attn_block_sdpa(q, k, v, None, causal, compute_dtype=torch.float32)
-
-    pair(False)  # warm-up
+def settle(torch, fn, max_s=0.3, need=10, tol=0.02):
+    """Repeats fn until `need` consecutive launches agree within `tol`, or max_s have passed.
+    Returns (launches, ms spent, mean ms of the first 5 launches)."""
     t0 = time.perf_counter()
-    n = 0
-    flops = 0.0
+    times = []
     while True:
-        pair(True)
-        pair(False)
-        n += 1
-        flops += full * 1.5
-        if time.perf_counter() - t0 > budget_s or n >= 400:
+        chunk = []
+        for _ in range(need):
+            a = torch.cuda.Event(enable_timing=True)
+            b = torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            chunk.append((a, b))
+        torch.cuda.synchronize()
+        times += [a.elapsed_time(b) for a, b in chunk]
+        last = times[-need:]
+        spent = time.perf_counter() - t0
+        if max(last) <= min(last) * (1.0 + tol) or spent >= max_s:
             break
-    dt = time.perf_counter() - t0
-    return {
-        "value": flops / dt / 1e12,
-        "unit": "TFLOP/s",
-        "cores": cores,
-        "kind": "port",
-        "sample": f"{n} x (1 diagonal + 1 full block pair of config 3: B1 H32 s1024 D128), bf16 inputs up-cast "
-                  f"to fp32, torch CPU SDPA + second QK^T/logsumexp, {dt:.1f} s",
-    }
+    return len(times), spent * 1e3, sum(times[:5]) / min(5, len(times))
 
 
+def measure(torch, fn, steps, warmup, min_s=MIN_TIMED_S, do_settle=True):
+    """The protocol of the module docstring for one callable.  Returns a dict."""
+    res = {}
+    if do_settle:
+        n, ms, cold = settle(torch, fn)
+        res.update(settle_launches=n, settle_ms=round(ms, 2), cold_ms_per_step=round(cold, 4))
+    for _ in range(warmup):
+        fn()
+    blocks = []
+    covered = 0.0
+    while covered < min_s and len(blocks) < MAX_BLOCKS:
+        t = timed_block(torch, fn, steps)
+        blocks.append(t)
+        covered += t * steps * 1e-3
+    res.update(ms_per_step=statistics.median(blocks), timed_blocks=len(blocks), block_ms_min=round(min(blocks), 4),
+               block_ms_max=round(max(blocks), 4), timed_region_s=round(covered, 3))
+    return res
+
+
+# ------------------------------------------------------------------------------------ CPU baseline
+def host_threads():
+    """Threads for the CPU legs: every core this process may run on, bounded by the share the
+    environment assigns through OMP_NUM_THREADS when it sets one."""
+    logical = os.cpu_count() or 1
+    try:
+        affinity = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        affinity = logical
+    physical = None
+    try:
+        cores = set()
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("physical id"):
+                phys = line.split(":")[1].strip()
+            elif line.startswith("core id"):
+                core = line.split(":")[1].strip()
+            elif not line.strip():
+                if phys is not None and core is not None:
+                    cores.add((phys, core))
+                phys = core = None
+        physical = len(cores) or None
+    except OSError:
+        pass
+    env = os.environ.get("OMP_NUM_THREADS")
+    used = affinity
+    if env and env.isdigit() and int(env) > 0:
+        used = min(used, int(env))
+    return used, {"logical": logical, "physical": physical, "affinity": affinity, "omp_num_threads_env": env}
+
+
+def cpu_time(fn, warm=2, timed=5):
+    for _ in range(warm):
+        fn()
+    ts = []
+    for _ in range(timed):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return statistics.median(ts)
+
+
+class CpuLegs:
+    """The reference's op sequence per row on the host cores (oracle restatements, fp32 torch;
+    bf16 inputs are up-cast to fp32: no fast bf16 GEMM is assumed on the host)."""
+
+    def __init__(self, torch):
+        from oracle import attn_oracle as O
+        self.torch, self.O = torch, O
+        self.threads, self.host = host_threads()
+        torch.set_num_threads(self.threads)
+        self.host["torch_num_threads"] = torch.get_num_threads()
+        self._pair_cache = {}
+
+    def _entry(self, value, unit, sample, kind="port"):
+        return {"value": value, "unit": unit, "cores": self.threads, "kind": kind, "sample": sample, "host": self.host}
+
+    def pair_times(self, Bn, Hn, sn, Dn, seed):
+        """seconds for one diagonal and one full block pair [Bn,Hn,sn,Dn] (SDPA + second QK^T/logsumexp)."""
+        key = (Bn, Hn, sn, Dn)
+        if key not in self._pair_cache:
+            torch, O = self.torch, self.O
+            q, k, v = rand_tensors(torch, (Bn, Hn, sn, Dn), seed, 3, INPUT_SCALE)
+            f = lambda causal: O.attn_block_sdpa(q, k, v, None, causal, compute_dtype=torch.float32)
+            self._pair_cache[key] = (cpu_time(lambda: f(True)), cpu_time(lambda: f(False)))
+        return self._pair_cache[key]
+
+    def ring_forward(self, Bn, Hn, sn, Dn, n_diag, n_full, seed, what):
+        """Extrapolation from one measured diagonal and one measured full pair."""
+        t_d, t_f = self.pair_times(Bn, Hn, sn, Dn, seed)
+        full = 4.0 * Bn * Hn * sn * sn * Dn
+        flops = n_full * full + n_diag * full / 2
+        secs = n_diag * t_d + n_full * t_f
+        return self._entry(flops / secs / 1e12, "TFLOP/s",
+                           f"{what}: measured 1 diagonal ({t_d * 1e3:.1f} ms) + 1 full ({t_f * 1e3:.1f} ms) block pair "
+                           f"[B{Bn},H{Hn},s{sn},D{Dn}] (median of 5 after 2 warm-up), extrapolated to {n_diag} diagonal + "
+                           f"{n_full} full pairs = {secs * 1e3:.0f} ms; bf16 inputs up-cast to fp32, torch CPU SDPA + second QK^T/logsumexp")
+
+    def config1(self):
+        torch, O = self.torch, self.O
+        q, k, v = rand_tensors(torch, (1, 8, 512, 64), 0, 3, 1.0, torch.float32)
+        t = cpu_time(lambda: O.attn_block_sdpa(q, k, v, 0.125, False, compute_dtype=torch.float32))
+        return self._entry(4.0 * 8 * 512 * 512 * 64 / t / 1e12, "TFLOP/s",
+                           f"config 1 in full: fp32 [1,8,512,64] non-causal, SDPA + second QK^T/logsumexp, {t * 1e3:.2f} ms (median of 5)")
+
+    def config2(self):
+        """Rank 2 of the P=4 ring in full: 3 block pairs + 1 init, 2 merges (sigmoid / logsigmoid form)."""
+        torch, O = self.torch, self.O
+        Bn, Hn, sn, Dn = 2, 32, 1024, 64
+        q, = rand_tensors(torch, (Bn, Hn, sn, Dn), 1, 1)
+        ks = rand_tensors(torch, (Bn, Hn, sn, Dn), 11, 3)
+        vs = rand_tensors(torch, (Bn, Hn, sn, Dn), 12, 3)
+
+        def run():
+            out = lse = None
+            for t, c in enumerate((2, 1, 0)):
+                bo, bl = O.attn_block_sdpa(q, ks[c], vs[c], None, t == 0, compute_dtype=torch.float32)
+                if out is None:
+                    out, lse = bo.float(), bl.unsqueeze(-1)
+                else:
+                    out, lse = O.merge(out, lse, bo, bl.unsqueeze(-1))
+            return out.to(torch.bfloat16), lse
+
+        t = cpu_time(run)
+        flops = 2.5 * 4.0 * Bn * Hn * sn * sn * Dn
+        return self._entry(flops / t / 1e12, "TFLOP/s",
+                           f"config 2 in full: rank 2 of P=4, [B2,H32,s1024,D64], 1 diagonal + 2 full pairs + merges, {t * 1e3:.0f} ms (median of 5); "
+                           "bf16 inputs up-cast to fp32")
+
+    def relayout(self):
+        torch, O = self.torch, self.O
+        x, = rand_tensors(torch, (8, 1, 2048, 32, 128), 3, 1)
+        xs = list(x)
+        t_s2h = cpu_time(lambda: O.all_to_all_4d_s2h(xs), 1, 3)
+        ys = O.all_to_all_4d_s2h(xs)
+        t_h2s = cpu_time(lambda: O.all_to_all_4d_h2s(ys), 1, 3)
+        nbytes = 2 * x.numel() * 2
+        mk = lambda t, d: self._entry(nbytes / t / 1e9, "GB/s", f"config 4 tensor [8,1,2048,32,128] bf16 in full, {d}: the reference's "
+                                      f"reshape/transpose/contiguous chains around the exchange, {t * 1e3:.0f} ms (median of 3)")
+        return mk(t_s2h, "s2h"), mk(t_h2s, "h2s")
+
+    def merge(self):
+        torch, O = self.torch, self.O
+        g = torch.Generator().manual_seed(3)
+        acc = torch.randn((1, 32, 1024, 128), generator=g)
+        lse = torch.randn((1, 32, 1024, 1), generator=g)
+        blk = torch.randn((1, 32, 1024, 128), generator=g).to(torch.bfloat16)
+        bl = torch.randn((1, 32, 1024, 1), generator=g)
+        t = cpu_time(lambda: O.merge(acc, lse, blk.float(), bl))
+        return self._entry((acc.numel() * 10 + lse.numel() * 12) / t / 1e9, "GB/s",
+                           f"one config-3 chunk [1,32,1024,128]: sigmoid / logsigmoid merge of a bf16 block into fp32 (out, lse), {t * 1e3:.1f} ms (median of 5)")
+
+    def backward(self, n_diag, n_full):
+        torch, O = self.torch, self.O
+        q, k, v, do = rand_tensors(torch, (1, 2048, 16, 128), 4, 4)
+        f = lambda causal: O.attn_backward_autograd(q, k, v, do, None, causal, compute_dtype=torch.float32)
+        t_d = cpu_time(lambda: f(True), 1, 3)
+        t_f = cpu_time(lambda: f(False), 1, 3)
+        full = 2.5 * 4.0 * 16 * 2048 * 2048 * 128
+        secs = n_diag * t_d + n_full * t_f
+        return self._entry((n_full * full + n_diag * full / 2) / secs / 1e12, "TFLOP/s",
+                           f"config 5 backward: measured 1 diagonal ({t_d * 1e3:.0f} ms) + 1 full ({t_f * 1e3:.0f} ms) block pair [1,2048,16,128] "
+                           f"through torch CPU autograd of softmax(QK^T)V (forward recompute included, as in the reference), median of 3, "
+                           f"extrapolated to {n_diag} + {n_full} pairs = {secs:.1f} s; 5-GEMM FLOP count; bf16 up-cast to fp32")
+
+
+# ------------------------------------------------------------------------------------ rows
+def roof(bound, kernel, achieved, peak, unit, **extra):
+    r = {"bound": bound, "kernel": kernel, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+         "frac": round(achieved / peak, 4), "traffic": None}
+    r.update(extra)
+    return r
+
+
+def gpu_rows(torch, spa, ops, which, steps, warmup):
+    """GPU legs of the side rows.  Returns {name: row-dict without cpu_baseline}."""
+    dev = torch.device("cuda:0")
+    rows = {}
+    light = dict(min_s=0.05, do_settle=False)
+
+    def finish(name, m, config, value, unit, roofline):
+        rows[name] = {"row": name, "value": round(value, 2), "unit": unit, "ms_per_step": round(m["ms_per_step"], 4),
+                      "timed_blocks": m["timed_blocks"], "config": config, "roofline": roofline}
+
+    if "config1" in which:
+        q, k, v = rand_tensors(torch, (1, 512, 8, 64), 0, 3, 1.0, torch.float32, dev)
+        out = torch.empty_like(q)
+        lse = torch.empty((1, 8, 512), dtype=torch.float32, device=dev)
+        fn = lambda: ops.flash_fwd(q, k, v, 0.125, False, layout="bshd", out=out, lse=lse)
+        m = measure(torch, fn, 20, 5, **light)
+        tf = 4.0 * 8 * 512 * 512 * 64 / (m["ms_per_step"] * 1e-3) / 1e12
+        finish("config1_fp32_block_forward", m, {"workload": "config 1: fp32 B=1 S=512 H=8 D=64 non-causal block forward, out + lse"},
+               tf, "TFLOP/s", roof("mfma", "flash_fwd32_kernel<64>", tf, MFMA_F32_PEAK_TFLOPS, "TFLOP/s"))
+    if "config2" in which:
+        Bn, Sn, Hn, Dn, Pn, r = 2, 4096, 32, 64, 4, 2
+        q, k, v = rand_tensors(torch, (Bn, Sn, Hn, Dn), 1, 3, 1.0, torch.bfloat16, dev)
+        out = torch.empty_like(q)
+        lse = torch.empty((Bn, Hn, Sn), dtype=torch.float32, device=dev)
+        ws = ops.ring_fwd_workspace(q, Pn)
+        flops = 2.5 * 4.0 * Bn * Hn * (Sn // Pn) ** 2 * Dn
+        sched = {}
+        for fuse in ("step", "rank"):
+            fn = lambda fuse=fuse: ops.ring_fwd(q, k, v, Pn, None, True, rank=r, out=out, lse=lse, workspace=ws, fuse=fuse)
+            sched[fuse] = measure(torch, fn, 20, 5, **light)
+        m = sched["rank"]
+        tf = flops / (m["ms_per_step"] * 1e-3) / 1e12
+        tf_step = flops / (sched["step"]["ms_per_step"] * 1e-3) / 1e12
+        finish("config2_ring_rank2_of_4", m,
+               {"workload": "config 2: bf16 B=2 S=4096 (P=4 chunks of 1024) H=32 D=64 causal, rank 2: diagonal chunk 2, then chunks 1, 0, merged",
+                "flops_per_step": flops, "one_launch_per_ring_step": {"ms_per_step": round(sched["step"]["ms_per_step"], 4), "tflops": round(tf_step, 2),
+                                                                        "launches_per_step": 3}},
+               tf, "TFLOP/s", roof("mfma", "flash_fwd16_kernel<bf16,64,2>", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", launches_per_step=1))
+    if "config4" in which:
+        Pn, Bn, sn, Hn, Dn = 8, 1, 2048, 32, 128
+        q, k, v = rand_tensors(torch, (Pn, Bn, sn, Hn, Dn), 3, 3, 1.0, torch.bfloat16, dev)
+        # q, k, v take turns (and so do three destinations): 805 MB in flight, so that a launch finds
+        # neither its source nor its destination in the 256 MB memory-side cache
+        xs = [q, k, v]
+        ys = [torch.empty((Pn, Bn, Pn * sn, Hn // Pn, Dn), dtype=q.dtype, device=dev) for _ in range(3)]
+        backs = [torch.empty_like(q) for _ in range(3)]
+        nbytes = 2 * q.numel() * 2
+        turn = [0]
+
+        def s2h():
+            i = turn[0] = (turn[0] + 1) % 3
+            ops.relayout_s2h(xs[i], Pn, out=ys[i])
+
+        def h2s():
+            i = turn[0] = (turn[0] + 1) % 3
+            ops.relayout_h2s(ys[i], Pn, out=backs[i])
+
+        for name, fn, kern in (("s2h", s2h, "relayout_kernel<16,s2h>"), ("h2s", h2s, "relayout_kernel<16,h2s>")):
+            m = measure(torch, fn, 21, 6, **light)
+            gb = nbytes / (m["ms_per_step"] * 1e-3) / 1e9
+            finish(f"config4_relayout_{name}", m,
+                   {"workload": f"config 4 re-layout {name}: [P=8,B=1,s=2048,H=32,D=128] bf16 <-> [8,1,16384,4,128], one tensor and one direction per "
+                                "launch, q / k / v in turn",
+                    "bytes_per_launch": nbytes, "includes": "host cost of the call (event-timed back to back); kernel-only time is in profiles/"},
+                   gb, "GB/s", roof("hbm", kern, gb, HBM_PEAK_GBPS, "GB/s"))
+        y = ys[0]
+        del ys, backs
+        scale = Dn ** -0.5
+        fn = lambda: spa.intel_ulysses_flash_attn_forward(None, q, k, v, scale, causal=True)
+        fn()
+        m = measure(torch, fn, 5, 2, **light)
+        flops = 4.0 * Bn * Hn * (Pn * sn) ** 2 * Dn / 2
+        tf = flops / (m["ms_per_step"] * 1e-3) / 1e12
+        finish("config4_ulysses_forward", m,
+               {"workload": "config 4: q,k,v [P=8,B=1,s=2048,H=32,D=128] bf16 -> head-sharded [8,1,16384,4,128], full causal attention per head group, "
+                            "inverse re-layout of out (3 re-layouts in, attention, 1 out; output allocation included)", "flops_per_step": flops},
+               tf, "TFLOP/s", roof("mfma", "relayout_kernel x4 + flash_fwd16_kernel<bf16,128,2>", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
+        del q, k, v, y, xs
+    if "merge" in which:
+        Bn, sn, Hn, Dn = 1, 1024, 32, 128
+        g = torch.Generator().manual_seed(3)
+        acc = torch.randn((Bn, sn, Hn, Dn), generator=g, dtype=torch.float32).to(dev)
+        lse = torch.randn((Bn, Hn, sn), generator=g, dtype=torch.float32).to(dev)
+        blk = torch.randn((Bn, sn, Hn, Dn), generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev)
+        blk_lse = torch.randn((Bn, Hn, sn), generator=g, dtype=torch.float32).to(dev)
+        fn = lambda: ops.merge(acc, lse, blk, blk_lse, layout="bshd")
+        m = measure(torch, fn, 20, 5, **light)
+        nbytes = acc.numel() * 10 + lse.numel() * 12
+        gb = nbytes / (m["ms_per_step"] * 1e-3) / 1e9
+        finish("merge_update_out_and_lse", m,
+               {"workload": "update_out_and_lse: merge of a bf16 block into the fp32 running (out, lse) of one config-3 rank [1,1024,32,128]",
+                "bytes_per_launch": nbytes, "includes": "host cost of the call (event-timed back to back); kernel-only time is in profiles/"},
+               gb, "GB/s", roof("hbm", "merge_kernel<bf16>", gb, HBM_PEAK_GBPS, "GB/s"))
+    if "config5" in which:
+        Bn, Sn, Hn, Dn, Pn = 1, 32768, 16, 128, 16
+        qkv, = rand_tensors(torch, (Bn, Sn, 3, Hn, Dn), 4, 1, 1.0, torch.bfloat16, dev)
+        dout, = rand_tensors(torch, (Bn, Sn, Hn, Dn), 5, 1, 1.0, torch.bfloat16, dev)
+        q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+        scale = Dn ** -0.5
+        fstep = spa.ring.make_ring_forward_step(q, k, v, scale, True, Pn, fuse="all")
+        out, lse = fstep()
+        m = measure(torch, fstep, 3, 1, **light)
+        fwd_flops = 4.0 * Bn * Hn * Sn * Sn * Dn / 2
+        tf = fwd_flops / (m["ms_per_step"] * 1e-3) / 1e12
+        finish("config5_ring_forward", m,
+               {"workload": "config 5 forward: bf16 qkv [1,32768,3,16,128] (strided views) causal, ring of 16 chunks of 2048, 16 diagonal + 120 full pairs, schedule 'all'",
+                "flops_per_step": fwd_flops},
+               tf, "TFLOP/s", roof("mfma", "flash_fwd16_kernel<bf16,128,2>", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", launches_per_step=1))
+        fn = lambda: spa.ring.ring_flash_attn_backward(dout, q, k, v, out, lse, scale, True, Pn, fuse="all")
+        fn()
+        m = measure(torch, fn, 3, 1, **light)
+        bwd_flops = 2.5 * fwd_flops
+        tf = bwd_flops / (m["ms_per_step"] * 1e-3) / 1e12
+        finish("config5_ring_backward", m,
+               {"workload": "config 5 backward: dq/dk/dv by block-wise recompute with the global lse over the same 136 block pairs, one launch per kernel "
+                            "(delta pre-pass, fp32 accumulator zeroing and final casts included); 5-GEMM FLOP count (the two kernels execute 7)",
+                "flops_per_step": bwd_flops},
+               tf, "TFLOP/s", roof("mfma", "flash_bwd_dq_kernel + flash_bwd_dkdv_kernel", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
+        del qkv, dout, out, lse
+    torch.cuda.empty_cache()
+    return rows
+
+
+def attach_cpu(rows, cpu):
+    """cpu_baseline per row (host legs run after every GPU leg, so they do not sit between launches)."""
+    if "config1_fp32_block_forward" in rows:
+        rows["config1_fp32_block_forward"]["cpu_baseline"] = cpu.config1()
+    if "config2_ring_rank2_of_4" in rows:
+        rows["config2_ring_rank2_of_4"]["cpu_baseline"] = cpu.config2()
+    if "config4_relayout_s2h" in rows:
+        a, b = cpu.relayout()
+        rows["config4_relayout_s2h"]["cpu_baseline"] = a
+        rows["config4_relayout_h2s"]["cpu_baseline"] = b
+        rows["config4_ulysses_forward"]["cpu_baseline"] = cpu.ring_forward(
+            1, 4, 2048, 128, 8, 28, 3, "config 4 attention of one head group [1,4,16384,128] as 2048-row blocks (x 8 groups: same ratio); re-layouts not included")
+    if "merge_update_out_and_lse" in rows:
+        rows["merge_update_out_and_lse"]["cpu_baseline"] = cpu.merge()
+    if "config5_ring_forward" in rows:
+        rows["config5_ring_forward"]["cpu_baseline"] = cpu.ring_forward(1, 16, 2048, 128, 16, 120, 4, "config 5 forward")
+        rows["config5_ring_backward"]["cpu_baseline"] = cpu.backward(16, 120)
+
+
+# ------------------------------------------------------------------------------------ traffic helper
 def pmc_summary(fetch_dir, write_dir):
     """FETCH_SIZE / WRITE_SIZE (KiB per dispatch) of the attention kernel, each scaled by what the
     same counter reads for the calibration copy of COPY_BYTES."""
@@ -177,190 +493,92 @@ def pmc_summary(fetch_dir, write_dir):
     print(json.dumps(res, indent=1))
 
 
-def side_workload(torch, name, steps, warmup):
-    """The other rows of the path: one JSON line with the same keys, roofline against its own bound."""
-    import sp_aurora_amd as spa
-    from sp_aurora_amd import ops
-    dev = torch.device("cuda:0")
-    g = torch.Generator().manual_seed(3)
-    rnd = lambda shape, dt=torch.bfloat16: torch.randn(shape, generator=g, dtype=torch.float32).to(dt).to(dev)
-    if name == "relayout":
-        Pn, Bn, sn, Hn, Dn = 8, 1, 2048, 32, 128
-        x = rnd((Pn, Bn, sn, Hn, Dn))
-        y = torch.empty((Pn, Bn, Pn * sn, Hn // Pn, Dn), dtype=x.dtype, device=dev)
-        back = torch.empty_like(x)
-        fn = lambda: (ops.relayout_s2h(x, Pn, out=y), ops.relayout_h2s(y, Pn, out=back))
-        units, unit_bytes = 2, 2 * x.numel() * 2   # two launches per step, each reads and writes the tensor once
-        bound, kernel, metric = "hbm", "relayout_kernel<16>", "Ulysses re-layout GB/s, config 4 [8,1,2048,32,128] bf16, s2h + h2s"
-        work = {"workload": "config 4 re-layout: [P=8,B=1,s=2048,H=32,D=128] bf16 -> [8,1,16384,4,128] and back", "bytes_per_launch": unit_bytes}
-    elif name == "ulysses":
-        Pn, Bn, sn, Hn, Dn = 8, 1, 2048, 32, 128
-        q, k, v = rnd((Pn, Bn, sn, Hn, Dn)), rnd((Pn, Bn, sn, Hn, Dn)), rnd((Pn, Bn, sn, Hn, Dn))
-        scale = Dn ** -0.5
-        fn = lambda: spa.intel_ulysses_flash_attn_forward(None, q, k, v, scale, causal=True)
-        unit_flops = 4.0 * Bn * Hn * (Pn * sn) ** 2 * Dn / 2
-        units = 1
-        bound, kernel, metric = "mfma", "relayout_kernel x4 + flash_fwd16_kernel<bf16,128,2>", "Ulysses forward TFLOP/s (causal-adjusted attention FLOPs over the whole step: 3 re-layouts in, attention, 1 out), config 4"
-        work = {"workload": "config 4: q,k,v [P=8,B=1,s=2048,H=32,D=128] bf16 -> head-sharded [8,1,16384,4,128], full causal attention "
-                            "per head group, inverse re-layout of out", "flops_per_step": unit_flops}
-    elif name == "merge":
-        Bn, sn, Hn, Dn = 1, 1024, 32, 128
-        acc = torch.randn((Bn, sn, Hn, Dn), generator=g, dtype=torch.float32).to(dev)
-        lse = torch.randn((Bn, Hn, sn), generator=g, dtype=torch.float32).to(dev)
-        blk = rnd((Bn, sn, Hn, Dn))
-        blk_lse = torch.randn((Bn, Hn, sn), generator=g, dtype=torch.float32).to(dev)
-        fn = lambda: ops.merge(acc, lse, blk, blk_lse, layout="bshd")
-        units, unit_bytes = 1, acc.numel() * 10 + lse.numel() * 12
-        bound, kernel, metric = "hbm", "merge_kernel<bf16>", "update_out_and_lse GB/s, one config-3 chunk [1,1024,32,128]"
-        work = {"workload": "merge of a bf16 block into the fp32 running (out, lse) of one config-3 rank", "bytes_per_launch": unit_bytes}
-    elif name == "backward":
-        Bn, Sn, Hn, Dn, Pn = 1, 32768, 16, 128, 16
-        qkv = rnd((Bn, Sn, 3, Hn, Dn))
-        dout = rnd((Bn, Sn, Hn, Dn))
-        q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
-        scale = Dn ** -0.5
-        out, lse = spa.ring.ring_flash_attn_forward(q, k, v, scale, True, Pn, fuse="all")
-        fn = lambda: spa.ring.ring_flash_attn_backward(dout, q, k, v, out, lse, scale, True, Pn, fuse="all")
-        fn_step = lambda: spa.ring.ring_flash_attn_backward(dout, q, k, v, out, lse, scale, True, Pn, fuse="step")
-        fwd_flops = 4.0 * Bn * Hn * Sn * Sn * Dn / 2
-        units, unit_flops = 1, 2.5 * fwd_flops   # five GEMMs of the algorithm (the two kernels recompute S and dP: 7 executed)
-        bound, kernel, metric = "mfma", "flash_bwd_dq_kernel + flash_bwd_dkdv_kernel", "ring backward TFLOP/s (5-GEMM count, causal-adjusted), config 5 S=32K H16 D128 P=16"
-        work = {"workload": "config 5 backward: bf16 qkv [1,32768,3,16,128] causal, ring of 16 chunks, dq/dk/dv by block-wise "
-                            "recompute with the global lse; value = the 136 block pairs walked inside one launch per kernel "
-                            "(delta pre-pass, fp32 accumulator zeroing and the final casts included)", "flops_per_step": unit_flops}
-        fn_step()
-        t_step = time_region(torch, fn_step, 3)
-        work["one_launch_per_block_pair"] = {"ms_per_step": round(t_step, 3), "tflops": round(unit_flops / (t_step * 1e-3) / 1e12, 2)}
-    else:
-        raise SystemExit(f"unknown workload {name}")
-    for _ in range(warmup):
-        fn()
-    ms = time_region(torch, fn, steps)
-    cpu = side_cpu_baseline(torch, name) if name != "ulysses" else None
-    if bound == "hbm":
-        achieved = units * unit_bytes / (ms * 1e-3) / 1e9
-        peak, unit = HBM_PEAK_GBPS, "GB/s"
-    else:
-        achieved = unit_flops / (ms * 1e-3) / 1e12
-        peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
-    print(json.dumps({
-        "metric": metric, "value": round(achieved, 2), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
-        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic", "config": work,
-        "roofline": {"bound": bound, "kernel": kernel, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-                     "frac": round(achieved / peak, 4), "traffic": None},
-        "cpu_baseline": cpu,
-    }))
-
-
-def side_cpu_baseline(torch, name, budget_s=10.0):
-    """The reference's op sequence for the row on the host cores (oracle restatements, fp32 torch)."""
-    from oracle import attn_oracle as O
-    cores = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(cores)
-    g = torch.Generator().manual_seed(3)
-    if name == "relayout":
-        # the reference's reshape / transpose / contiguous chain around all_to_all_single
-        # (sp_aurora/intel_ulysses_attn.py:95-138) on the full config-4 tensor, both directions
-        x = torch.randn((8, 1, 2048, 32, 128), generator=g).to(torch.bfloat16)
-        xs = list(x)
-        fn = lambda: O.all_to_all_4d_h2s(O.all_to_all_4d_s2h(xs))
-        work, unit = 2 * 2 * x.numel() * 2 / 1e9, "GB/s"
-        sample = "config 4 tensor [8,1,2048,32,128] bf16, s2h then h2s, literal reshape/transpose/contiguous chains"
-    elif name == "merge":
-        acc = torch.randn((1, 32, 1024, 128), generator=g)
-        lse = torch.randn((1, 32, 1024, 1), generator=g)
-        blk = torch.randn((1, 32, 1024, 128), generator=g).to(torch.bfloat16)
-        bl = torch.randn((1, 32, 1024, 1), generator=g)
-        fn = lambda: O.merge(acc, lse, blk.float(), bl)
-        work, unit = (acc.numel() * 10 + lse.numel() * 12) / 1e9, "GB/s"
-        sample = "one config-3 chunk [1,32,1024,128]: sigmoid / logsigmoid merge of a bf16 block into fp32 (out, lse)"
-    else:
-        # one diagonal + one full block pair of config 5 through autograd of the closed form
-        q, k, v, do = (torch.randn((1, 2048, 16, 128), generator=g).to(torch.bfloat16) for _ in range(4))
-        fn = lambda: (O.attn_backward_autograd(q, k, v, do, None, True, compute_dtype=torch.float32),
-                      O.attn_backward_autograd(q, k, v, do, None, False, compute_dtype=torch.float32))
-        work, unit = 2.5 * 1.5 * 4.0 * 16 * 2048 * 2048 * 128 / 1e12, "TFLOP/s"
-        sample = "1 diagonal + 1 full block pair of config 5 ([1,16,2048,128] bf16 up-cast to fp32), torch CPU autograd of softmax(QK^T)V"
-    fn()  # warm-up
-    t0 = time.perf_counter()
-    n = 0
-    while time.perf_counter() - t0 < budget_s and n < 2000:
-        fn()
-        n += 1
-    dt = time.perf_counter() - t0
-    return {"value": work * n / dt, "unit": unit, "cores": cores, "kind": "port", "sample": f"{n} x ({sample}), {dt:.1f} s"}
+# ------------------------------------------------------------------------------------ main
+ROW_SETS = {"relayout": {"config4"}, "ulysses": {"config4"}, "merge": {"merge"}, "backward": {"config5"},
+            "config1": {"config1"}, "config2": {"config2"}}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=50,
-                    help="the first ~50 launches after an idle period run slower while the GPU settles its clocks")
-    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline leg")
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side baseline legs")
+    ap.add_argument("--no-rows", action="store_true", help="headline only (profiling runs)")
     ap.add_argument("--only-all", action="store_true", help="skip the rank / step schedules (profiling runs)")
+    ap.add_argument("--schedule", default="all", choices=["all", "rank", "step"],
+                    help="which schedule --only-all runs (profiling runs); `value` is always the `all` schedule otherwise")
     ap.add_argument("--traffic-leg", action="store_true", help="also run the calibration copy (for --pmc runs)")
     ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"))
-    ap.add_argument("--workload", default="config3", choices=["config3", "relayout", "merge", "backward", "ulysses"])
+    ap.add_argument("--workload", default="config3", choices=["config3"] + sorted(ROW_SETS))
     args = ap.parse_args()
     if args.pmc_summary:
         pmc_summary(*args.pmc_summary)
         return
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU (the ring is simulated on it); --gpus must be 1", file=sys.stderr)
+        print("bench.py: this build measures one GPU (the ring is simulated on it, no collectives); --gpus must be 1", file=sys.stderr)
         sys.exit(2)
 
     import torch
     import sp_aurora_amd as spa
+    from sp_aurora_amd import ops
 
     if not torch.cuda.is_available():
         print("bench.py: no HIP device visible", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
     if args.workload != "config3":
-        heavy = args.workload in ("backward", "ulysses")
-        side_workload(torch, args.workload, min(args.steps, 5) if heavy else args.steps, min(args.warmup, 2) if heavy else args.warmup)
+        rows = gpu_rows(torch, spa, ops, ROW_SETS[args.workload], args.steps, args.warmup)
+        if not args.no_cpu_baseline:
+            attach_cpu(rows, CpuLegs(torch))
+        print(json.dumps({"rows": list(rows.values())}))
         return
-    q, k, v = make_inputs(torch, dev)
+
+    q, k, v = rand_tensors(torch, (B, S, H, D), SEED, 3, INPUT_SCALE, torch.bfloat16, dev)
     scale = D ** -0.5
     total_flops, n_pairs, full_flops = sweep_flops()
 
     # preallocated buffers, no allocation per step
     steps = {m: spa.ring.make_ring_forward_step(q, k, v, scale, True, P, fuse=m) for m in ("all", "rank", "step")}
-
-    step = steps["all"]
-    for _ in range(args.warmup):
-        step()
-    ms = time_region(torch, step, args.steps)
+    head = args.schedule if args.only_all else "all"
+    m_all = measure(torch, steps[head], args.steps, args.warmup)
+    ms = m_all["ms_per_step"]
     tflops = total_flops / (ms * 1e-3) / 1e12
 
     other = {}
     if not args.only_all:
-        for m in ("rank", "step"):
-            for _ in range(max(3, args.warmup // 4)):
-                steps[m]()
-            t = time_region(torch, steps[m], max(5, args.steps // 4))
-            other[m] = {"ms_per_step": round(t, 4), "tflops": round(total_flops / (t * 1e-3) / 1e12, 2),
-                        "launches_per_step": P if m == "rank" else n_pairs}
+        for name in ("rank", "step"):
+            mm = measure(torch, steps[name], args.steps, args.warmup, min_s=0.1, do_settle=False)
+            t = mm["ms_per_step"]
+            launches = P if name == "rank" else n_pairs
+            other[name] = {"ms_per_step": round(t, 4), "tflops": round(total_flops / (t * 1e-3) / 1e12, 2),
+                           "pct_of_bf16_mfma_peak": round(100.0 * total_flops / (t * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
+                           "launches_per_step": launches, "avg_launch_us": round(t * 1e3 / launches, 2), "timed_blocks": mm["timed_blocks"]}
 
     if args.traffic_leg:
         src = torch.empty(COPY_BYTES, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
+        del src, dst
 
-    traffic = None
+    traffic = traffic_src = None
     if os.path.exists(TRAFFIC_JSON):
         try:
             traffic = json.load(open(TRAFFIC_JSON)).get("hbm_bytes_per_launch")
+            traffic_src = ("profiles/flash_fwd_traffic.json: two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of an earlier build of this "
+                           "kernel, scaled by a 1 GiB copy; a recorded constant, not measured in this run")
         except (ValueError, OSError):
             traffic = None
 
-    # dominant kernel: in the `all` schedule the timed region is args.steps launches of the
-    # attention kernel and nothing else, so its average launch duration is ms
-    achieved = total_flops / (ms * 1e-3) / 1e12
+    rows = {}
+    if not args.no_rows and not args.only_all:
+        del steps
+        rows = gpu_rows(torch, spa, ops, {"config1", "config2", "config4", "merge", "config5"}, args.steps, args.warmup)
+
+    launches = {"all": 1, "rank": P, "step": n_pairs}[head]
     line = {
         "metric": "fwd attn TFLOP/s + % bf16 MFMA peak, ring-step causal S=8K H32 D128",
         "value": round(tflops, 2),
@@ -376,29 +594,40 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "config 3: simulated ring P=8 on one GPU, bf16 B=1 S=8192 (8 chunks of 1024) H=32 D=128 causal, "
-                        "8 diagonal + 28 full block pairs in ring order, step merge, seed 2 N(0,1)*0.5; "
-                        "schedule 'all' (one launch walks every rank's ring)",
+                        "8 diagonal + 28 full block pairs in ring order, seed 2 N(0,1)*0.5; "
+                        f"schedule '{head}'" + (" (one launch holds every rank's ring; ring steps merge in the online softmax; a one-GPU fusion)" if head == "all" else ""),
             "flops_per_step": total_flops,
             "block_pairs": n_pairs,
         },
         "pct_of_bf16_mfma_peak": round(100.0 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
+        "protocol": {k2: m_all[k2] for k2 in ("settle_launches", "settle_ms", "cold_ms_per_step", "timed_blocks", "block_ms_min",
+                                              "block_ms_max", "timed_region_s") if k2 in m_all},
         "other_schedules": other,
         "roofline": {
             "bound": "mfma",
             "kernel": "flash_fwd16_kernel<bf16,128,2>",
-            "achieved": round(achieved, 2),
+            "achieved": round(tflops, 2),
             "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
-            "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
+            "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
             "traffic": traffic,
-            "avg_launch_us": round(ms * 1e3, 2),
-            "flops_per_launch": total_flops,
-            "launches_per_step": 1,
-            "algorithmic_bytes_per_launch": algorithmic_bytes(),
+            "traffic_source": traffic_src,
+            "avg_launch_us": round(ms * 1e3 / launches, 2),
+            "flops_per_launch": total_flops / launches,
+            "launches_per_step": launches,
+            "algorithmic_bytes_per_launch": algorithmic_bytes() / launches,
         },
     }
+    if "step" in other:
+        line["ring_step"] = {"what": "the per-ring-step schedule (one launch per (rank, step), merge in the epilogue): what a rank of a real ring runs",
+                             "tflops": other["step"]["tflops"], "pct_of_bf16_mfma_peak": other["step"]["pct_of_bf16_mfma_peak"],
+                             "avg_launch_us": other["step"]["avg_launch_us"]}
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(torch)
+        cpu = CpuLegs(torch)
+        line["cpu_baseline"] = cpu.ring_forward(B, H, S // P, D, P, P * (P - 1) // 2, SEED, "config 3")
+        attach_cpu(rows, cpu)
+    if rows:
+        line["rows"] = list(rows.values())
     print(json.dumps(line))
 
 

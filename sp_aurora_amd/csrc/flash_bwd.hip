@@ -353,7 +353,9 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
 #pragma unroll
     for (int list = 0; list < 2; ++list) {
       const int key0 = (2 * i + list) * 32;  // first key of the half-tile whose dS is formed in this list
-      if (p.causal && key0 + 31 > qw0) {     // diagonal: hide the keys after each lane's query
+      // diagonal: hide the keys after each lane's query; last tile: hide the keys past the end (their K
+      // and V rows arrive as zeros, but P = exp(0 - lse) overflows for lse < -88 and inf * 0 is NaN)
+      if ((p.causal && key0 + 31 > qw0) || key0 + 31 >= p.Sk) {
 #pragma unroll
         for (int v = 0; v < 16; ++v)
           if (key0 + 8 * (v >> 2) + 4 * hh + (v & 3) > lim) sc[v] = -INFINITY;
@@ -407,7 +409,9 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
     }
   }
   wait_loads_but<0>();  // nothing may still be writing LDS when the workgroup ends
-  if (MIXED) asm volatile("s_nop 15\n s_nop 15" ::: "memory");  // the last MFMAs must have written dq before it is read
+  // The last MFMAs must have written dq before it is read.  The accumulators are operands of the
+  // wait, so no read of them can be scheduled above it.
+  if constexpr (MIXED) asm volatile("s_nop 15\n s_nop 15" : "+a"(dq[0]), "+a"(dq[1]), "+a"(dq[2]), "+a"(dq[3])::"memory");
 
   if (qrow < p.Sq) {
     float* dqp = p.dq + b * p.dqs.b + h * p.dqs.h + (int64_t)qrow * p.dqs.s;
@@ -675,8 +679,11 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
     }
     wait_loads_but<0>();
   }
-  // the last MFMAs must have written dk / dv before they are read
-  if (MIXED) asm volatile("s_nop 15\n s_nop 15" ::: "memory");
+  // The last MFMAs must have written dk / dv before they are read; the accumulators are operands of
+  // the wait, so no read of them can be scheduled above it.
+  if constexpr (MIXED)
+    asm volatile("s_nop 15\n s_nop 15"
+                 : "+a"(dk[0]), "+a"(dk[1]), "+a"(dk[2]), "+a"(dk[3]), "+a"(dv[0]), "+a"(dv[1]), "+a"(dv[2]), "+a"(dv[3])::"memory");
 
   if (krow < p.Sk) {
     float* dkp = p.dk + b * p.dks.b + h * p.dks.h + (int64_t)krow * p.dks.s;

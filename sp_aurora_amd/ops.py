@@ -217,22 +217,37 @@ def bwd_delta(out, dout, layout="bshd"):
 def flash_bwd(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, softmax_scale=None, causal=False,
               layout="bshd"):
     """Block-wise backward of one (q chunk, kv chunk) pair; adds into fp32 dq/dk/dv accumulators."""
-    lib = _lib.load()
-    q, k, v, dout = _prep(q), _prep(k), _prep(v), _prep(dout)
-    (B, H, Sq, D), qs = _bhs(q, layout)
-    (_, _, Sk, _), ks = _bhs(k, layout)
-    _, vs = _bhs(v, layout)
-    _, dos = _bhs(dout, layout)
-    _, dqs = _bhs(dq_acc, layout)
-    _, dks = _bhs(dk_acc, layout)
-    _, dvs = _bhs(dv_acc, layout)
+    if not (q.dtype == k.dtype == v.dtype == dout.dtype):
+        raise TypeError("flash_bwd: q, k, v, dout must share a dtype")
+    (B, H, Sq, D), _ = _bhs(q, layout)
+    shp_k, shp_v, shp_do = _bhs(k, layout)[0], _bhs(v, layout)[0], _bhs(dout, layout)[0]
+    shp_dq, dqs = _bhs(dq_acc, layout)
+    shp_dk, dks = _bhs(dk_acc, layout)
+    shp_dv, dvs = _bhs(dv_acc, layout)
+    Sk = shp_k[2]
+    # the kernels index every tensor with these sizes: a mismatch would be an out-of-bounds access
+    if shp_k != (B, H, Sk, D) or shp_v != shp_k:
+        raise ValueError(f"flash_bwd: shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    if shp_do != (B, H, Sq, D) or shp_dq != (B, H, Sq, D):
+        raise ValueError(f"flash_bwd: dout {tuple(dout.shape)} and dq_acc {tuple(dq_acc.shape)} must have q's shape {tuple(q.shape)}")
+    if shp_dk != shp_k or shp_dv != shp_k:
+        raise ValueError(f"flash_bwd: dk_acc {tuple(dk_acc.shape)} and dv_acc {tuple(dv_acc.shape)} must have k's shape {tuple(k.shape)}")
+    if tuple(lse.shape) != (B, H, Sq) or tuple(delta.shape) != (B, H, Sq):
+        raise ValueError(f"flash_bwd: lse {tuple(lse.shape)} and delta {tuple(delta.shape)} must be [B,H,Sq] = {(B, H, Sq)}")
     if softmax_scale is None:
         softmax_scale = D ** (-0.5)
     for t in (dq_acc, dk_acc, dv_acc, lse, delta):
         if t.dtype != torch.float32:
             raise TypeError("flash_bwd: accumulators, lse and delta must be float32")
+        if t.device != q.device:
+            raise ValueError("flash_bwd: every tensor must live on q's device")
     if not (lse.is_contiguous() and delta.is_contiguous()):
         raise ValueError("flash_bwd: lse and delta must be contiguous [B,H,Sq]")
+    lib = _lib.load()
+    q, k, v, dout = _prep(q), _prep(k), _prep(v), _prep(dout)
+    qs, ks, vs, dos = _bhs(q, layout)[1], _bhs(k, layout)[1], _bhs(v, layout)[1], _bhs(dout, layout)[1]
+    if not (_rows_ok(dq_acc, 4) and _rows_ok(dk_acc, 4) and _rows_ok(dv_acc, 4)):
+        raise ValueError("flash_bwd: accumulators need an inner stride of 1 and 16-byte aligned rows")
     with torch.cuda.device(q.device):
         _lib.check(lib.spa_flash_bwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
@@ -246,6 +261,23 @@ def flash_bwd(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, softmax_scale=N
 
 
 # ------------------------------------------------------------------ variable-length batches
+def check_cu_seqlens(cu, total, max_seqlen, what):
+    """One host-side look at a cu_seqlens array (a device-to-host read): offsets start at 0, never
+    decrease, end at `total` rows, and no sequence is longer than `max_seqlen`.  The kernels trust
+    these values when they index the packed tensors, so a bad array would be an out-of-bounds access."""
+    c = cu.detach().to("cpu", torch.int64)
+    if c.dim() != 1 or c.numel() < 2:
+        raise ValueError(f"{what} must be a 1-D tensor of nseq + 1 offsets, got {tuple(cu.shape)}")
+    lens = c[1:] - c[:-1]
+    if int(c[0]) != 0 or bool((lens < 0).any()):
+        raise ValueError(f"{what} must start at 0 and never decrease")
+    if int(c[-1]) != int(total):
+        raise ValueError(f"{what} ends at {int(c[-1])}, the packed tensor has {int(total)} rows")
+    if int(lens.max()) > int(max_seqlen):
+        raise ValueError(f"{what}: longest sequence {int(lens.max())} exceeds max_seqlen {int(max_seqlen)}")
+
+
+
 def _thd(t, what):
     """(rows, H, D) sizes and (head, row) element strides of a packed 3-D tensor."""
     if t.dim() != 3:
@@ -298,20 +330,32 @@ def flash_bwd_varlen(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, cu_seqle
                      max_seqlen_k, softmax_scale=None, causal=False):
     """Backward of flash_fwd_varlen; adds into the fp32 accumulators dq [total_q,H,D], dk, dv
     [total_k,H,D].  lse, delta: fp32 [H,total_q].  Calls spa_flash_bwd_varlen."""
-    lib = _lib.load()
-    q, k, v, dout = _prep(q), _prep(k), _prep(v), _prep(dout)
-    (Tq, H, D), qs = _thd(q, "q")
-    (Tk, _, _), ks = _thd(k, "k")
-    _, vs = _thd(v, "v")
-    _, dos = _thd(dout, "dout")
-    _, dqs = _thd(dq_acc, "dq_acc")
-    _, dks = _thd(dk_acc, "dk_acc")
-    _, dvs = _thd(dv_acc, "dv_acc")
+    if not (q.dtype == k.dtype == v.dtype == dout.dtype):
+        raise TypeError("flash_bwd_varlen: q, k, v, dout must share a dtype")
+    (Tq, H, D), _ = _thd(q, "q")
+    shp_k, shp_v, shp_do = _thd(k, "k")[0], _thd(v, "v")[0], _thd(dout, "dout")[0]
+    shp_dq, dqs = _thd(dq_acc, "dq_acc")
+    shp_dk, dks = _thd(dk_acc, "dk_acc")
+    shp_dv, dvs = _thd(dv_acc, "dv_acc")
+    Tk = shp_k[0]
+    if shp_k != (Tk, H, D) or shp_v != shp_k or shp_dk != shp_k or shp_dv != shp_k:
+        raise ValueError(f"flash_bwd_varlen: k {shp_k}, v {shp_v}, dk_acc {shp_dk}, dv_acc {shp_dv} must agree (heads and head dim as q {tuple(q.shape)})")
+    if shp_do != (Tq, H, D) or shp_dq != (Tq, H, D):
+        raise ValueError(f"flash_bwd_varlen: dout {shp_do} and dq_acc {shp_dq} must have q's shape {tuple(q.shape)}")
     for t in (dq_acc, dk_acc, dv_acc, lse, delta):
         if t.dtype != torch.float32:
             raise TypeError("accumulators, lse and delta must be float32")
+        if t.device != q.device:
+            raise ValueError("flash_bwd_varlen: every tensor must live on q's device")
     if tuple(lse.shape) != (H, Tq) or tuple(delta.shape) != (H, Tq) or not lse.is_contiguous() or not delta.is_contiguous():
         raise ValueError("lse and delta must be contiguous [H, total_q]")
+    if cu_seqlens_q.numel() != cu_seqlens_k.numel():
+        raise ValueError("cu_seqlens_q and cu_seqlens_k must describe the same number of sequences")
+    lib = _lib.load()
+    q, k, v, dout = _prep(q), _prep(k), _prep(v), _prep(dout)
+    qs, ks, vs, dos = _thd(q, "q")[1], _thd(k, "k")[1], _thd(v, "v")[1], _thd(dout, "dout")[1]
+    if not (_rows_ok(dq_acc, 4) and _rows_ok(dk_acc, 4) and _rows_ok(dv_acc, 4)):
+        raise ValueError("flash_bwd_varlen: accumulators need an inner stride of 1 and 16-byte aligned rows")
     cu_q, cu_k = _cu(cu_seqlens_q, q.device, "cu_seqlens_q"), _cu(cu_seqlens_k, q.device, "cu_seqlens_k")
     if softmax_scale is None:
         softmax_scale = D ** (-0.5)

@@ -61,6 +61,12 @@ def sp_aurora_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k=None, max_seqlen=N
         max_seqlen = int((cu_seqlens_q[1:] - cu_seqlens_q[:-1]).max())
     if max_seqlen_k is None:
         max_seqlen_k = max_seqlen if cu_seqlens_k is cu_seqlens_q else int((cu_seqlens_k[1:] - cu_seqlens_k[:-1]).max())
+    # the kernels index q/k/v with these offsets: look at them once on the host
+    ops.check_cu_seqlens(cu_seqlens_q, q.shape[0], max_seqlen, "cu_seqlens_q")
+    if cu_seqlens_k is not cu_seqlens_q or k.shape[0] != q.shape[0] or max_seqlen_k != max_seqlen:
+        ops.check_cu_seqlens(cu_seqlens_k, k.shape[0], max_seqlen_k, "cu_seqlens_k")
+    if cu_seqlens_q.numel() != cu_seqlens_k.numel():
+        raise ValueError("cu_seqlens_q and cu_seqlens_k must describe the same number of sequences")
     return VarlenFlashAttnFunc.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen, max_seqlen_k, softmax_scale,
                                      causal, return_attn_probs)
 

@@ -138,3 +138,69 @@ def test_unsupported_features_raise_before_any_launch():
         spa.sp_aurora_varlen_func(q[0], q[0], q[0], cu, cu, max_seqlen=8, dropout_p=0.1)
     with pytest.raises(ValueError, match="HIP device"):
         spa.sp_aurora_varlen_func(q[0], q[0], q[0], cu, cu, max_seqlen=8)
+
+
+def test_backward_wrappers_check_shapes_before_any_launch():
+    """The backward kernels index every tensor with q's and k's sizes; a mismatched call must be
+    refused on the host (here with CPU tensors: the shape checks come before the device check)."""
+    import torch
+    from sp_aurora_amd import ops
+    B, Sq, Sk, H, D = 1, 16, 24, 2, 64
+    mk = lambda *shape, dt=torch.bfloat16: torch.zeros(shape, dtype=dt)
+    good = dict(q=mk(B, Sq, H, D), k=mk(B, Sk, H, D), v=mk(B, Sk, H, D), dout=mk(B, Sq, H, D),
+                lse=mk(B, H, Sq, dt=torch.float32), delta=mk(B, H, Sq, dt=torch.float32),
+                dq_acc=mk(B, Sq, H, D, dt=torch.float32), dk_acc=mk(B, Sk, H, D, dt=torch.float32),
+                dv_acc=mk(B, Sk, H, D, dt=torch.float32))
+    with pytest.raises(ValueError, match="HIP device"):  # well-formed, but on the CPU
+        ops.flash_bwd(**good)
+    bad = {
+        "v": mk(B, Sk + 8, H, D), "dout": mk(B, Sq + 8, H, D), "dq_acc": mk(B, Sq - 8, H, D, dt=torch.float32),
+        "dk_acc": mk(B, Sk, H + 1, D, dt=torch.float32), "dv_acc": mk(B, Sq, H, D, dt=torch.float32),
+        "lse": mk(B, H, Sq + 1, dt=torch.float32), "delta": mk(B, H + 1, Sq, dt=torch.float32),
+        "k": mk(B, Sk, H, 2 * D),
+    }
+    for name, t in bad.items():
+        with pytest.raises(ValueError, match="shape|must have|must be"):
+            ops.flash_bwd(**{**good, name: t})
+    with pytest.raises(TypeError):
+        ops.flash_bwd(**{**good, "dout": mk(B, Sq, H, D, dt=torch.float16)})
+    with pytest.raises(TypeError):
+        ops.flash_bwd(**{**good, "lse": mk(B, H, Sq)})
+
+    # packed variable-length batches
+    Tq, Tk = 40, 48
+    cu_q = torch.tensor([0, 16, 40], dtype=torch.int32)
+    cu_k = torch.tensor([0, 24, 48], dtype=torch.int32)
+    vgood = dict(q=mk(Tq, H, D), k=mk(Tk, H, D), v=mk(Tk, H, D), dout=mk(Tq, H, D),
+                 lse=mk(H, Tq, dt=torch.float32), delta=mk(H, Tq, dt=torch.float32),
+                 dq_acc=mk(Tq, H, D, dt=torch.float32), dk_acc=mk(Tk, H, D, dt=torch.float32),
+                 dv_acc=mk(Tk, H, D, dt=torch.float32), cu_seqlens_q=cu_q, cu_seqlens_k=cu_k,
+                 max_seqlen_q=24, max_seqlen_k=24)
+    with pytest.raises(ValueError, match="HIP device"):
+        ops.flash_bwd_varlen(**vgood)
+    vbad = {"dout": mk(Tq + 1, H, D), "dk_acc": mk(Tk - 8, H, D, dt=torch.float32), "lse": mk(H, Tq + 4, dt=torch.float32),
+            "v": mk(Tk, H + 1, D), "cu_seqlens_k": torch.tensor([0, 48], dtype=torch.int32)}
+    for name, t in vbad.items():
+        with pytest.raises(ValueError):
+            ops.flash_bwd_varlen(**{**vgood, name: t})
+
+
+def test_cu_seqlens_are_checked_on_the_host():
+    import torch
+    from sp_aurora_amd import ops
+    ok = torch.tensor([0, 5, 5, 12], dtype=torch.int32)
+    ops.check_cu_seqlens(ok, 12, 7, "cu")
+    for cu, total, mx in [(torch.tensor([1, 5, 12]), 12, 12),      # does not start at 0
+                          (torch.tensor([0, 7, 5, 12]), 12, 12),   # decreases
+                          (ok, 16, 7),                             # does not end at the row count
+                          (ok, 12, 6),                             # longest sequence above max_seqlen
+                          (torch.tensor([0]), 0, 1)]:              # no sequence
+        with pytest.raises(ValueError):
+            ops.check_cu_seqlens(cu, total, mx, "cu")
+    # the public function refuses a bad array before touching the device
+    import sp_aurora_amd as spa
+    q = torch.zeros((12, 2, 64), dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="ends at"):
+        spa.sp_aurora_varlen_func(q, q, q, torch.tensor([0, 5, 10], dtype=torch.int32), max_seqlen=5)
+    with pytest.raises(ValueError, match="exceeds"):
+        spa.sp_aurora_varlen_func(q, q, q, torch.tensor([0, 5, 12], dtype=torch.int32), max_seqlen=5)
