@@ -80,6 +80,27 @@ int spa_flash_fwd(const void* q, const void* k, const void* v, void* out, float*
                   float scale, int mask_mode, int dtype, void* stream);
 
 /*
+ * spa_flash_fwd with K and V held as 8-bit floats (OCP e4m3, "float8_e4m3fn") plus one fp32
+ * dequantisation scale per (batch, head): K = k8 * k_scale[b*H + h], V = v8 * v_scale[b*H + h].
+ * q and out have element type `dtype` (SPA_BF16 or SPA_F16); k8, v8: [B,H,Sk,D] by strides in
+ * ELEMENTS (= bytes), rows 8-byte aligned; k_scale, v_scale: fp32 contiguous [B,H], positive.
+ * D in {64, 128}.  The tiles are widened to `dtype` between HBM and LDS (exact: every e4m3 value
+ * is a bf16 and an fp16 value), both contractions run on the 16-bit MFMAs with fp32 accumulation,
+ * k_scale is folded into the softmax scale and v_scale into the final normalisation, so the
+ * result is that of spa_flash_fwd on the dequantised tensors up to fp32 rounding.
+ * The reference has no 8-bit path; the call sites this serves are the ones that hand a KV cache
+ * to the attention operator: the variable-length adapter
+ * (sp_aurora/adapters/hf_adapter.py:141-155) and the call the variable-length tests are written
+ * against (test/flash_attention/test_intel_ring_flash_attn_varlen.py:23-26).
+ */
+int spa_flash_fwd_fp8kv(const void* q, const void* k8, const void* v8,
+                        const float* k_scale, const float* v_scale, void* out, float* lse,
+                        int B, int H, int Sq, int Sk, int D,
+                        const int64_t q_strides[3], const int64_t k_strides[3],
+                        const int64_t v_strides[3], const int64_t o_strides[3],
+                        float scale, int mask_mode, int dtype, void* stream);
+
+/*
  * Merge of one block result into the running (out_acc, lse_acc):
  *   lse' = logaddexp(lse, lse_b);  out' = out - sigmoid(lse_b - lse) * (out - out_b)
  * Replaces update_out_and_lse / _update_out_and_lse (sp_aurora/utils.py:47-147).
@@ -224,6 +245,19 @@ int spa_flash_fwd_varlen(const void* q, const void* k, const void* v, void* out,
                          const int64_t q_strides[2], const int64_t k_strides[2],
                          const int64_t v_strides[2], const int64_t o_strides[2],
                          float scale, int mask_mode, int dtype, void* stream);
+
+/*
+ * spa_flash_fwd_varlen with e4m3 K / V as in spa_flash_fwd_fp8kv: k8, v8 [total_k, H, D] by
+ * (head, row) strides in bytes, k_scale / v_scale fp32 contiguous [nseq, H] (one scale per
+ * sequence and head).  Same call sites as spa_flash_fwd_fp8kv.
+ */
+int spa_flash_fwd_varlen_fp8kv(const void* q, const void* k8, const void* v8,
+                               const float* k_scale, const float* v_scale, void* out, float* lse,
+                               const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                               int nseq, int H, int total_q, int total_k, int max_sq, int max_sk, int D,
+                               const int64_t q_strides[2], const int64_t k_strides[2],
+                               const int64_t v_strides[2], const int64_t o_strides[2],
+                               float scale, int mask_mode, int dtype, void* stream);
 
 /*
  * Backward of spa_flash_fwd_varlen, same packing.  lse and delta: fp32

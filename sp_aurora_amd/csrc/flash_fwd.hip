@@ -76,8 +76,14 @@ __device__ __forceinline__ int v_swizzle(int row) {
   return D == 128 ? (row & 3) << 2 : D == 64 ? ((row >> 1) & 1) << 2 : 0;
 }
 
-template <typename T, int D, int NG, bool SHARE>
+// KV8: K and V hold OCP e4m3 bytes (K = k8 * k_scale[b,h], V = v8 * v_scale[b,h]).  The tiles travel
+// global -> registers -> LDS and are widened to T on the way (every e4m3 value is exact in bf16 and
+// fp16), once per workgroup, so LDS holds the same swizzled 16-bit tiles as without KV8 and both
+// contractions run unchanged; k_scale folds into the softmax scale, v_scale into the final 1 / l.
+template <typename T, int D, int NG, bool SHARE, bool KV8 = false>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams pk) {
+  static_assert(!(KV8 && SHARE), "e4m3 K/V tiles are staged through registers per wave group");
+  typedef typename std::conditional<KV8, unsigned char, T>::type KVT;  // element type of K / V in memory
   typedef Fwd16Cfg<D, NG, SHARE> C;
   FwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
   typedef Mma16<T> M;
@@ -96,21 +102,24 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // Consecutive workgroup ids walk the (batch, head) pairs first: with round-robin placement of
   // workgroups on the 8 XCDs, all query tiles of a head share one XCD's L2 for K/V.
   // Then query tiles and ranks, heaviest first.
-  int bid = blockIdx.x;
-  const int bh = bid % (p.B * p.H);  // (batch, head) pairs first: each keeps to one XCD also when H < 8
-  bid /= p.B * p.H;
+  // (grid.x = (batch, head) pairs, grid.y = query tiles, grid.z = ranks: workgroups are dispatched
+  // x first, and the decomposition costs no divisions)
+  const int bh = blockIdx.x;  // (batch, head) pairs first: each keeps to one XCD also when H < 8
   const int h = bh % p.H;
   int b = bh / p.H;
-  const int qt = p.nqt - 1 - (bid % p.nqt);
-  const int rank = p.rank0 + p.nranks - 1 - bid / p.nqt;
+  // dequantisation scales of this (batch or sequence, head): K = k8 * ksc, V = v8 * vsc
+  const float ksc = KV8 ? p.k_scale[bh] : 1.f;
+  const float vsc = KV8 ? p.v_scale[bh] : 1.f;
+  const int qt = p.nqt - 1 - (int)blockIdx.y;
+  const int rank = p.rank0 + p.nranks - 1 - (int)blockIdx.z;
   const int q0 = qt * C::BMW;
   if (p.cu_q) {
     const int q_lo = p.cu_q[b], k_lo = p.cu_k[b];
     p.Sq = p.cu_q[b + 1] - q_lo;
     p.Sk = p.cu_k[b + 1] - k_lo;
     p.q = (const T*)p.q + (int64_t)q_lo * p.qs.s;
-    p.k = (const T*)p.k + (int64_t)k_lo * p.ks.s;
-    p.v = (const T*)p.v + (int64_t)k_lo * p.vs.s;
+    p.k = (const KVT*)p.k + (int64_t)k_lo * p.ks.s;
+    p.v = (const KVT*)p.v + (int64_t)k_lo * p.vs.s;
     p.out = (T*)p.out + (int64_t)q_lo * p.os.s;
     p.lse += q_lo;
     b = 0;
@@ -131,8 +140,8 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const int64_t qoff = (int64_t)rank * p.Sq;  // first row of this rank's query chunk
 
   const T* qp = (const T*)p.q + b * p.qs.b + h * p.qs.h + qoff * p.qs.s;
-  const T* kp = (const T*)p.k + b * p.ks.b + h * p.ks.h;
-  const T* vp = (const T*)p.v + b * p.vs.b + h * p.vs.h;
+  const KVT* kp = (const KVT*)p.k + b * p.ks.b + h * p.ks.h;
+  const KVT* vp = (const KVT*)p.v + b * p.vs.b + h * p.vs.h;
 
   const int qrow = qw0 + ln;
   const int qrow_c = qrow < p.Sq ? qrow : p.Sq - 1;
@@ -165,47 +174,11 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     int kend;   // one past the chunk's last row
     bool masked;
   };
-  auto locate = [&](int i) {
-    Sub r;
-    int t, j;
-    if (i < n_diag) {
-      t = 0;
-      j = i;
-      r.masked = true;
-    } else {
-      const int x = i - n_diag;
-      const int tt = x / npc;
-      t = t_full0 + tt;
-      j = x - tt * npc;
-      r.masked = false;
-    }
-    int ch = (rank - t) % p.P;
-    ch = ch < 0 ? ch + p.P : ch;
-    r.krel = (j * KSTEP + (SHARE ? 0 : grp)) * FWD_BN;
-    r.krow = ch * p.Sk + r.krel;
-    r.kend = ch * p.Sk + p.Sk;
-    return r;
-  };
-  // The loop walks the sub-tiles in order with three cursors (softmax at i, V loads at i+2,
-  // K loads at i+3); a cursor steps without divisions.
+  // The loop walks the sub-tiles in order with three cursors (softmax at i, V loads at i+1,
+  // K loads at i+2); a cursor steps without divisions.
   struct Cursor {
     int i, j, t;
     Sub sb;
-  };
-  auto cursor_at = [&](int i) {
-    Cursor c;
-    c.i = i;
-    if (i < n_diag) {
-      c.t = 0;
-      c.j = i;
-    } else {
-      const int x = i - n_diag;
-      const int tt = x / npc;
-      c.t = t_full0 + tt;
-      c.j = x - tt * npc;
-    }
-    c.sb = locate(i);
-    return c;
   };
   auto cursor_next = [&](Cursor& c) {
     ++c.i;
@@ -238,13 +211,13 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // any tensor and stores zeros into a buffer nobody reads.
   constexpr unsigned OFF_NONE = 0x80000000u;
   const int drow = tg / C::CPR, dpos = tg % C::CPR;
-  const unsigned kdoff = (unsigned)((drow * p.ks.s + ((dpos ^ k_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(T));
-  const unsigned vdoff = (unsigned)((drow * p.vs.s + ((dpos ^ v_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(T));
-  const unsigned krow_b = (unsigned)(p.ks.s * (int64_t)sizeof(T));  // bytes per K row
-  const unsigned vrow_b = (unsigned)(p.vs.s * (int64_t)sizeof(T));
+  const unsigned kdoff = (unsigned)((drow * p.ks.s + ((dpos ^ k_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(KVT));
+  const unsigned vdoff = (unsigned)((drow * p.vs.s + ((dpos ^ v_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(KVT));
+  const unsigned krow_b = (unsigned)(p.ks.s * (int64_t)sizeof(KVT));  // bytes per K row
+  const unsigned vrow_b = (unsigned)(p.vs.s * (int64_t)sizeof(KVT));
   const int64_t rows_all = (int64_t)p.P * p.Sk;
-  const u32x4 krsrc = buffer_descriptor(kp, (unsigned)(((rows_all - 1) * p.ks.s + D) * (int64_t)sizeof(T)));
-  const u32x4 vrsrc = buffer_descriptor(vp, (unsigned)(((rows_all - 1) * p.vs.s + D) * (int64_t)sizeof(T)));
+  const u32x4 krsrc = buffer_descriptor(kp, (unsigned)(((rows_all - 1) * p.ks.s + D) * (int64_t)sizeof(KVT)));
+  const u32x4 vrsrc = buffer_descriptor(vp, (unsigned)(((rows_all - 1) * p.vs.s + D) * (int64_t)sizeof(KVT)));
   // LDS byte addresses of this group's buffers and of this wave's 1 KB share of a round
   const unsigned lds_group = (unsigned)(uintptr_t)(lds_u8*)smem + (SHARE ? 0 : grp * C::GROUP);
   const unsigned lds_wave = lds_group + (SHARE ? wave : w) * 1024;
@@ -252,25 +225,54 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   auto v_lds = [&](int i) { return (unsigned)(2 * C::TILEB + (i & 1) * C::TILEB); };
   // load number q of the pair (K sub-tile with first row k_row into buffer kb, V sub-tile v_row into vb)
   constexpr int NLOADS = 2 * C::NDMA;
+  // the same two descriptors as compiler-visible resources, for loads into registers
+  const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, (int)krsrc[2], 0x00020000);
+  const __amdgpu_buffer_rsrc_t vrs = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, (int)vrsrc[2], 0x00020000);
+  // KV8: a thread's 8 e4m3 bytes per slot wait in registers from the MFMA phase that loads them to
+  // the next VALU phase, which widens them and writes the 16-byte LDS slot (store_staged).
+  u32x2 stage[KV8 ? NLOADS : 1];
   auto load_one = [&](int q, bool kon, int k_row, unsigned kb, bool von, int v_row, unsigned vb) {
     if (q < C::NDMA) {
       const unsigned u = kon ? (unsigned)(k_row + q * C::RPD) * krow_b : OFF_NONE;
-      load_to_lds_b128(krsrc, kdoff + u, lds_wave + kb + q * (C::DTHREADS * 16));
+      if constexpr (KV8)
+        stage[q] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(krs, kdoff + u, 0, 0));
+      else
+        load_to_lds_b128(krsrc, kdoff + u, lds_wave + kb + q * (C::DTHREADS * 16));
     } else {
       const int r = q - C::NDMA;
       const unsigned u = von ? (unsigned)(v_row + r * C::RPD) * vrow_b : OFF_NONE;
-      load_to_lds_b128(vrsrc, vdoff + u, lds_wave + vb + r * (C::DTHREADS * 16));
+      if constexpr (KV8)
+        stage[q] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(vrs, vdoff + u, 0, 0));
+      else
+        load_to_lds_b128(vrsrc, vdoff + u, lds_wave + vb + r * (C::DTHREADS * 16));
     }
   };
-  auto load_k = [&](int i) {
-    const Sub sb = locate(i < n ? i : 0);
+  // 8 e4m3 bytes -> 8 elements of T, 16 bytes
+  auto widen = [&](u32x2 x) {
+    u32x4 r;
 #pragma unroll
-    for (int q = 0; q < C::NDMA; ++q) load_one(q, i < n, sb.krow, k_lds(i), false, 0, 0);
+    for (int i = 0; i < 2; ++i) {
+      if constexpr (std::is_same<T, __bf16>::value) {
+        r[2 * i] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(x[i], 1.0f, false));
+        r[2 * i + 1] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(x[i], 1.0f, true));
+      } else {
+        r[2 * i] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(x[i], 1.0f, false));
+        r[2 * i + 1] = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(x[i], 1.0f, true));
+      }
+    }
+    return r;
   };
-  auto load_v = [&](int i) {
-    const Sub sb = locate(i < n ? i : 0);
+  // the staged K sub-tile goes to the K buffer at kb, the staged V sub-tile to the V buffer at vb
+  // (slot of thread tg in round q: the 16 bytes the direct load would have written)
+  auto store_staged = [&](unsigned kb, unsigned vb) {
+    if constexpr (KV8) {
+      const unsigned slot = lds_group + (unsigned)tg * 16;
 #pragma unroll
-    for (int q = 0; q < C::NDMA; ++q) load_one(C::NDMA + q, false, 0, 0, i < n, sb.krow, v_lds(i));
+      for (int q = 0; q < NLOADS; ++q) {
+        const unsigned a = slot + (q < C::NDMA ? kb + q * (C::DTHREADS * 16) : vb + (q - C::NDMA) * (C::DTHREADS * 16));
+        *(__attribute__((address_space(3))) u32x4*)(lds_u8*)(uintptr_t)a = widen(stage[q]);
+      }
+    }
   };
   auto loads_landed = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };  // vmcnt(0)
 
@@ -300,7 +302,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     for (int v = 0; v < 16; ++v) o[i][v] = 0.f;
   float m_run = -INFINITY;  // reference row max of the raw scores (may lag the true max, see below)
   float l_run = 0.f;        // this lane's share of the running row sum
-  const float c = p.scale_log2;
+  const float c = p.scale_log2 * ksc;  // scores are q . k8: the scale of K rides on the softmax scale
 
   // per-lane LDS addresses of the operands of MFMA phase i: V(i) and K(i+1); computed before the
   // barrier that opens the phase
@@ -452,10 +454,41 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   };
 
   // ---- prologue: K(0), V(0), K(1) on their way into LDS together with Q into registers ----
-  load_k(0);
-  load_v(0);
-  load_k(1);
-  loads_landed();
+  // The three cursors of the loop (softmax at i, V loads at i + 1, K loads at i + 2) start at
+  // sub-tiles 0, 1, 2; the first loads take their rows from them (no divisions).
+  Cursor cs, cv, ck;
+  cs.i = 0;
+  cs.j = 0;
+  cs.t = n_diag > 0 ? 0 : t_full0;
+  {
+    int ch = rank - cs.t;
+    ch = ch < 0 ? ch + p.P : ch;
+    cs.sb.masked = n_diag > 0;
+    cs.sb.krel = (SHARE ? 0 : grp) * FWD_BN;
+    cs.sb.krow = ch * p.Sk + cs.sb.krel;
+    cs.sb.kend = ch * p.Sk + p.Sk;
+  }
+  cv = cs;
+  cursor_next(cv);
+  ck = cv;
+  cursor_next(ck);
+#pragma unroll
+  for (int q = 0; q < C::NDMA; ++q) load_one(q, 0 < n, cs.sb.krow, k_lds(0), false, 0, 0);            // K(0)
+#pragma unroll
+  for (int q = 0; q < C::NDMA; ++q) load_one(C::NDMA + q, false, 0, 0, 0 < n, cs.sb.krow, v_lds(0));   // V(0)
+  if constexpr (KV8) {
+    // K(0) goes to LDS now; V(0) stays staged together with K(1), loaded next, and both are written
+    // by the first VALU phase like every later pair
+#pragma unroll
+    for (int q = 0; q < C::NDMA; ++q)
+      *(__attribute__((address_space(3))) u32x4*)(lds_u8*)(uintptr_t)(lds_group + (unsigned)tg * 16 + k_lds(0) + q * (C::DTHREADS * 16)) = widen(stage[q]);
+  }
+#pragma unroll
+  for (int q = 0; q < C::NDMA; ++q) load_one(q, 1 < n, cv.sb.krow, k_lds(1), false, 0, 0);            // K(1)
+  // S(0) needs Q and K(0) only: loads complete in the order of issue, so at most the 2 NDMA loads
+  // of V(0) and K(1) may still be in flight here; they are waited for before the barrier that
+  // opens the first MFMA phase reading them.
+  __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * C::NDMA) & 15) | (((2 * C::NDMA) >> 4) << 14));  // vmcnt(2 NDMA)
   __syncthreads();
   {
     frag none[2][2];
@@ -464,7 +497,10 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     mfma_phase(std::false_type{}, std::true_type{}, va, ka, none, [](int) {});  // S(0)
   }
   __syncthreads();
-  if (NG > 1 && grp == 1) __syncthreads();  // group 1 runs one phase behind group 0
+  if (NG > 1 && grp == 1) {  // group 1 runs one phase behind group 0
+    loads_landed();          // (with shared buffers group 0 reads this group's share of V(0), K(1) after this barrier)
+    __syncthreads();
+  }
 
   // One loop, no branch around an MFMA, the same barriers per step for every wave of a group.  A wave
   // whose rows see none of a diagonal sub-tile's keys (at most the last two sub-tiles of the
@@ -475,7 +511,6 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // phase of the workgroup: group 0 during its MFMA phase, group 1 (one phase behind) at the start
   // of its VALU phase; each waits for its loads before the barrier two phases later.
   const bool early = SHARE && grp == 1;  // wave-uniform
-  Cursor cs = cursor_at(0), cv = cursor_at(1), ck = cursor_at(2);
   // The loop body comes in two copies, one per buffer parity of the step, so that every LDS address of
   // the MFMA phase is a per-lane constant plus an immediate offset (no address arithmetic per step).
   auto body = [&](auto parity, int i) __attribute__((always_inline)) {
@@ -497,6 +532,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     // at the end of its VALU phase, group 1 at the end of its MFMA phase, the same physical
     // barrier); the other one only holds the two groups in step, and they drift little without it.
     if (!early) loads_landed();
+    store_staged((unsigned)((PAR ^ 1) * C::TILEB), (unsigned)(2 * C::TILEB + PAR * C::TILEB));  // K(i + 1), V(i)
     if (!SHARE || !early) __syncthreads();
     __builtin_amdgcn_s_setprio(3);
     mfma_phase(std::true_type{}, std::true_type{}, va, ka, pf, [&](int j) {
@@ -526,6 +562,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     unsigned va[D / 32], ka[D / 16];
     operand_addresses(n - 1, va, ka);
     loads_landed();
+    store_staged(k_lds(n), v_lds(n - 1));  // V(n - 1) (and whatever K(n) stands for: never read)
     if (!SHARE || !early) __syncthreads();
     mfma_phase(std::true_type{}, std::false_type{}, va, ka, pf, [](int) {});
     if (!SHARE || early) __syncthreads();
@@ -574,6 +611,35 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   float* const ml = (float*)smem + NG * FWD_BM * TP;  // [NG][128](m, l), then lse_b[rows of the workgroup]
   float* const lsb = ml + NG * FWD_BM * 2;
   const int rloc = w * 32 + ln;
+  // The final pass walks the tile row-major, a thread owning 8 head dims of NIT rows; the CH lanes of
+  // a row share a wave.  A merging step fetches its pieces of the running (acc, lse) NOW, so that
+  // their latency passes under the exchange and the staging below instead of after them.
+  constexpr int CH = D / 8;                                   // 8-element chunks per row
+  constexpr int NIT = C::BMW * CH / (FWD_THREADS * NG);       // chunks per thread
+  constexpr int NPRE = NIT < 4 ? NIT : 4;                     // of which fetched before the staging
+  static_assert(NIT * FWD_THREADS * NG == C::BMW * CH, "the final pass must tile the workgroup's rows");
+  const int epi = p.epi;
+  const bool merging = epi >= SPA_EPI_MERGE;
+  f32x4 pa[NIT][2];
+  float pl[NIT];
+  auto acc_ptr = [&](int it, int& grow, int& ch) -> float* {
+    const int cidx = tid + it * (FWD_THREADS * NG);
+    const int row = cidx / CH;
+    ch = cidx % CH;
+    grow = q0 + row;
+    return p.acc + b * p.as.b + h * p.as.h + (int64_t)grow * p.as.s + ch * 8;
+  };
+  auto fetch_acc = [&](int it) {
+    int grow, ch;
+    const float* ap = acc_ptr(it, grow, ch);
+    if (merging && grow < p.Sq) {
+      pa[it][0] = *(const f32x4*)ap;
+      pa[it][1] = *(const f32x4*)(ap + 4);
+      pl[it] = p.lse[((int64_t)b * p.H + h) * p.lse_bh + qoff + grow];
+    }
+  };
+#pragma unroll
+  for (int it = 0; it < NPRE; ++it) fetch_acc(it);
   const float l_own = halves_sum(l_run);
   float scale, lse_b;
   if (NG > 1 && !SHARE) {
@@ -588,10 +654,10 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     const float a1 = fast_exp2((m_run - m_all) * c);
     const float a2 = fast_exp2((m2 - m_all) * c);
     const float l_all = l_own * a1 + l2 * a2;
-    scale = a1 / l_all;
+    scale = a1 * vsc / l_all;
     lse_b = (m_all * c + fast_log2(l_all)) * 0.6931471805599453f;
   } else {
-    scale = 1.f / l_own;
+    scale = vsc / l_own;
     lse_b = (m_run * c + fast_log2(l_own)) * 0.6931471805599453f;
   }
 #pragma unroll
@@ -607,13 +673,15 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     }
   if ((SHARE || grp == 0) && hh == 0) lsb[(SHARE ? grp * FWD_BM : 0) + rloc] = lse_b;
   __syncthreads();
+#pragma unroll
+  for (int it = NPRE; it < NIT; ++it) fetch_acc(it);  // the accumulators are staged: registers are free for the rest
   {
-    constexpr int CH = D / 8;  // 8-element chunks per row; the CH lanes of a row share a wave
     const float* t0 = (const float*)smem;
-    const int epi = p.epi;
-    for (int cidx = tid; cidx < C::BMW * CH; cidx += FWD_THREADS * NG) {
-      const int row = cidx / CH, ch = cidx % CH;
-      const int grow = q0 + row;
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      int grow, ch;
+      float* ap = acc_ptr(it, grow, ch);
+      const int row = grow - q0;
       if (grow >= p.Sq) continue;
       float x[8];
       {
@@ -631,11 +699,10 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       }
       float lb = lsb[row];
       const int64_t li = ((int64_t)b * p.H + h) * p.lse_bh + qoff + grow;
-      float* ap = p.acc + b * p.as.b + h * p.as.h + (int64_t)grow * p.as.s + ch * 8;
-      if (epi >= SPA_EPI_MERGE) {  // merge with the running accumulators (sp_aurora/utils.py:103-104)
-        const float la = p.lse[li];
-        const f32x4 a = *(const f32x4*)ap;
-        const f32x4 bq = *(const f32x4*)(ap + 4);
+      if (merging) {  // merge with the running accumulators (sp_aurora/utils.py:103-104)
+        const float la = pl[it];
+        const f32x4 a = pa[it][0];
+        const f32x4 bq = pa[it][1];
         const float xa[8] = {a[0], a[1], a[2], a[3], bq[0], bq[1], bq[2], bq[3]};
         const float d = lb - la;
         float wgt, ln_;
@@ -701,11 +768,9 @@ __global__ void __launch_bounds__(FWD_THREADS, 1) flash_fwd32_kernel(const FwdPa
   const int ln = lane & 31;
   const int hh = lane >> 5;
 
-  int bid = blockIdx.x;
-  const int h = bid % p.H;
-  bid /= p.H;
-  const int qt = p.nqt - 1 - (bid % p.nqt);
-  int b = bid / p.nqt;
+  const int h = blockIdx.x % p.H;
+  int b = blockIdx.x / p.H;
+  const int qt = p.nqt - 1 - (int)blockIdx.y;
   const int q0 = qt * FWD_BM;
   const int qw0 = q0 + w * 32;
   if (p.cu_q) {
@@ -888,7 +953,8 @@ template <auto kernel>
 hipError_t launch(int threads, int smem, const FwdParams& p, hipStream_t stream) {
   const hipError_t e = spa_allow_dynamic_lds<kernel>(smem);
   if (e != hipSuccess) return e;
-  const dim3 grid((unsigned)((int64_t)p.B * p.H * p.nqt * p.nranks));
+  if (p.nqt > 65535 || p.nranks > 65535) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)((int64_t)p.B * p.H), (unsigned)p.nqt, (unsigned)p.nranks);
   hipLaunchKernelGGL(kernel, grid, dim3(threads), smem, stream, p);
   return hipGetLastError();
 }
@@ -914,11 +980,31 @@ hipError_t launch16(FwdParams p, hipStream_t stream) {
   return launch<flash_fwd16_kernel<T, D, 1, false>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
 }
 
+// e4m3 K/V: the register-staged variants (no shared-buffer form).
+template <typename T, int D>
+hipError_t launch16_kv8(FwdParams p, hipStream_t stream) {
+  const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
+  const bool two = force ? force == 2 : p.Sk > FWD_BN;
+  if (two) return launch<flash_fwd16_kernel<T, D, 2, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+  return launch<flash_fwd16_kernel<T, D, 1, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+}
+
 }  // namespace
 
 // Returns hipSuccess, or hipErrorInvalidValue for an unsupported (dtype, D).
 hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream) {
   p.nqt = (p.Sq + FWD_BM - 1) / FWD_BM;
+  if (p.k_scale) {  // K / V are e4m3 bytes, q / out of type `dtype`
+    if (!p.v_scale) return hipErrorInvalidValue;
+    if (dtype == 1) {
+      if (D == 128) return launch16_kv8<__bf16, 128>(p, stream);
+      if (D == 64) return launch16_kv8<__bf16, 64>(p, stream);
+    } else if (dtype == 2) {
+      if (D == 128) return launch16_kv8<_Float16, 128>(p, stream);
+      if (D == 64) return launch16_kv8<_Float16, 64>(p, stream);
+    }
+    return hipErrorInvalidValue;
+  }
   if (dtype == 1) {
     if (D == 128) return launch16<__bf16, 128>(p, stream);
     if (D == 64) return launch16<__bf16, 64>(p, stream);

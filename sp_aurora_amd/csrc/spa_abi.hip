@@ -95,24 +95,42 @@ int spa_device_info(char* buf, int n) {
   return SPA_OK;
 }
 
-int spa_flash_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int B, int H, int Sq,
-                  int Sk, int D, const int64_t q_strides[3], const int64_t k_strides[3],
-                  const int64_t v_strides[3], const int64_t o_strides[3], float scale, int mask_mode,
-                  int dtype, void* stream) {
-  if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "spa_flash_fwd: null pointer");
-  if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(SPA_EINVAL, "spa_flash_fwd: null strides");
-  if (!dims_ok(B, H, Sq, D) || Sk <= 0) return fail(SPA_EINVAL, "spa_flash_fwd: sizes must be positive (B=%d H=%d Sq=%d Sk=%d D=%d)", B, H, Sq, Sk, D);
-  if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "spa_flash_fwd: bad dtype %d", dtype);
-  if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "spa_flash_fwd: bad mask_mode %d", mask_mode);
-  if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "spa_flash_fwd: softmax scale must be positive and finite");
-  if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "spa_flash_fwd: head dim %d not in {32,64,128}", D);
-  const int esz = elem_size(dtype);
-  if (!aligned16(q, q_strides, esz) || !aligned16(k, k_strides, esz) || !aligned16(v, v_strides, esz) ||
-      !aligned16(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0)
-    return fail(SPA_EALIGN, "spa_flash_fwd: pointers and row strides must be 16-byte aligned");
-  if ((int64_t)B * H * ((Sq + 127) / 128) > 0x7fffffffLL) return fail(SPA_EINVAL, "spa_flash_fwd: grid too large");
-  if (!span_ok(Sk, k_strides[2], D, esz) || !span_ok(Sk, v_strides[2], D, esz))
-    return fail(SPA_EUNSUPPORTED, "spa_flash_fwd: K/V of one (batch, head) span more than 2 GiB");
+}  // extern "C"
+
+namespace {
+
+// 8-byte alignment of an e4m3 tensor's base and rows (a thread moves 8 elements at a time).
+bool aligned8(const void* p, const int64_t* s, int n) {
+  if (((uintptr_t)p & 7) != 0) return false;
+  for (int i = 0; i < n; ++i)
+    if (s[i] % 8 != 0) return false;
+  return true;
+}
+
+// k_scale / v_scale non-null: K and V are e4m3 bytes (strides in bytes), q / out of type `dtype`.
+int flash_fwd(const char* what, const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+              void* out, float* lse, int B, int H, int Sq, int Sk, int D, const int64_t q_strides[3],
+              const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3], float scale,
+              int mask_mode, int dtype, void* stream) {
+  const bool kv8 = k_scale || v_scale;
+  if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "%s: null pointer", what);
+  if (kv8 && (!k_scale || !v_scale)) return fail(SPA_EINVAL, "%s: null scale pointer", what);
+  if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(SPA_EINVAL, "%s: null strides", what);
+  if (!dims_ok(B, H, Sq, D) || Sk <= 0) return fail(SPA_EINVAL, "%s: sizes must be positive (B=%d H=%d Sq=%d Sk=%d D=%d)", what, B, H, Sq, Sk, D);
+  if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "%s: bad dtype %d", what, dtype);
+  if (kv8 && dtype == SPA_F32) return fail(SPA_EUNSUPPORTED, "%s: e4m3 K/V go with bf16 or fp16 queries", what);
+  if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "%s: bad mask_mode %d", what, mask_mode);
+  if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "%s: softmax scale must be positive and finite", what);
+  if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "%s: head dim %d not in {32,64,128}", what, D);
+  if (kv8 && D == 32) return fail(SPA_EUNSUPPORTED, "%s: e4m3 K/V need head dim 64 or 128", what);
+  const int esz = elem_size(dtype), kesz = kv8 ? 1 : esz;
+  const bool kv_aligned = kv8 ? aligned8(k, k_strides, 3) && aligned8(v, v_strides, 3) && (((uintptr_t)k_scale | (uintptr_t)v_scale) & 3) == 0
+                              : aligned16(k, k_strides, esz) && aligned16(v, v_strides, esz);
+  if (!aligned16(q, q_strides, esz) || !kv_aligned || !aligned16(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0)
+    return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned (8-byte for e4m3 K/V)", what);
+  if ((int64_t)B * H > 0x7fffffffLL || (Sq + 127) / 128 > 65535) return fail(SPA_EINVAL, "%s: grid too large", what);
+  if (!span_ok(Sk, k_strides[2], D, kesz) || !span_ok(Sk, v_strides[2], D, kesz))
+    return fail(SPA_EUNSUPPORTED, "%s: K/V of one (batch, head) span more than 2 GiB", what);
   FwdParams p;
   p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
   p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
@@ -127,7 +145,29 @@ int spa_flash_fwd(const void* q, const void* k, const void* v, void* out, float*
   p.epi = SPA_EPI_PLAIN;
   p.P = 1; p.rank0 = 0; p.nranks = 1; p.t_begin = 0; p.t_count = -1;
   p.cu_q = nullptr; p.cu_k = nullptr;
-  return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), "spa_flash_fwd");
+  p.k_scale = k_scale; p.v_scale = v_scale;
+  return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), what);
+}
+
+}  // namespace
+
+extern "C" {
+
+int spa_flash_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int B, int H, int Sq,
+                  int Sk, int D, const int64_t q_strides[3], const int64_t k_strides[3],
+                  const int64_t v_strides[3], const int64_t o_strides[3], float scale, int mask_mode,
+                  int dtype, void* stream) {
+  return flash_fwd("spa_flash_fwd", q, k, v, nullptr, nullptr, out, lse, B, H, Sq, Sk, D, q_strides, k_strides, v_strides,
+                   o_strides, scale, mask_mode, dtype, stream);
+}
+
+int spa_flash_fwd_fp8kv(const void* q, const void* k8, const void* v8, const float* k_scale, const float* v_scale,
+                        void* out, float* lse, int B, int H, int Sq, int Sk, int D, const int64_t q_strides[3],
+                        const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
+                        float scale, int mask_mode, int dtype, void* stream) {
+  if (!k_scale || !v_scale) return fail(SPA_EINVAL, "spa_flash_fwd_fp8kv: null scale pointer");
+  return flash_fwd("spa_flash_fwd_fp8kv", q, k8, v8, k_scale, v_scale, out, lse, B, H, Sq, Sk, D, q_strides, k_strides,
+                   v_strides, o_strides, scale, mask_mode, dtype, stream);
 }
 
 int spa_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* blk_lse, int B, int H, int Sq,
@@ -205,7 +245,7 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, void
     return fail(SPA_EINVAL, "%s: these sizes need %lld bytes of scratch, the built-in buffer holds %lld", what,
                 (long long)spa_ring_fwd_workspace_bytes(B, H, S, D, P, dtype), (long long)ws_bytes);
   const int r_lo = rank < 0 ? 0 : rank, r_hi = rank < 0 ? P : rank + 1;
-  if ((int64_t)B * H * ((s + 127) / 128) * (r_hi - r_lo) > 0x7fffffffLL) return fail(SPA_EINVAL, "%s: grid too large", what);
+  if ((int64_t)B * H > 0x7fffffffLL || (s + 127) / 128 > 65535 || r_hi - r_lo > 65535) return fail(SPA_EINVAL, "%s: grid too large", what);
   hipStream_t st = (hipStream_t)stream;
 
   // workspace carve-up; the running output of one rank is laid out [B, s, H, D]
@@ -230,6 +270,7 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, void
   p.P = P;
   p.epi = SPA_EPI_PLAIN;
   p.cu_q = nullptr; p.cu_k = nullptr;
+  p.k_scale = nullptr; p.v_scale = nullptr;
 
   if (fuse == SPA_RING_ALL_RANKS) {  // one launch: every requested rank, every step
     p.rank0 = r_lo; p.nranks = r_hi - r_lo; p.t_begin = 0; p.t_count = -1;
@@ -428,28 +469,37 @@ int varlen_sizes_ok(const char* what, const void* cu_q, const void* cu_k, int ns
   if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "%s: bad mask_mode %d", what, mask_mode);
   if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "%s: softmax scale must be positive and finite", what);
   if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "%s: head dim %d not in {32,64,128}", what, D);
-  if ((int64_t)nseq * H * ((max_sq + 127) / 128) > 0x7fffffffLL || (int64_t)nseq * H * ((max_sk + 127) / 128) > 0x7fffffffLL)
+  if ((max_sq + 127) / 128 > 65535 || (int64_t)nseq * H * ((max_sq + 127) / 128) > 0x7fffffffLL ||
+      (int64_t)nseq * H * ((max_sk + 127) / 128) > 0x7fffffffLL)
     return fail(SPA_EINVAL, "%s: grid too large", what);
   return SPA_OK;
 }
 }  // namespace
 
-int spa_flash_fwd_varlen(const void* q, const void* k, const void* v, void* out, float* lse,
-                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int nseq, int H, int total_q,
-                         int total_k, int max_sq, int max_sk, int D, const int64_t q_strides[2],
-                         const int64_t k_strides[2], const int64_t v_strides[2], const int64_t o_strides[2],
-                         float scale, int mask_mode, int dtype, void* stream) {
-  if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "spa_flash_fwd_varlen: null pointer");
-  if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(SPA_EINVAL, "spa_flash_fwd_varlen: null strides");
-  const int rc = varlen_sizes_ok("spa_flash_fwd_varlen", cu_seqlens_q, cu_seqlens_k, nseq, H, total_q, total_k, max_sq,
-                                 max_sk, D, dtype, mask_mode, scale);
+}  // extern "C"
+
+namespace {
+int flash_fwd_varlen(const char* what, const void* q, const void* k, const void* v, const float* k_scale,
+                     const float* v_scale, void* out, float* lse, const int32_t* cu_seqlens_q,
+                     const int32_t* cu_seqlens_k, int nseq, int H, int total_q, int total_k, int max_sq, int max_sk,
+                     int D, const int64_t q_strides[2], const int64_t k_strides[2], const int64_t v_strides[2],
+                     const int64_t o_strides[2], float scale, int mask_mode, int dtype, void* stream) {
+  const bool kv8 = k_scale || v_scale;
+  if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "%s: null pointer", what);
+  if (kv8 && (!k_scale || !v_scale)) return fail(SPA_EINVAL, "%s: null scale pointer", what);
+  if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(SPA_EINVAL, "%s: null strides", what);
+  const int rc = varlen_sizes_ok(what, cu_seqlens_q, cu_seqlens_k, nseq, H, total_q, total_k, max_sq, max_sk, D, dtype,
+                                 mask_mode, scale);
   if (rc != SPA_OK) return rc;
-  const int esz = elem_size(dtype);
-  if (!aligned16v(q, q_strides, esz) || !aligned16v(k, k_strides, esz) || !aligned16v(v, v_strides, esz) ||
-      !aligned16v(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0)
-    return fail(SPA_EALIGN, "spa_flash_fwd_varlen: pointers and row strides must be 16-byte aligned");
-  if (!span_ok(max_sk, k_strides[1], D, esz) || !span_ok(max_sk, v_strides[1], D, esz))
-    return fail(SPA_EUNSUPPORTED, "spa_flash_fwd_varlen: K/V of one (sequence, head) span more than 2 GiB");
+  if (kv8 && dtype == SPA_F32) return fail(SPA_EUNSUPPORTED, "%s: e4m3 K/V go with bf16 or fp16 queries", what);
+  if (kv8 && D == 32) return fail(SPA_EUNSUPPORTED, "%s: e4m3 K/V need head dim 64 or 128", what);
+  const int esz = elem_size(dtype), kesz = kv8 ? 1 : esz;
+  const bool kv_aligned = kv8 ? aligned8(k, k_strides, 2) && aligned8(v, v_strides, 2) && (((uintptr_t)k_scale | (uintptr_t)v_scale) & 3) == 0
+                              : aligned16v(k, k_strides, esz) && aligned16v(v, v_strides, esz);
+  if (!aligned16v(q, q_strides, esz) || !kv_aligned || !aligned16v(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0)
+    return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned (8-byte for e4m3 K/V)", what);
+  if (!span_ok(max_sk, k_strides[1], D, kesz) || !span_ok(max_sk, v_strides[1], D, kesz))
+    return fail(SPA_EUNSUPPORTED, "%s: K/V of one (sequence, head) span more than 2 GiB", what);
   FwdParams p;
   p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
   p.B = nseq; p.H = H; p.Sq = max_sq; p.Sk = max_sk;
@@ -464,7 +514,33 @@ int spa_flash_fwd_varlen(const void* q, const void* k, const void* v, void* out,
   p.epi = SPA_EPI_PLAIN;
   p.P = 1; p.rank0 = 0; p.nranks = 1; p.t_begin = 0; p.t_count = -1;
   p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
-  return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), "spa_flash_fwd_varlen");
+  p.k_scale = k_scale; p.v_scale = v_scale;
+  return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), what);
+}
+}  // namespace
+
+extern "C" {
+
+int spa_flash_fwd_varlen(const void* q, const void* k, const void* v, void* out, float* lse,
+                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int nseq, int H, int total_q,
+                         int total_k, int max_sq, int max_sk, int D, const int64_t q_strides[2],
+                         const int64_t k_strides[2], const int64_t v_strides[2], const int64_t o_strides[2],
+                         float scale, int mask_mode, int dtype, void* stream) {
+  return flash_fwd_varlen("spa_flash_fwd_varlen", q, k, v, nullptr, nullptr, out, lse, cu_seqlens_q, cu_seqlens_k, nseq, H,
+                          total_q, total_k, max_sq, max_sk, D, q_strides, k_strides, v_strides, o_strides, scale,
+                          mask_mode, dtype, stream);
+}
+
+int spa_flash_fwd_varlen_fp8kv(const void* q, const void* k8, const void* v8, const float* k_scale,
+                               const float* v_scale, void* out, float* lse, const int32_t* cu_seqlens_q,
+                               const int32_t* cu_seqlens_k, int nseq, int H, int total_q, int total_k, int max_sq,
+                               int max_sk, int D, const int64_t q_strides[2], const int64_t k_strides[2],
+                               const int64_t v_strides[2], const int64_t o_strides[2], float scale, int mask_mode,
+                               int dtype, void* stream) {
+  if (!k_scale || !v_scale) return fail(SPA_EINVAL, "spa_flash_fwd_varlen_fp8kv: null scale pointer");
+  return flash_fwd_varlen("spa_flash_fwd_varlen_fp8kv", q, k8, v8, k_scale, v_scale, out, lse, cu_seqlens_q, cu_seqlens_k,
+                          nseq, H, total_q, total_k, max_sq, max_sk, D, q_strides, k_strides, v_strides, o_strides,
+                          scale, mask_mode, dtype, stream);
 }
 
 int spa_flash_bwd_varlen(const void* q, const void* k, const void* v, const void* dout, const float* lse,

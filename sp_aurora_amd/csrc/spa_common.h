@@ -40,6 +40,10 @@ struct FwdParams {
   // Sq and Sk are the longest sequence's sizes (they shape the grid) and lse is [H][lse_bh]
   const int* cu_q;
   const int* cu_k;
+  // e4m3 K/V (16-bit kernels; null: K and V have q's element type): K = k8 * k_scale[b*H + h],
+  // V = v8 * v_scale[b*H + h], fp32, one per (batch or sequence, head); strides of k, v in bytes
+  const float* k_scale;
+  const float* v_scale;
 };
 
 enum {

@@ -44,16 +44,54 @@ def _prep(t):
     return t if _rows_ok(t, t.element_size()) else t.contiguous()
 
 
+FP8 = torch.float8_e4m3fn  # OCP e4m3: the 8-bit K/V format of spa_flash_fwd_fp8kv
+
+
+def _fp8_scales(k, v, k_scale, v_scale, n_lead, H):
+    """Checks the (k8, v8, k_scale, v_scale) quadruple of an e4m3 K/V call; returns the scales as
+    contiguous fp32 [n_lead, H] tensors on k's device."""
+    if k.dtype != FP8 or v.dtype != FP8:
+        raise TypeError("e4m3 K/V: k and v must both be torch.float8_e4m3fn")
+    if k_scale is None or v_scale is None:
+        raise ValueError("e4m3 K/V need k_scale and v_scale (fp32, one per (batch or sequence, head))")
+    out = []
+    for name, sc in (("k_scale", k_scale), ("v_scale", v_scale)):
+        if tuple(sc.shape) != (n_lead, H):
+            raise ValueError(f"{name} must have shape {(n_lead, H)}, got {tuple(sc.shape)}")
+        out.append(sc.to(device=k.device, dtype=torch.float32).contiguous())
+    return out
+
+
+def quantize_fp8_per_head(x, layout="bshd"):
+    """x [B,S,H,D] (or [B,H,S,D]) -> (x8 e4m3 of the same shape, scale fp32 [B,H]) with
+    x ~= x8 * scale[b,h]: one absmax scale per (batch, head), 448 = the largest e4m3 value.
+    A convenience for producing the inputs of the e4m3 K/V entry points (torch ops)."""
+    dims = (1, 3) if layout == "bshd" else (2, 3)
+    amax = x.detach().abs().amax(dim=dims, keepdim=True).float().clamp_min(1e-12)
+    scale = amax / 448.0
+    x8 = (x.float() / scale).clamp(-448.0, 448.0).to(FP8)
+    return x8, scale.reshape(x.shape[0], -1).contiguous()
+
+
 def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
-def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None, lse=None):
-    """Block attention forward -> (out like q, lse fp32 [B,H,Sq]).  Calls spa_flash_fwd."""
+def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None, lse=None, k_scale=None, v_scale=None):
+    """Block attention forward -> (out like q, lse fp32 [B,H,Sq]).  Calls spa_flash_fwd, or
+    spa_flash_fwd_fp8kv when k, v are torch.float8_e4m3fn (then k_scale, v_scale fp32 [B,H] give
+    K = k * k_scale[b,h], V = v * v_scale[b,h]; q bf16 or fp16)."""
     lib = _lib.load()
-    q, k, v = _prep(q), _prep(k), _prep(v)
-    if not (q.dtype == k.dtype == v.dtype):
-        raise TypeError("q, k, v must share a dtype")
+    fp8 = k.dtype == FP8 or v.dtype == FP8
+    if fp8:
+        q = _prep(q)
+        k, v = [t if t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1]) and t.data_ptr() % 8 == 0 else t.contiguous() for t in (k, v)]
+        if not k.is_cuda or not v.is_cuda:
+            raise ValueError("sp_aurora_amd kernels need tensors on a HIP device (got a CPU tensor)")
+    else:
+        q, k, v = _prep(q), _prep(k), _prep(v)
+        if not (q.dtype == k.dtype == v.dtype):
+            raise TypeError("q, k, v must share a dtype")
     (B, H, Sq, D), qs = _bhs(q, layout)
     (Bk, Hk, Sk, Dk), ks = _bhs(k, layout)
     (Bv, Hv, Sv, Dv), vs = _bhs(v, layout)
@@ -66,13 +104,15 @@ def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None
     if lse is None:
         lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
     _, os_ = _bhs(out, layout)
+    tail = (B, H, Sq, Sk, D, _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
+            float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(q), _stream())
     with torch.cuda.device(q.device):
-        _lib.check(lib.spa_flash_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
-            B, H, Sq, Sk, D,
-            _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
-            float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE,
-            _dtype_code(q), _stream()))
+        if fp8:
+            ksc, vsc = _fp8_scales(k, v, k_scale, v_scale, B, H)
+            _lib.check(lib.spa_flash_fwd_fp8kv(q.data_ptr(), k.data_ptr(), v.data_ptr(), ksc.data_ptr(), vsc.data_ptr(),
+                                               out.data_ptr(), lse.data_ptr(), *tail))
+        else:
+            _lib.check(lib.spa_flash_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), *tail))
     return out, lse
 
 
@@ -294,14 +334,22 @@ def _cu(cu, device, what):
 
 
 def flash_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale=None,
-                     causal=False, out=None, lse=None):
+                     causal=False, out=None, lse=None, k_scale=None, v_scale=None):
     """Attention inside each sequence of a packed batch: q [total_q,H,D], k,v [total_k,H,D],
     cu_seqlens_* int32 [nseq+1] on the device.  Returns (out like q, lse fp32 [H,total_q]).
-    Calls spa_flash_fwd_varlen."""
+    Calls spa_flash_fwd_varlen, or spa_flash_fwd_varlen_fp8kv when k, v are torch.float8_e4m3fn
+    (k_scale, v_scale: fp32 [nseq, H])."""
     lib = _lib.load()
-    q, k, v = _prep(q), _prep(k), _prep(v)
-    if not (q.dtype == k.dtype == v.dtype):
-        raise TypeError("q, k, v must share a dtype")
+    fp8 = k.dtype == FP8 or v.dtype == FP8
+    if fp8:
+        q = _prep(q)
+        k, v = [t if t.is_contiguous() else t.contiguous() for t in (k, v)]
+        if not k.is_cuda or not v.is_cuda:
+            raise ValueError("sp_aurora_amd kernels need tensors on a HIP device (got a CPU tensor)")
+    else:
+        q, k, v = _prep(q), _prep(k), _prep(v)
+        if not (q.dtype == k.dtype == v.dtype):
+            raise TypeError("q, k, v must share a dtype")
     (Tq, H, D), qs = _thd(q, "q")
     (Tk, Hk, Dk), ks = _thd(k, "k")
     shp_v, vs = _thd(v, "v")
@@ -317,12 +365,16 @@ def flash_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
     if lse is None:
         lse = torch.empty((H, Tq), dtype=torch.float32, device=q.device)
     _, os_ = _thd(out, "out")
-    with torch.cuda.device(q.device):
-        _lib.check(lib.spa_flash_fwd_varlen(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(),
-            cu_q.numel() - 1, H, Tq, Tk, int(max_seqlen_q), int(max_seqlen_k), D,
+    tail = (cu_q.data_ptr(), cu_k.data_ptr(), cu_q.numel() - 1, H, Tq, Tk, int(max_seqlen_q), int(max_seqlen_k), D,
             _lib.strides2(qs), _lib.strides2(ks), _lib.strides2(vs), _lib.strides2(os_),
-            float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(q), _stream()))
+            float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(q), _stream())
+    with torch.cuda.device(q.device):
+        if fp8:
+            ksc, vsc = _fp8_scales(k, v, k_scale, v_scale, cu_q.numel() - 1, H)
+            _lib.check(lib.spa_flash_fwd_varlen_fp8kv(q.data_ptr(), k.data_ptr(), v.data_ptr(), ksc.data_ptr(), vsc.data_ptr(),
+                                                      out.data_ptr(), lse.data_ptr(), *tail))
+        else:
+            _lib.check(lib.spa_flash_fwd_varlen(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), *tail))
     return out, lse
 
 

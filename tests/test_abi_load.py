@@ -67,6 +67,18 @@ def test_bad_arguments_return_codes_without_touching_a_device():
     f = ctypes.c_void_p(4096)
     args = [f] * 9 + [1, 1, 8, 8, 64] + [st] * 7
     assert lib.spa_flash_bwd(*args, 1.0, 0, 9, None) == -1
+    # e4m3 K/V: scales required, fp32 queries and head dim 32 unsupported, 8-byte alignment of k8 / v8
+    a8 = [p, p, p, p, p, p, p, 1, 1, 8, 8, 64, st, st, st, st, 1.0, 0, 1, None]
+    bad = list(a8); bad[3] = None
+    assert lib.spa_flash_fwd_fp8kv(*bad) == -1 and b"scale" in lib.spa_last_error()
+    bad = list(a8); bad[18] = 0
+    assert lib.spa_flash_fwd_fp8kv(*bad) == -2
+    bad = list(a8); bad[11] = 32
+    assert lib.spa_flash_fwd_fp8kv(*bad) == -2
+    bad = list(a8); bad[1] = ctypes.c_void_p(4100)
+    assert lib.spa_flash_fwd_fp8kv(*bad) == -3
+    bad = list(a8); bad[13] = _s3(60, 60, 60)
+    assert lib.spa_flash_fwd_fp8kv(*bad) == -3
     # variable-length batches: (head, row) strides; the cu_seqlens arrays are never read on the host
     s2 = _lib.strides2((64, 64))
     ok = [p] * 7 + [2, 1, 16, 16, 8, 8, 64, s2, s2, s2, s2, 1.0, 1, 1, None]

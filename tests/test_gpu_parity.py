@@ -381,8 +381,27 @@ def test_backward_with_strongly_negative_scores_and_ragged_keys(Sq, Sk, causal, 
     dk = torch.zeros((B, Sk, H, D), dtype=torch.float32, device=DEV)
     dv = torch.zeros((B, Sk, H, D), dtype=torch.float32, device=DEV)
     ops.flash_bwd(qd, kd, vd, dd, lse, delta, dq, dk, dv, None, causal, layout="bshd")
-    for got, w, name in zip((dq, dk, dv), want, "qkv"):
-        check_grad(got, w, dtype, "d" + name)
+    # K (and Q) carry an offset 80 times their spread, so the element-wise errors of P and dS do not
+    # cancel the way the exact terms do in sum_j dS_ij K_j; the bound is that error itself:
+    # |err dq| <= eps * scale * |dS| |K|, likewise dk with |Q| and dv = P^T dO with |dO|, where eps is
+    # the relative error of one element of P / dS: 2^-8 for 16-bit types (they enter the gradient
+    # MFMAs rounded to the input type), 3e-4 for fp32 (scores near -128 summed from 64 fp32
+    # products of size 16 carry ~1e-4 of absolute error, which exp() turns into relative error).
+    eps = 3e-4 if dtype == torch.float32 else 2.0 ** -8
+    qt, kt, vt, dot = (tr(t).double() for t in (q, k, v, dout))
+    sc = D ** -0.5
+    sm = torch.matmul(qt, kt.transpose(-2, -1)) * sc
+    if causal:
+        sm = sm.masked_fill(O.causal_mask(Sq, Sk), float("-inf"))
+    pm = torch.exp(sm - want_lse.unsqueeze(-1))
+    dsm = (pm * (torch.matmul(dot, vt.transpose(-2, -1)) - want_delta.unsqueeze(-1))).abs()
+    bounds = [tr(torch.matmul(dsm, kt.abs()) * sc), tr(torch.matmul(dsm.transpose(-2, -1), qt.abs()) * sc),
+              tr(torch.matmul(pm.transpose(-2, -1), dot.abs()))]
+    for got, w, bound, name in zip((dq, dk, dv), want, bounds, "qkv"):
+        got = got.cpu().double()
+        assert torch.isfinite(got).all(), f"d{name}: non-finite values"
+        bad = (got - w).abs() > eps * bound + 1e-6
+        assert not bad.any(), f"d{name}: {int(bad.sum())} beyond the rounding bound, max abs err {(got - w).abs().max():.3e}"
 
 
 @pytest.mark.parametrize("causal", [False, True])
