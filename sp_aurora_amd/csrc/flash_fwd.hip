@@ -38,7 +38,12 @@
 namespace {
 
 constexpr int FWD_BM = 128;  // query rows per workgroup
-constexpr int FWD_BN = 64;   // keys per LDS sub-tile
+// Keys per LDS sub-tile (one VALU phase + one MFMA phase of a wave).  The kernel is written for 64 or
+// 128.  128-key sub-tiles for D = 64 (whose phases hold half the MFMA work against the same softmax
+// work) were measured 5-8 % slower than 64-key ones on every shape tried, long rows included:
+// fewer barriers do not pay for the coarser ping-pong and the 247-register VALU phase.
+template <int D>
+constexpr int fwd_bn() { return 64; }
 constexpr int FWD_THREADS = 256;  // threads of one wave group (4 waves x 32 query rows)
 constexpr int FWD_LOOK = 8;       // MFMA operands are fetched from LDS this many MFMAs ahead
 
@@ -48,8 +53,10 @@ constexpr int FWD_LOOK = 8;       // MFMA operands are fetched from LDS this man
 // buffers together: half the global -> LDS traffic per FLOP and half as many workgroups.
 template <int D, int NG, bool SHARE>
 struct Fwd16Cfg {
+  static constexpr int BN = fwd_bn<D>();       // keys per sub-tile
+  static constexpr int NT = BN / 32;           // 32-key score tiles per sub-tile
   static constexpr int ROWB = D * 2;           // bytes per K / V row in LDS: no padding, the tiles are swizzled
-  static constexpr int TILEB = FWD_BN * ROWB;  // one K or V sub-tile
+  static constexpr int TILEB = BN * ROWB;      // one K or V sub-tile
   static constexpr int GROUP = 4 * TILEB;      // one set of K[2] and V[2] buffers
   static constexpr int BMW = SHARE ? NG * FWD_BM : FWD_BM;  // query rows per workgroup
   static constexpr int EPI = (NG * FWD_BM * (D + 4) + NG * FWD_BM * 2 + BMW) * 4;  // epilogue staging
@@ -157,7 +164,8 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // [t_begin, t_end) of that schedule; a plain block call is P = 1, one step.
   // A group's work is a sequence of 64-key sub-tiles: first those of the masked (diagonal)
   // chunk up to the last key any row of the workgroup sees, then every full chunk.
-  constexpr int TILE = SHARE ? FWD_BN : FWD_BN * NG;  // keys between two sub-tiles of one group
+  constexpr int BN = C::BN, NT = C::NT;
+  constexpr int TILE = SHARE ? BN : BN * NG;  // keys between two sub-tiles of one group
   constexpr int KSTEP = SHARE ? 1 : NG;
   const int nsteps = p.causal ? (rank + 1 < p.P ? rank + 1 : p.P) : p.P;
   const int t_end = p.t_count < 0 || p.t_begin + p.t_count > nsteps ? nsteps : p.t_begin + p.t_count;
@@ -194,7 +202,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     ch = ch < 0 ? ch + p.P : ch;
     ch = ch < 0 ? 0 : ch;  // only past the end of the schedule, where nothing is used
     c.sb.masked = c.i < n_diag;
-    c.sb.krel = (c.j * KSTEP + (SHARE ? 0 : grp)) * FWD_BN;
+    c.sb.krel = (c.j * KSTEP + (SHARE ? 0 : grp)) * BN;
     c.sb.krow = ch * p.Sk + c.sb.krel;
     c.sb.kend = ch * p.Sk + p.Sk;
   };
@@ -294,7 +302,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     }
   }
 
-  f32x16 s[2];
+  f32x16 s[NT];
   f32x16 o[D / 32];
 #pragma unroll
   for (int i = 0; i < D / 32; ++i)
@@ -317,12 +325,12 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // MFMA phase of step i: O += V(i)^T P(i) (if PV) followed by S(i+1) = K(i+1) Q^T (if NS).
   // The LDS operand of MFMA number j is fetched LOOK MFMAs ahead of its use, so the whole
   // phase runs off a rolling window of LOOK fragments instead of stalling on every read.
-  auto mfma_phase = [&](auto do_pv, auto do_s, const unsigned (&va)[D / 32], const unsigned (&ka)[D / 16], frag (&pfr)[2][2], auto&& side) {
+  auto mfma_phase = [&](auto do_pv, auto do_s, const unsigned (&va)[D / 32], const unsigned (&ka)[D / 16], frag (&pfr)[NT][2], auto&& side) {
     constexpr bool PV = decltype(do_pv)::value, NS = decltype(do_s)::value;
-    constexpr int NPV = PV ? (D / 32) * 4 : 0;
-    constexpr int NSS = NS ? (D / 16) * 2 : 0;
+    constexpr int NPV = PV ? (D / 32) * (BN / 16) : 0;
+    constexpr int NSS = NS ? (D / 16) * NT : 0;
     constexpr int TOTAL = NPV + NSS;
-    constexpr int LOOK = FWD_LOOK;
+    constexpr int LOOK = KV8 && D == 64 ? FWD_LOOK - 2 : FWD_LOOK;  // (the staged e4m3 bytes take the registers of two fragments)
     auto fetch = [&](int j) -> frag {
       if (j < NPV) {  // j = (t*2+u)*(D/32) + db : consecutive MFMAs hit different accumulators
         const int db = j % (D / 32), tu = j / (D / 32);
@@ -337,8 +345,8 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         x[3] = r1[1];
         return as_frag<frag>(x);
       }
-      const int jj = j - NPV;  // jj = ks*2 + t
-      const int t = jj & 1, ks = jj >> 1;
+      const int jj = j - NPV;  // jj = ks*NT + t
+      const int t = jj % NT, ks = jj / NT;
       return as_frag<frag>(*(const __attribute__((address_space(3))) u32x4*)((const lds_u8*)(uintptr_t)ka[ks] + t * 32 * C::ROWB));
     };
     frag win[LOOK];
@@ -356,7 +364,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         o[db] = M::run(a, pfr[tu >> 1][tu & 1], o[db]);
       } else {
         const int jj = j - NPV;
-        const int t = jj & 1, ks = jj >> 1;
+        const int t = jj % NT, ks = jj / NT;
         if (ks == 0) {
           f32x16 z;
 #pragma unroll
@@ -371,14 +379,14 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   };
 
   // VALU phase of step i: softmax of S(i) -> P(i) as MFMA operands, O rescaled if needed.
-  auto softmax_phase = [&](const Sub& sb, frag (&pfr)[2][2]) {
+  auto softmax_phase = [&](const Sub& sb, frag (&pfr)[NT][2]) {
     const int key0 = sb.krel;
     const bool causal_here = sb.masked;
-    const bool need_mask = (causal_here && key0 + FWD_BN - 1 > qw0) || (key0 + FWD_BN > p.Sk);
+    const bool need_mask = (causal_here && key0 + BN - 1 > qw0) || (key0 + BN > p.Sk);
     if (need_mask) {
       const int lim = causal_here ? (qrow < p.Sk - 1 ? qrow : p.Sk - 1) : p.Sk - 1;  // last visible key
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int key = key0 + t * 32 + 8 * (v >> 2) + 4 * hh + (v & 3);
@@ -386,27 +394,40 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         }
     }
 
-    // row max of the lane's 32 scores: 3-input maxima in four independent chains.  (Through the
-    // instruction itself: fmaxf() makes the compiler quiet possible signalling NaNs first, one
-    // extra instruction per MFMA result; the scores are finite or -inf here.)
+    // row max of the lane's 32 NT scores: 3-input maxima, two independent chains per 32-key tile.
+    // (Through the instruction itself: fmaxf() makes the compiler quiet possible signalling NaNs
+    // first, one extra instruction per MFMA result; the scores are finite or -inf here.)
     auto max3 = [](float a, float b, float c3) {
       float r;
       asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c3));
       return r;
     };
-    float mxa = max3(s[0][0], s[0][1], s[0][2]), mxb = max3(s[0][8], s[0][9], s[0][10]);
-    float mxc = max3(s[1][0], s[1][1], s[1][2]), mxd = max3(s[1][8], s[1][9], s[1][10]);
-    mxa = max3(mxa, s[0][3], s[0][4]);
-    mxb = max3(mxb, s[0][11], s[0][12]);
-    mxc = max3(mxc, s[1][3], s[1][4]);
-    mxd = max3(mxd, s[1][11], s[1][12]);
-    mxa = max3(mxa, s[0][5], s[0][6]);
-    mxb = max3(mxb, s[0][13], s[0][14]);
-    mxc = max3(mxc, s[1][5], s[1][6]);
-    mxd = max3(mxd, s[1][13], s[1][14]);
-    mxa = max3(mxa, s[0][7], mxb);
-    mxc = max3(mxc, s[1][7], mxd);
-    float mx = max3(mxa, mxc, fmaxf(s[0][15], s[1][15]));
+    float mxa[NT], mxb[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      mxa[t] = max3(s[t][0], s[t][1], s[t][2]);
+      mxb[t] = max3(s[t][8], s[t][9], s[t][10]);
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      mxa[t] = max3(mxa[t], s[t][3], s[t][4]);
+      mxb[t] = max3(mxb[t], s[t][11], s[t][12]);
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      mxa[t] = max3(mxa[t], s[t][5], s[t][6]);
+      mxb[t] = max3(mxb[t], s[t][13], s[t][14]);
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) mxa[t] = max3(mxa[t], s[t][7], mxb[t]);
+    float mx;
+    if constexpr (NT == 2) {
+      mx = max3(mxa[0], mxa[1], fmaxf(s[0][15], s[1][15]));
+    } else {
+      static_assert(NT == 4, "sub-tiles of 64 or 128 keys");
+      const float u = max3(mxa[0], mxa[1], s[0][15]), w2 = max3(mxa[2], mxa[3], s[1][15]);
+      mx = max3(u, w2, fmaxf(s[2][15], s[3][15]));
+    }
     mx = halves_max(mx);
     // Lazy rescale: the reference max only moves when some row's max grew by more than
     // 2^8 in the exp2 domain; until then P <= 256, harmless in fp32 sums and bf16 operands.
@@ -425,7 +446,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
 
     float ps[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const float e = fast_exp2(__builtin_fmaf(s[t][v], c, -mc));
@@ -436,7 +457,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     asm volatile("" : "+v"(l_run));  // keep the row sum in this phase as well (see below)
 
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int u = 0; u < 2; ++u)
         pfr[t][u] = M::pack(s[t][8 * u + 0], s[t][8 * u + 1], s[t][8 * u + 2], s[t][8 * u + 3],
@@ -444,7 +465,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     // P must exist in registers when the phase ends: without this the compiler sinks the
     // exponentials past the barrier into the MFMA phase they are meant to overlap with.
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         u32x4 x = __builtin_bit_cast(u32x4, pfr[t][u]);
@@ -464,7 +485,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     int ch = rank - cs.t;
     ch = ch < 0 ? ch + p.P : ch;
     cs.sb.masked = n_diag > 0;
-    cs.sb.krel = (SHARE ? 0 : grp) * FWD_BN;
+    cs.sb.krel = (SHARE ? 0 : grp) * BN;
     cs.sb.krow = ch * p.Sk + cs.sb.krel;
     cs.sb.kend = ch * p.Sk + p.Sk;
   }
@@ -491,7 +512,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * C::NDMA) & 15) | (((2 * C::NDMA) >> 4) << 14));  // vmcnt(2 NDMA)
   __syncthreads();
   {
-    frag none[2][2];
+    frag none[NT][2];
     unsigned va[D / 32], ka[D / 16];
     operand_addresses(-1, va, ka);
     mfma_phase(std::false_type{}, std::true_type{}, va, ka, none, [](int) {});  // S(0)
@@ -515,7 +536,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // the MFMA phase is a per-lane constant plus an immediate offset (no address arithmetic per step).
   auto body = [&](auto parity, int i) __attribute__((always_inline)) {
     constexpr int PAR = decltype(parity)::value;  // == i & 1
-    frag pf[2][2];
+    frag pf[NT][2];
     const bool kon = ck.i < n, von = cv.i < n;
     constexpr unsigned kb = (unsigned)(PAR * C::TILEB), vb = (unsigned)(2 * C::TILEB + (PAR ^ 1) * C::TILEB);  // k_lds(i), v_lds(i + 1)
     if (early) {
@@ -536,7 +557,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     if (!SHARE || !early) __syncthreads();
     __builtin_amdgcn_s_setprio(3);
     mfma_phase(std::true_type{}, std::true_type{}, va, ka, pf, [&](int j) {
-      constexpr int TOTAL = (D / 32) * 4 + (D / 16) * 2;
+      constexpr int TOTAL = (D / 32) * (BN / 16) + (D / 16) * NT;
 #pragma unroll
       for (int q = 0; q < NLOADS; ++q)
         if ((q * TOTAL + TOTAL / 2) / NLOADS == j && !early) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb);
@@ -557,7 +578,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     if (i + 1 < n) body(std::integral_constant<int, 0>{}, i);
   }
   {  // last sub-tile: nothing to prepare behind it
-    frag pf[2][2];
+    frag pf[NT][2];
     softmax_phase(cs.sb, pf);
     unsigned va[D / 32], ka[D / 16];
     operand_addresses(n - 1, va, ka);
@@ -966,7 +987,7 @@ template <typename T, int D>
 hipError_t launch16(FwdParams p, hipStream_t stream) {
   const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
   const int force_share = spa_knob(SPA_KNOB_FWD_SHARE);
-  const bool two = force ? force == 2 : p.Sk > FWD_BN;
+  const bool two = force ? force == 2 : p.Sk > fwd_bn<D>();
   if (two && D >= 64) {
     const int nqt2 = (p.Sq + 2 * FWD_BM - 1) / (2 * FWD_BM);
     const int64_t wgs = (int64_t)p.B * p.H * nqt2 * p.nranks;
@@ -984,7 +1005,7 @@ hipError_t launch16(FwdParams p, hipStream_t stream) {
 template <typename T, int D>
 hipError_t launch16_kv8(FwdParams p, hipStream_t stream) {
   const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
-  const bool two = force ? force == 2 : p.Sk > FWD_BN;
+  const bool two = force ? force == 2 : p.Sk > fwd_bn<D>();
   if (two) return launch<flash_fwd16_kernel<T, D, 2, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
   return launch<flash_fwd16_kernel<T, D, 1, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
 }

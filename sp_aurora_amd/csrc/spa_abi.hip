@@ -380,6 +380,7 @@ static int relayout(const void* src, void* dst, int P, int B, int s, int H, int 
     return fail(SPA_EINVAL, "%s: elem_bytes must be 1, 2, 4 or 8", what);
   if (H % P != 0) return fail(SPA_EINVAL, "%s: heads (%d) not divisible by ranks (%d)", what, H, P);
   if (src == dst) return fail(SPA_EINVAL, "%s: in-place re-layout is not supported", what);
+  if ((int64_t)P * pack > 65535 || (int64_t)P * B > 65535) return fail(SPA_EINVAL, "%s: grid too large (P * B and P * pack must stay below 65536)", what);
   return launch_result(spa_launch_relayout(src, dst, P, B, s, H, D, pack, elem_bytes, s2h, (hipStream_t)stream), what);
 }
 
