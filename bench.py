@@ -381,6 +381,27 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
                             "inverse re-layout of out (3 re-layouts in, attention, 1 out; output allocation included)", "flops_per_step": flops},
                tf, "TFLOP/s", roof("mfma", "relayout_kernel x4 + flash_fwd16_kernel<bf16,128,2>", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
         del q, k, v, y, xs
+    if "fp8kv" in which:
+        # the config-3 sequence as one causal block call, K / V in e4m3 with per-head scales, against
+        # the same call with bf16 K / V (same kernel family, direct-to-LDS tiles)
+        Bn, Sn, Hn, Dn = 1, 8192, 32, 128
+        q, k, v = rand_tensors(torch, (Bn, Sn, Hn, Dn), SEED, 3, INPUT_SCALE, torch.bfloat16, dev)
+        k8, ksc = ops.quantize_fp8_per_head(k)
+        v8, vsc = ops.quantize_fp8_per_head(v)
+        out = torch.empty_like(q)
+        lse = torch.empty((Bn, Hn, Sn), dtype=torch.float32, device=dev)
+        flops = 4.0 * Bn * Hn * Sn * Sn * Dn / 2
+        f8 = lambda: ops.flash_fwd(q, k8, v8, None, True, out=out, lse=lse, k_scale=ksc, v_scale=vsc)
+        f16 = lambda: ops.flash_fwd(q, k, v, None, True, out=out, lse=lse)
+        m16 = measure(torch, f16, 20, 5, **light)
+        m = measure(torch, f8, 20, 5, **light)
+        tf = flops / (m["ms_per_step"] * 1e-3) / 1e12
+        finish("block_forward_fp8_kv", m,
+               {"workload": "causal block forward over the config-3 sequence (bf16 q [1,8192,32,128], K / V e4m3 + fp32 scale per (batch, head)), one call",
+                "flops_per_step": flops, "same_call_with_bf16_kv": {"ms_per_step": round(m16["ms_per_step"], 4),
+                                                                     "tflops": round(flops / (m16["ms_per_step"] * 1e-3) / 1e12, 2)}},
+               tf, "TFLOP/s", roof("mfma", "flash_fwd16_kernel<bf16,128,2,e4m3 K/V>", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
+        del q, k, v, k8, v8
     if "merge" in which:
         Bn, sn, Hn, Dn = 1, 1024, 32, 128
         g = torch.Generator().manual_seed(3)
@@ -438,6 +459,9 @@ def attach_cpu(rows, cpu):
         rows["config4_relayout_h2s"]["cpu_baseline"] = b
         rows["config4_ulysses_forward"]["cpu_baseline"] = cpu.ring_forward(
             1, 4, 2048, 128, 8, 28, 3, "config 4 attention of one head group [1,4,16384,128] as 2048-row blocks (x 8 groups: same ratio); re-layouts not included")
+    if "block_forward_fp8_kv" in rows:
+        rows["block_forward_fp8_kv"]["cpu_baseline"] = cpu.ring_forward(
+            1, 32, 1024, 128, 8, 28, SEED, "the same attention with dequantised K / V as 1024-row blocks (the reference has no 8-bit path)")
     if "merge_update_out_and_lse" in rows:
         rows["merge_update_out_and_lse"]["cpu_baseline"] = cpu.merge()
     if "config5_ring_forward" in rows:
@@ -494,7 +518,7 @@ def pmc_summary(fetch_dir, write_dir):
 
 
 # ------------------------------------------------------------------------------------ main
-ROW_SETS = {"relayout": {"config4"}, "ulysses": {"config4"}, "merge": {"merge"}, "backward": {"config5"},
+ROW_SETS = {"fp8kv": {"fp8kv"}, "relayout": {"config4"}, "ulysses": {"config4"}, "merge": {"merge"}, "backward": {"config5"},
             "config1": {"config1"}, "config2": {"config2"}}
 
 
@@ -576,7 +600,7 @@ def main():
     rows = {}
     if not args.no_rows and not args.only_all:
         del steps
-        rows = gpu_rows(torch, spa, ops, {"config1", "config2", "config4", "merge", "config5"}, args.steps, args.warmup)
+        rows = gpu_rows(torch, spa, ops, {"config1", "config2", "config4", "fp8kv", "merge", "config5"}, args.steps, args.warmup)
 
     launches = {"all": 1, "rank": P, "step": n_pairs}[head]
     line = {

@@ -442,14 +442,16 @@ struct DkvCfg {
   static constexpr int NL = 2 * C::NDMA + 1;          // loads per thread and stage
 };
 
-template <typename T, int D>
+// ASM = false: the D = 128 kernel with every MFMA left to the compiler (its uniform accumulator
+// form, its own hazard handling): slower, kept as the test twin of the hand-issued form.
+template <typename T, int D, bool ASM = true>
 __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const BwdParams pk) {
   BwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
   typedef BwdCfg<D> C;
   typedef DkvCfg<D> G;
   typedef Mma16<T> M;
   typedef MmaAsm<T> MA;
-  constexpr bool MIXED = D == 128;  // see the dq kernel; here 16 gradient MFMAs separate a tile's MFMAs from its VALU reads
+  constexpr bool MIXED = D == 128 && ASM;  // see the dq kernel; here 16 gradient MFMAs separate a tile's MFMAs from its VALU reads
   typedef typename M::frag frag;
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -1028,6 +1030,8 @@ hipError_t launch_both(const BwdParams& p, hipStream_t stream) {
   }
   if (!wide) e = launch<flash_bwd_dq_kernel<T, D, 4>>(DqCfg<D, 4>::SMEM, (unsigned)((int64_t)p.B * p.H * p.nqt), p, stream);
   if (e != hipSuccess) return e;
+  if constexpr (D == 128)
+    if (spa_knob(SPA_KNOB_BWD_DKDV_FORM) == 1) return launch<flash_bwd_dkdv_kernel<T, D, false>>(DkvCfg<D>::SMEM, kblocks, p, stream);
   return launch<flash_bwd_dkdv_kernel<T, D>>(DkvCfg<D>::SMEM, kblocks, p, stream);
 }
 

@@ -444,6 +444,31 @@ def test_dq_kernel_workgroup_sizes_agree(B, S, H, D, causal, dtype):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,S,H,D,causal", [(1, 300, 2, 128, True), (2, 515, 2, 128, False), (1, 1000, 2, 128, True),
+                                            (1, 77, 1, 128, True), (1, 2048, 1, 128, True)])
+def test_dkdv_kernel_hand_issued_and_compiler_scheduled_forms_agree(B, S, H, D, causal, dtype):
+    """The D = 128 dk/dv kernel issues its MFMAs from inline assembly with the MFMA -> VALU hazard
+    distances kept by the order of the loop; its twin leaves every MFMA (and every hazard) to the
+    compiler.  Same operations in the same order on the same values: the gradients must be
+    bit-identical, and right."""
+    q, k, v, dout = rand_qkv((B, S, H, D), 141, dtype, n=4)
+    want = O.attn_backward_autograd(q, k, v, dout, None, causal)
+    got = {}
+    try:
+        for form in (0, 1):
+            _lib.tune("bwd_dkdv_form", form)
+            xs = [t.to(DEV).requires_grad_(True) for t in (q, k, v)]
+            spa.ring_flash_attn_func(*xs, causal=causal).backward(dout.to(DEV))
+            got[form] = [x.grad for x in xs]
+            for g, w, name in zip(got[form], want, "qkv"):
+                check_grad(g, w, dtype, f"d{name}, form {form}")
+    finally:
+        _lib.tune("bwd_dkdv_form", 0)
+    for a, b in zip(got[0], got[1]):
+        assert torch.equal(a, b)
+
+
 def test_backward_packed_and_operator_entry():
     B, S, H, D = 1, 256, 2, 128
     qkv = rand((B, S, 3, H, D), 101, torch.bfloat16)
