@@ -3,9 +3,10 @@
 //              stands in for update_out_and_lse (sp_aurora/utils.py:47-147)
 //   finalize : out = cast(out_acc)   (sp_aurora/intel_ring_flash_attn.py:141-143)
 //   delta    : delta = rowsum(dout * out), first pass of the block-wise backward
-// One thread owns 8 consecutive head dims of one (b, h, s) row; the D/8 threads
-// of a row sit in one wavefront, so every lane of the row has read lse_acc before
-// the row's first lane overwrites it.
+// One thread owns 8 consecutive head dims of two (b, h, s) rows (all loads of both rows are
+// issued before the first store); the D/8 threads of a row sit in one wavefront, so every lane of
+// the row has read lse_acc before the row's first lane overwrites it.  32-bit row arithmetic,
+// the batch index comes from the grid.
 #include "spa_common.h"
 
 namespace {
@@ -14,16 +15,18 @@ struct RowIdx {
   int b, h, s;
 };
 
-// rows are enumerated with the head index fastest after the sequence index of
-// the [B,S,H,D] accumulator: row = (b*Sq + s)*H + h.
-static __device__ __forceinline__ RowIdx decode_row(int64_t row, int H, int Sq) {
+// Rows of one batch entry are enumerated with the head index fastest after the sequence index of
+// the [B,S,H,D] accumulator: row = s*H + h (32-bit: a batch entry holds fewer than 2^31 rows, the
+// launchers check it); the batch index is the grid's y dimension.
+static __device__ __forceinline__ RowIdx decode_row(unsigned row, int H) {
   RowIdx r;
-  r.h = (int)(row % H);
-  const int64_t t = row / H;
-  r.s = (int)(t % Sq);
-  r.b = (int)(t / Sq);
+  r.s = (int)(row / (unsigned)H);
+  r.h = (int)(row - (unsigned)r.s * (unsigned)H);
+  r.b = (int)blockIdx.y;
   return r;
 }
+
+constexpr int ROWS_PER_THREAD = 1;  // rows a thread takes (two, `half` rows apart with all loads first, measured 10 % slower on the merge)
 
 template <typename T>
 struct Load8;  // 8 consecutive elements as floats
@@ -77,83 +80,137 @@ struct Load8<_Float16> {
   }
 };
 
+// A thread owns chunk `ch` (8 head dims) of ROWS_PER_THREAD rows, `half` rows apart; the D/8
+// lanes of a row share a wave, so every lane of the row has read lse_acc before lane 0 rewrites it.
 template <typename T, bool INIT>
 __global__ void __launch_bounds__(256) merge_kernel(float* __restrict__ out_acc, float* __restrict__ lse_acc,
                                                     const T* __restrict__ blk_out,
                                                     const float* __restrict__ blk_lse, int H, int Sq,
-                                                    int cpr /* D/8 */, int64_t nrows, Strides3 as,
-                                                    Strides3 bs, int64_t acc_lse_bh) {
-  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t row = gid / cpr;
-  const int ch = (int)(gid % cpr);
-  if (row >= nrows) return;
-  const RowIdx r = decode_row(row, H, Sq);
-  const int64_t li = ((int64_t)r.b * H + r.h) * Sq + r.s;          // block lse: contiguous [B,H,Sq]
-  const int64_t la_i = ((int64_t)r.b * H + r.h) * acc_lse_bh + r.s;  // running lse: row pitch acc_lse_bh
-  float* ap = out_acc + r.b * as.b + r.h * as.h + (int64_t)r.s * as.s + ch * 8;
-  const T* bp = blk_out + r.b * bs.b + r.h * bs.h + (int64_t)r.s * bs.s + ch * 8;
-  float xb[8];
-  Load8<T>::ld(bp, xb);
-  const float lb = blk_lse[li];
-  if (INIT) {
-    Load8<float>::st(ap, xb);
-    if (ch == 0) lse_acc[la_i] = lb;
-    return;
-  }
-  const float la = lse_acc[la_i];
-  float xa[8];
-  Load8<float>::ld(ap, xa);
-  // w = sigmoid(lb - la); lse' = max + log1p(exp(-|lb - la|))
-  const float d = lb - la;
-  float w, ln;
-  if (d == d) {  // also covers +-inf on one side
-    const float e = __expf(-fabsf(d));
-    const float inv = 1.f / (1.f + e);
-    w = d >= 0.f ? inv : e * inv;
-    ln = fmaxf(la, lb) + log1pf(e);
-  } else {  // both -inf: nothing accumulated on either side
-    w = 0.f;
-    ln = la;
+                                                    int cpr_shift /* log2(D/8) */, unsigned nrows, unsigned half,
+                                                    Strides3 as, Strides3 bs, int64_t acc_lse_bh) {
+  const unsigned gid = blockIdx.x * 256u + threadIdx.x;
+  const unsigned row0 = gid >> cpr_shift;
+  const int ch = (int)(gid & ((1u << cpr_shift) - 1u));
+  float xb[ROWS_PER_THREAD][8], xa[ROWS_PER_THREAD][8], lb[ROWS_PER_THREAD], la[ROWS_PER_THREAD];
+  float* ap[ROWS_PER_THREAD];
+  int64_t la_i[ROWS_PER_THREAD];
+  bool on[ROWS_PER_THREAD];
+#pragma unroll
+  for (int k = 0; k < ROWS_PER_THREAD; ++k) {
+    const unsigned row = row0 + k * half;
+    on[k] = row0 < half && row < nrows;
+    const RowIdx r = decode_row(on[k] ? row : 0u, H);
+    const int64_t li = ((int64_t)r.b * H + r.h) * Sq + r.s;     // block lse: contiguous [B,H,Sq]
+    la_i[k] = ((int64_t)r.b * H + r.h) * acc_lse_bh + r.s;        // running lse: row pitch acc_lse_bh
+    ap[k] = out_acc + r.b * as.b + r.h * as.h + (int64_t)r.s * as.s + ch * 8;
+    if (on[k]) {
+      Load8<T>::ld(blk_out + r.b * bs.b + r.h * bs.h + (int64_t)r.s * bs.s + ch * 8, xb[k]);
+      lb[k] = blk_lse[li];
+      if (!INIT) {
+        la[k] = lse_acc[la_i[k]];
+        Load8<float>::ld(ap[k], xa[k]);
+      }
+    }
   }
 #pragma unroll
-  for (int i = 0; i < 8; ++i) xa[i] = xa[i] - w * (xa[i] - xb[i]);
-  Load8<float>::st(ap, xa);
-  if (ch == 0) lse_acc[la_i] = ln;
+  for (int k = 0; k < ROWS_PER_THREAD; ++k) {
+    if (!on[k]) continue;
+    if (INIT) {
+      Load8<float>::st(ap[k], xb[k]);
+      if (ch == 0) lse_acc[la_i[k]] = lb[k];
+      continue;
+    }
+    // w = sigmoid(lb - la); lse' = max + log1p(exp(-|lb - la|))
+    const float d = lb[k] - la[k];
+    float w, ln;
+    if (d == d) {  // also covers +-inf on one side
+      const float e = __expf(-fabsf(d));
+      const float inv = 1.f / (1.f + e);
+      w = d >= 0.f ? inv : e * inv;
+      ln = fmaxf(la[k], lb[k]) + log1pf(e);
+    } else {  // both -inf: nothing accumulated on either side
+      w = 0.f;
+      ln = la[k];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xa[k][i] = xa[k][i] - w * (xa[k][i] - xb[k][i]);
+    Load8<float>::st(ap[k], xa[k]);
+    if (ch == 0) lse_acc[la_i[k]] = ln;
+  }
 }
 
 template <typename T>
 __global__ void __launch_bounds__(256) finalize_kernel(T* __restrict__ out, const float* __restrict__ out_acc,
-                                                       int H, int Sq, int cpr, int64_t nrows, Strides3 os,
-                                                       Strides3 as) {
-  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t row = gid / cpr;
-  const int ch = (int)(gid % cpr);
-  if (row >= nrows) return;
-  const RowIdx r = decode_row(row, H, Sq);
-  float x[8];
-  Load8<float>::ld(out_acc + r.b * as.b + r.h * as.h + (int64_t)r.s * as.s + ch * 8, x);
-  Load8<T>::st(out + r.b * os.b + r.h * os.h + (int64_t)r.s * os.s + ch * 8, x);
+                                                       int H, int cpr_shift, unsigned nrows, unsigned half,
+                                                       Strides3 os, Strides3 as) {
+  const unsigned gid = blockIdx.x * 256u + threadIdx.x;
+  const unsigned row0 = gid >> cpr_shift;
+  const int ch = (int)(gid & ((1u << cpr_shift) - 1u));
+  float x[ROWS_PER_THREAD][8];
+  T* op[ROWS_PER_THREAD];
+  bool on[ROWS_PER_THREAD];
+#pragma unroll
+  for (int k = 0; k < ROWS_PER_THREAD; ++k) {
+    const unsigned row = row0 + k * half;
+    on[k] = row0 < half && row < nrows;
+    const RowIdx r = decode_row(on[k] ? row : 0u, H);
+    op[k] = out + r.b * os.b + r.h * os.h + (int64_t)r.s * os.s + ch * 8;
+    if (on[k]) Load8<float>::ld(out_acc + r.b * as.b + r.h * as.h + (int64_t)r.s * as.s + ch * 8, x[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < ROWS_PER_THREAD; ++k)
+    if (on[k]) Load8<T>::st(op[k], x[k]);
 }
 
 // delta[b,h,s] = sum_d dout*out; the D/8 lanes of a row reduce with DPP-free shuffles.
 template <typename T>
 __global__ void __launch_bounds__(256) delta_kernel(const T* __restrict__ out, const T* __restrict__ dout,
-                                                    float* __restrict__ delta, int H, int Sq, int cpr,
-                                                    int64_t nrows, Strides3 os, Strides3 ds) {
-  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  int64_t row = gid / cpr;
-  const int ch = (int)(gid % cpr);
-  const bool valid = row < nrows;
-  if (!valid) row = nrows - 1;
-  const RowIdx r = decode_row(row, H, Sq);
-  float a[8], g[8];
-  Load8<T>::ld(out + r.b * os.b + r.h * os.h + (int64_t)r.s * os.s + ch * 8, a);
-  Load8<T>::ld(dout + r.b * ds.b + r.h * ds.h + (int64_t)r.s * ds.s + ch * 8, g);
-  float acc = 0.f;
+                                                    float* __restrict__ delta, int H, int Sq, int cpr_shift,
+                                                    unsigned nrows, unsigned half, Strides3 os, Strides3 ds) {
+  const unsigned gid = blockIdx.x * 256u + threadIdx.x;
+  const unsigned row0 = gid >> cpr_shift;
+  const int cpr = 1 << cpr_shift;
+  const int ch = (int)(gid & (unsigned)(cpr - 1));
+  float a[ROWS_PER_THREAD][8], g[ROWS_PER_THREAD][8];
+  int64_t di[ROWS_PER_THREAD];
+  bool on[ROWS_PER_THREAD];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) acc = __builtin_fmaf(a[i], g[i], acc);
-  for (int off = cpr >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-  if (valid && ch == 0) delta[((int64_t)r.b * H + r.h) * Sq + r.s] = acc;
+  for (int k = 0; k < ROWS_PER_THREAD; ++k) {
+    const unsigned row = row0 + k * half;
+    on[k] = row0 < half && row < nrows;
+    const RowIdx r = decode_row(on[k] ? row : 0u, H);  // (rows past the end reread row 0: every lane takes part in the shuffles)
+    di[k] = ((int64_t)r.b * H + r.h) * Sq + r.s;
+    Load8<T>::ld(out + r.b * os.b + r.h * os.h + (int64_t)r.s * os.s + ch * 8, a[k]);
+    Load8<T>::ld(dout + r.b * ds.b + r.h * ds.h + (int64_t)r.s * ds.s + ch * 8, g[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < ROWS_PER_THREAD; ++k) {
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc = __builtin_fmaf(a[k][i], g[k][i], acc);
+    for (int off = cpr >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (on[k] && ch == 0) delta[di[k]] = acc;
+  }
+}
+
+// Grid of the three kernels: x covers half the rows of one batch entry (a thread takes a row of
+// each half), y the batch.
+struct RowGrid {
+  dim3 grid;
+  unsigned nrows, half;
+  int cpr_shift;
+  bool ok;
+};
+RowGrid row_grid(int B, int H, int Sq, int D) {
+  RowGrid g;
+  const int64_t nrows = (int64_t)H * Sq;
+  g.cpr_shift = __builtin_ctz((unsigned)(D / 8));
+  g.ok = nrows < 0x7fffffffLL / (D / 8) && B <= 65535;
+  g.nrows = (unsigned)nrows;
+  g.half = (unsigned)((nrows + ROWS_PER_THREAD - 1) / ROWS_PER_THREAD);
+  const int64_t threads = (int64_t)g.half * (D / 8);
+  g.grid = dim3((unsigned)((threads + 255) / 256), (unsigned)B);
+  return g;
 }
 
 }  // namespace
@@ -161,13 +218,11 @@ __global__ void __launch_bounds__(256) delta_kernel(const T* __restrict__ out, c
 hipError_t spa_launch_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* blk_lse, int B,
                             int H, int Sq, int D, Strides3 as, Strides3 bs, int dtype, int init,
                             int64_t acc_lse_bh, hipStream_t stream) {
-  const int cpr = D / 8;
-  const int64_t nrows = (int64_t)B * H * Sq;
-  const int64_t nthreads = nrows * cpr;
-  const dim3 grid((unsigned)((nthreads + 255) / 256));
+  const RowGrid g = row_grid(B, H, Sq, D);
+  if (!g.ok) return hipErrorInvalidValue;
 #define SPA_MERGE(T, I)                                                                              \
-  hipLaunchKernelGGL((merge_kernel<T, I>), grid, dim3(256), 0, stream, out_acc, lse_acc, (const T*)blk_out, \
-                     blk_lse, H, Sq, cpr, nrows, as, bs, acc_lse_bh)
+  hipLaunchKernelGGL((merge_kernel<T, I>), g.grid, dim3(256), 0, stream, out_acc, lse_acc, (const T*)blk_out, \
+                     blk_lse, H, Sq, g.cpr_shift, g.nrows, g.half, as, bs, acc_lse_bh)
   if (dtype == 0) { if (init) SPA_MERGE(float, true); else SPA_MERGE(float, false); }
   else if (dtype == 1) { if (init) SPA_MERGE(__bf16, true); else SPA_MERGE(__bf16, false); }
   else if (dtype == 2) { if (init) SPA_MERGE(_Float16, true); else SPA_MERGE(_Float16, false); }
@@ -178,15 +233,14 @@ hipError_t spa_launch_merge(float* out_acc, float* lse_acc, const void* blk_out,
 
 hipError_t spa_launch_finalize(void* out, const float* out_acc, int B, int H, int Sq, int D, Strides3 os,
                                Strides3 as, int dtype, hipStream_t stream) {
-  const int cpr = D / 8;
-  const int64_t nrows = (int64_t)B * H * Sq;
-  const dim3 grid((unsigned)((nrows * cpr + 255) / 256));
+  const RowGrid g = row_grid(B, H, Sq, D);
+  if (!g.ok) return hipErrorInvalidValue;
   if (dtype == 0)
-    hipLaunchKernelGGL((finalize_kernel<float>), grid, dim3(256), 0, stream, (float*)out, out_acc, H, Sq, cpr, nrows, os, as);
+    hipLaunchKernelGGL((finalize_kernel<float>), g.grid, dim3(256), 0, stream, (float*)out, out_acc, H, g.cpr_shift, g.nrows, g.half, os, as);
   else if (dtype == 1)
-    hipLaunchKernelGGL((finalize_kernel<__bf16>), grid, dim3(256), 0, stream, (__bf16*)out, out_acc, H, Sq, cpr, nrows, os, as);
+    hipLaunchKernelGGL((finalize_kernel<__bf16>), g.grid, dim3(256), 0, stream, (__bf16*)out, out_acc, H, g.cpr_shift, g.nrows, g.half, os, as);
   else if (dtype == 2)
-    hipLaunchKernelGGL((finalize_kernel<_Float16>), grid, dim3(256), 0, stream, (_Float16*)out, out_acc, H, Sq, cpr, nrows, os, as);
+    hipLaunchKernelGGL((finalize_kernel<_Float16>), g.grid, dim3(256), 0, stream, (_Float16*)out, out_acc, H, g.cpr_shift, g.nrows, g.half, os, as);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();
@@ -194,15 +248,14 @@ hipError_t spa_launch_finalize(void* out, const float* out_acc, int B, int H, in
 
 hipError_t spa_launch_delta(const void* out, const void* dout, float* delta, int B, int H, int Sq, int D,
                             Strides3 os, Strides3 ds, int dtype, hipStream_t stream) {
-  const int cpr = D / 8;
-  const int64_t nrows = (int64_t)B * H * Sq;
-  const dim3 grid((unsigned)((nrows * cpr + 255) / 256));
+  const RowGrid g = row_grid(B, H, Sq, D);
+  if (!g.ok) return hipErrorInvalidValue;
   if (dtype == 0)
-    hipLaunchKernelGGL((delta_kernel<float>), grid, dim3(256), 0, stream, (const float*)out, (const float*)dout, delta, H, Sq, cpr, nrows, os, ds);
+    hipLaunchKernelGGL((delta_kernel<float>), g.grid, dim3(256), 0, stream, (const float*)out, (const float*)dout, delta, H, Sq, g.cpr_shift, g.nrows, g.half, os, ds);
   else if (dtype == 1)
-    hipLaunchKernelGGL((delta_kernel<__bf16>), grid, dim3(256), 0, stream, (const __bf16*)out, (const __bf16*)dout, delta, H, Sq, cpr, nrows, os, ds);
+    hipLaunchKernelGGL((delta_kernel<__bf16>), g.grid, dim3(256), 0, stream, (const __bf16*)out, (const __bf16*)dout, delta, H, Sq, g.cpr_shift, g.nrows, g.half, os, ds);
   else if (dtype == 2)
-    hipLaunchKernelGGL((delta_kernel<_Float16>), grid, dim3(256), 0, stream, (const _Float16*)out, (const _Float16*)dout, delta, H, Sq, cpr, nrows, os, ds);
+    hipLaunchKernelGGL((delta_kernel<_Float16>), g.grid, dim3(256), 0, stream, (const _Float16*)out, (const _Float16*)dout, delta, H, Sq, g.cpr_shift, g.nrows, g.half, os, ds);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();

@@ -180,7 +180,7 @@ int spa_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* 
   if (!pow2_8_512(D)) return fail(SPA_EUNSUPPORTED, "spa_merge: head dim %d must be a power of two in [8,512]", D);
   if (!aligned16(out_acc, acc_strides, 4) || !aligned16(blk_out, blk_strides, elem_size(blk_dtype)))
     return fail(SPA_EALIGN, "spa_merge: pointers and row strides must be 16-byte aligned");
-  if ((int64_t)B * H * Sq * (D / 8) / 256 > 0x7ffffff0LL) return fail(SPA_EINVAL, "spa_merge: grid too large");
+  if (B > 65535 || (int64_t)H * Sq * (D / 8) >= 0x7fffffffLL) return fail(SPA_EINVAL, "spa_merge: grid too large");
   return launch_result(spa_launch_merge(out_acc, lse_acc, blk_out, blk_lse, B, H, Sq, D, S3(acc_strides),
                                         S3(blk_strides), blk_dtype, init, Sq, (hipStream_t)stream),
                        "spa_merge");
@@ -365,7 +365,7 @@ int spa_finalize(void* out, const float* out_acc, int B, int H, int Sq, int D, c
   if (!pow2_8_512(D)) return fail(SPA_EUNSUPPORTED, "spa_finalize: head dim %d must be a power of two in [8,512]", D);
   if (!aligned16(out_acc, acc_strides, 4) || !aligned16(out, o_strides, elem_size(dtype)))
     return fail(SPA_EALIGN, "spa_finalize: pointers and row strides must be 16-byte aligned");
-  if ((int64_t)B * H * Sq * (D / 8) / 256 > 0x7ffffff0LL) return fail(SPA_EINVAL, "spa_finalize: grid too large");
+  if (B > 65535 || (int64_t)H * Sq * (D / 8) >= 0x7fffffffLL) return fail(SPA_EINVAL, "spa_finalize: grid too large");
   return launch_result(spa_launch_finalize(out, out_acc, B, H, Sq, D, S3(o_strides), S3(acc_strides), dtype,
                                            (hipStream_t)stream),
                        "spa_finalize");
@@ -403,7 +403,7 @@ int spa_bwd_delta(const void* out, const void* dout, float* delta, int B, int H,
   const int esz = elem_size(dtype);
   if (!aligned16(out, o_strides, esz) || !aligned16(dout, do_strides, esz))
     return fail(SPA_EALIGN, "spa_bwd_delta: pointers and row strides must be 16-byte aligned");
-  if ((int64_t)B * H * Sq * (D / 8) / 256 > 0x7ffffff0LL) return fail(SPA_EINVAL, "spa_bwd_delta: grid too large");
+  if (B > 65535 || (int64_t)H * Sq * (D / 8) >= 0x7fffffffLL) return fail(SPA_EINVAL, "spa_bwd_delta: grid too large");
   return launch_result(spa_launch_delta(out, dout, delta, B, H, Sq, D, S3(o_strides), S3(do_strides), dtype,
                                         (hipStream_t)stream),
                        "spa_bwd_delta");
