@@ -53,9 +53,37 @@ class SpaError(RuntimeError):
         self.code = code
 
 
+class _Recorder:
+    """Stands in for the library while ops.prepared() records a call sequence: every spa_* call is
+    stored with its arguments converted to ctypes objects once, and reports success."""
+
+    def __init__(self, lib):
+        self._lib = lib
+        self.calls = []
+
+    def __getattr__(self, name):
+        fn = getattr(self._lib, name)
+        if name not in SIGNATURES or fn.restype is not _i or name in ("spa_abi_version", "spa_tune"):
+            return fn  # queries run as they are
+
+        def record(*args):
+            if len(args) != len(fn.argtypes):
+                raise TypeError(f"{name}: expected {len(fn.argtypes)} arguments, got {len(args)}")
+            cargs = tuple(a if isinstance(a, ctypes.Array) else t(a) for a, t in zip(args, fn.argtypes))
+            self.calls.append((fn, cargs))
+            return 0
+
+        return record
+
+
+_recorder = None
+
+
 def load():
     """Load the shared library once and attach the prototypes.  Raises if it was not built."""
     global _lib
+    if _recorder is not None:
+        return _recorder
     if _lib is not None:
         return _lib
     if not os.path.exists(LIB_PATH):
@@ -74,12 +102,45 @@ def load():
     return lib
 
 
+_STRIDE_CACHE = {}
+
+
+def _strides(vals, n):
+    """An int64[n] argument; the arrays are read-only for the library, so equal stride tuples share one."""
+    key = tuple(vals)
+    arr = _STRIDE_CACHE.get(key)
+    if arr is None:
+        if len(key) != n:
+            raise ValueError(f"expected {n} strides, got {key}")
+        if len(_STRIDE_CACHE) > 4096:
+            _STRIDE_CACHE.clear()
+        arr = _STRIDE_CACHE[key] = (ctypes.c_int64 * n)(*[int(v) for v in key])
+    return arr
+
+
 def strides3(vals):
-    return _I64x3(*[int(v) for v in vals])
+    return _strides(vals, 3)
 
 
 def strides2(vals):
-    return (ctypes.c_int64 * 2)(*[int(v) for v in vals])
+    return _strides(vals, 2)
+
+
+class recording:
+    """Context manager: inside it, load() hands out a recorder instead of the library."""
+
+    def __enter__(self):
+        global _recorder
+        if _recorder is not None:
+            raise RuntimeError("recording() does not nest")
+        lib = load()
+        _recorder = _Recorder(lib)
+        return _recorder
+
+    def __exit__(self, *exc):
+        global _recorder
+        _recorder = None
+        return False
 
 
 def check(code):

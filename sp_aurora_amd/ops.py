@@ -77,6 +77,52 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+class _Current:
+    """Stands in for torch.cuda.device(d) when d is the current device already (the usual case):
+    entering and leaving the real context costs several microseconds per call."""
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_CURRENT = _Current()
+
+
+def _on(device):
+    idx = device.index
+    if idx is None or idx == torch.cuda.current_device():
+        return _CURRENT
+    return torch.cuda.device(device)
+
+
+def prepared(fn, *args, **kwargs):
+    """Runs `fn(*args, **kwargs)` (any function of this module, or a composition of them) once in
+    recording mode and returns (run, result): `run()` replays exactly the C calls `fn` made, with
+    every argument already converted, and `result` is what `fn` returned (the tensors the calls
+    write into).  For loops that issue the same call on the same buffers many times: a replay costs
+    the ctypes call and the kernel launch, not the Python-side checks (about 11 -> 3 us of host time
+    per call for a merge or a re-layout).
+    The tensors must be kernel-ready as passed (no hidden .contiguous() copies: a copy made while
+    recording would be the buffer the replays read), stay alive and keep their addresses; the stream
+    is the one current while recording."""
+    with _lib.recording() as rec:
+        result = fn(*args, **kwargs)
+    calls = tuple(rec.calls)
+    keep = (args, kwargs, result)  # the recorded pointers refer to these
+
+    def run():
+        for cfn, cargs in calls:
+            rc = cfn(*cargs)
+            if rc:
+                _lib.check(rc)
+        return keep[2]
+
+    return run, result
+
+
 def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None, lse=None, k_scale=None, v_scale=None):
     """Block attention forward -> (out like q, lse fp32 [B,H,Sq]).  Calls spa_flash_fwd, or
     spa_flash_fwd_fp8kv when k, v are torch.float8_e4m3fn (then k_scale, v_scale fp32 [B,H] give
@@ -106,7 +152,7 @@ def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None
     _, os_ = _bhs(out, layout)
     tail = (B, H, Sq, Sk, D, _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
             float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(q), _stream())
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         if fp8:
             ksc, vsc = _fp8_scales(k, v, k_scale, v_scale, B, H)
             _lib.check(lib.spa_flash_fwd_fp8kv(q.data_ptr(), k.data_ptr(), v.data_ptr(), ksc.data_ptr(), vsc.data_ptr(),
@@ -155,7 +201,7 @@ def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layo
     if workspace is None and (fuse == "step" or q.dtype == torch.float32):
         workspace = ring_fwd_workspace(q, ring_size, layout)
     _, os_ = _bhs(out, layout)
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         _lib.check(lib.spa_ring_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
             workspace.data_ptr() if workspace is not None else None,
@@ -178,7 +224,7 @@ def merge(out_acc, lse_acc, blk_out, blk_lse, layout="bshd", init=False):
         raise TypeError("merge: accumulators and lse must be float32")
     if not (lse_acc.is_contiguous() and blk_lse.is_contiguous() and _rows_ok(out_acc, 4)):
         raise ValueError("merge: lse tensors must be contiguous and out_acc 16-byte aligned")
-    with torch.cuda.device(out_acc.device):
+    with _on(out_acc.device):
         _lib.check(lib.spa_merge(
             out_acc.data_ptr(), lse_acc.data_ptr(), blk_out.data_ptr(), blk_lse.data_ptr(),
             B, H, Sq, D, _lib.strides3(as_), _lib.strides3(bs), _dtype_code(blk_out),
@@ -193,7 +239,7 @@ def finalize(out_acc, dtype, layout="bshd", out=None):
     if out is None:
         out = torch.empty(out_acc.shape, dtype=dtype, device=out_acc.device)
     _, os_ = _bhs(out, layout)
-    with torch.cuda.device(out_acc.device):
+    with _on(out_acc.device):
         _lib.check(lib.spa_finalize(out.data_ptr(), out_acc.data_ptr(), B, H, Sq, D,
                                     _lib.strides3(os_), _lib.strides3(as_), _dtype_code(out), _stream()))
     return out
@@ -224,7 +270,7 @@ def _relayout(x, P, s2h, out=None):
     if out is None:
         out = torch.empty(oshape, dtype=x.dtype, device=x.device)
     fn = lib.spa_relayout_s2h if s2h else lib.spa_relayout_h2s
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         _lib.check(fn(x.data_ptr(), out.data_ptr(), P, B, s, H, D, pack, x.element_size(), _stream()))
     return out
 
@@ -248,7 +294,7 @@ def bwd_delta(out, dout, layout="bshd"):
     if shp != (B, H, Sq, D) or out.dtype != dout.dtype:
         raise ValueError("bwd_delta: out and dout must match in shape and dtype")
     delta = torch.empty((B, H, Sq), dtype=torch.float32, device=out.device)
-    with torch.cuda.device(out.device):
+    with _on(out.device):
         _lib.check(lib.spa_bwd_delta(out.data_ptr(), dout.data_ptr(), delta.data_ptr(), B, H, Sq, D,
                                      _lib.strides3(os_), _lib.strides3(ds), _dtype_code(out), _stream()))
     return delta
@@ -288,7 +334,7 @@ def flash_bwd(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, softmax_scale=N
     qs, ks, vs, dos = _bhs(q, layout)[1], _bhs(k, layout)[1], _bhs(v, layout)[1], _bhs(dout, layout)[1]
     if not (_rows_ok(dq_acc, 4) and _rows_ok(dk_acc, 4) and _rows_ok(dv_acc, 4)):
         raise ValueError("flash_bwd: accumulators need an inner stride of 1 and 16-byte aligned rows")
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         _lib.check(lib.spa_flash_bwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
             dq_acc.data_ptr(), dk_acc.data_ptr(), dv_acc.data_ptr(),
@@ -368,7 +414,7 @@ def flash_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
     tail = (cu_q.data_ptr(), cu_k.data_ptr(), cu_q.numel() - 1, H, Tq, Tk, int(max_seqlen_q), int(max_seqlen_k), D,
             _lib.strides2(qs), _lib.strides2(ks), _lib.strides2(vs), _lib.strides2(os_),
             float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(q), _stream())
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         if fp8:
             ksc, vsc = _fp8_scales(k, v, k_scale, v_scale, cu_q.numel() - 1, H)
             _lib.check(lib.spa_flash_fwd_varlen_fp8kv(q.data_ptr(), k.data_ptr(), v.data_ptr(), ksc.data_ptr(), vsc.data_ptr(),
@@ -411,7 +457,7 @@ def flash_bwd_varlen(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, cu_seqle
     cu_q, cu_k = _cu(cu_seqlens_q, q.device, "cu_seqlens_q"), _cu(cu_seqlens_k, q.device, "cu_seqlens_k")
     if softmax_scale is None:
         softmax_scale = D ** (-0.5)
-    with torch.cuda.device(q.device):
+    with _on(q.device):
         _lib.check(lib.spa_flash_bwd_varlen(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
             dq_acc.data_ptr(), dk_acc.data_ptr(), dv_acc.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(),

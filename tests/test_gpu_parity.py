@@ -601,3 +601,29 @@ def test_ring_forward_replays_from_a_captured_graph(fuse):
         torch.cuda.synchronize()
         q.mul_(-1)
         k.mul_(-1)
+
+
+def test_prepared_calls_replay_the_recorded_sequence():
+    """ops.prepared records the C calls of a composition once; a replay must do what the direct
+    calls do, on the same buffers, as often as asked."""
+    B, S, H, D, P = 1, 256, 2, 64, 2
+    q, k, v = [t.to(DEV) for t in rand_qkv((B, S, H, D), 160, torch.bfloat16)]
+    want_out, want_lse = ops.ring_fwd(q, k, v, P, None, True, fuse="step")
+    out = torch.zeros_like(q)
+    lse = torch.zeros((B, H, S), dtype=torch.float32, device=DEV)
+    ws = ops.ring_fwd_workspace(q, P)
+    run, (o2, l2) = ops.prepared(ops.ring_fwd, q, k, v, P, None, True, out=out, lse=lse, workspace=ws, fuse="step")
+    assert o2 is out and l2 is lse
+    assert torch.count_nonzero(out) == 0  # recording launches nothing
+    for _ in range(3):
+        out.zero_()
+        lse.zero_()
+        run()
+        assert torch.equal(out, want_out) and torch.equal(lse, want_lse)
+    # a composition: re-layout there and back
+    x = rand((2, 1, 64, 4, 32), 161, torch.bfloat16).to(DEV)
+    y = torch.empty((2, 1, 128, 2, 32), dtype=x.dtype, device=DEV)
+    back = torch.empty_like(x)
+    run, _ = ops.prepared(lambda: (ops.relayout_s2h(x, 2, out=y), ops.relayout_h2s(y, 2, out=back)))
+    run()
+    assert torch.equal(back, x) and torch.equal(y, ops.relayout_s2h(x, 2))
