@@ -41,6 +41,9 @@ Two helper modes for the HBM traffic figure (roofline.traffic):
                          both the attention kernel and a calibration kernel
   --pmc-summary F W      reads the two counter_collection.csv files of such runs and writes
                          profiles/flash_fwd_traffic.json (no GPU needed)
+`--transient` prints, instead of the benchmark, the per-launch durations of the first 120 launches
+after 3 s of idle together with the clock and board power read from sysfs (what the settle phase
+is for).
 """
 import argparse
 import csv
@@ -484,6 +487,60 @@ def attach_cpu(rows, cpu):
         rows["config5_ring_backward"]["cpu_baseline"] = cpu.backward(16, 120)
 
 
+# ------------------------------------------------------------------------------------ post-idle transient
+def transient(torch, spa, idle_s=3.0, launches=120):
+    """Per-launch durations of the config-3 `all` sweep after an idle period, with the shader
+    clock and board power the driver reports (sysfs) sampled alongside.  One JSON line."""
+    import threading
+
+    def find(pattern):
+        r = sorted(glob.glob(pattern))
+        return r[0] if r else None
+
+    f_sclk = find("/sys/class/drm/card*/device/pp_dpm_sclk")
+    f_pow = find("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") or find("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average")
+
+    def rd(path):
+        try:
+            return open(path).read()
+        except OSError:
+            return ""
+
+    dev = torch.device("cuda:0")
+    q, k, v = rand_tensors(torch, (B, S, H, D), SEED, 3, INPUT_SCALE, torch.bfloat16, dev)
+    step = spa.ring.make_ring_forward_step(q, k, v, D ** -0.5, True, P, fuse="all")
+    step()
+    torch.cuda.synchronize()
+    time.sleep(idle_s)
+    samples, stop = [], []
+
+    def sampler():
+        while not stop:
+            t = time.perf_counter()
+            act = [l for l in rd(f_sclk).splitlines() if l.rstrip().endswith("*")] if f_sclk else []
+            mhz = int("".join(ch for ch in act[0].split(":")[1] if ch.isdigit())) if act else None
+            pw = rd(f_pow).strip() if f_pow else ""
+            samples.append((t, mhz, int(pw) / 1e6 if pw.isdigit() else None))
+            time.sleep(0.002)
+
+    th = threading.Thread(target=sampler)
+    th.start()
+    time.sleep(0.03)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(launches + 1)]
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(launches):
+        step()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    time.sleep(0.03)
+    stop.append(1)
+    th.join()
+    us = [round(ev[i].elapsed_time(ev[i + 1]) * 1e3, 1) for i in range(launches)]
+    print(json.dumps({"workload": "config 3, schedule all: one launch per sweep", "idle_s": idle_s, "us_per_launch": us,
+                      "samples_ms_mhz_watt": [(round((t - t0) * 1e3, 1), m, w) for t, m, w in samples]}))
+
+
 # ------------------------------------------------------------------------------------ traffic helper
 def pmc_summary(fetch_dir, write_dir):
     """FETCH_SIZE / WRITE_SIZE (KiB per dispatch) of the attention kernel, each scaled by what the
@@ -549,6 +606,8 @@ def main():
                     help="which schedule --only-all runs (profiling runs); `value` is always the `all` schedule otherwise")
     ap.add_argument("--traffic-leg", action="store_true", help="also run the calibration copy (for --pmc runs)")
     ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"))
+    ap.add_argument("--transient", action="store_true",
+                    help="instead of the benchmark: per-launch durations of the first 120 launches after 3 s of idle, with clock / power samples")
     ap.add_argument("--workload", default="config3", choices=["config3"] + sorted(ROW_SETS))
     args = ap.parse_args()
     if args.pmc_summary:
@@ -568,6 +627,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.transient:
+        transient(torch, spa)
+        return
     if args.workload != "config3":
         rows = gpu_rows(torch, spa, ops, ROW_SETS[args.workload], args.steps, args.warmup)
         if not args.no_cpu_baseline:
