@@ -446,9 +446,17 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
         m = measure(torch, fstep, 3, 1, **light)
         fwd_flops = 4.0 * Bn * Hn * Sn * Sn * Dn / 2
         tf = fwd_flops / (m["ms_per_step"] * 1e-3) / 1e12
+        sched5 = {}
+        for fuse, launches in (("rank", Pn), ("step", Pn * (Pn + 1) // 2)):
+            f5 = spa.ring.make_ring_forward_step(q, k, v, scale, True, Pn, fuse=fuse)
+            f5()
+            mm = measure(torch, f5, 3, 1, **light)
+            sched5[fuse] = {"ms_per_step": round(mm["ms_per_step"], 4), "tflops": round(fwd_flops / (mm["ms_per_step"] * 1e-3) / 1e12, 2),
+                            "launches_per_step": launches}
+            del f5
         finish("config5_ring_forward", m,
                {"workload": "config 5 forward: bf16 qkv [1,32768,3,16,128] (strided views) causal, ring of 16 chunks of 2048, 16 diagonal + 120 full pairs, schedule 'all'",
-                "flops_per_step": fwd_flops},
+                "flops_per_step": fwd_flops, "other_schedules": sched5},
                tf, "TFLOP/s", roof("mfma", "flash_fwd16_kernel<bf16,128,2>", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", launches_per_step=1))
         fn = lambda: spa.ring.ring_flash_attn_backward(dout, q, k, v, out, lse, scale, True, Pn, fuse="all")
         fn()
