@@ -176,11 +176,14 @@ RING_FUSE = {"step": _lib.SPA_RING_PER_STEP, "rank": _lib.SPA_RING_PER_RANK, "al
 
 
 def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layout="bshd", out=None, lse=None,
-             workspace=None, fuse="rank"):
+             workspace=None, fuse="rank", static_scratch=False):
     """Simulated ring forward of one rank (or all, rank=-1) over the full-sequence q,k,v: one C call
     that enqueues the kernels in ring order.  Calls spa_ring_fwd.  `fuse`: "step" = one launch per
     (q chunk, kv chunk) pair, "rank" = one launch per rank walking its chunks, "all" = one launch.
-    Returns (out like q, lse fp32 [B,H,S]); with rank >= 0 only that rank's rows are written."""
+    Returns (out like q, lse fp32 [B,H,S]); with rank >= 0 only that rank's rows are written.
+    static_scratch=True calls spa_ring_fwd_static instead: no workspace tensor, the library's built-in
+    32 MiB buffer holds the running output between step launches (for callers that must not allocate;
+    calls that overlap on one device race)."""
     lib = _lib.load()
     q, k, v = _prep(q), _prep(k), _prep(v)
     if not (q.dtype == k.dtype == v.dtype):
@@ -198,17 +201,21 @@ def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layo
         lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
     if fuse not in RING_FUSE:
         raise ValueError(f"fuse must be one of {sorted(RING_FUSE)}, got {fuse!r}")
-    if workspace is None and (fuse == "step" or q.dtype == torch.float32):
+    if static_scratch and workspace is not None:
+        raise ValueError("static_scratch=True takes no workspace")
+    if workspace is None and not static_scratch and (fuse == "step" or q.dtype == torch.float32):
         workspace = ring_fwd_workspace(q, ring_size, layout)
     _, os_ = _bhs(out, layout)
-    with _on(q.device):
-        _lib.check(lib.spa_ring_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
-            workspace.data_ptr() if workspace is not None else None,
-            B, H, S, D, int(ring_size), int(rank),
+    tail = (B, H, S, D, int(ring_size), int(rank),
             _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
             float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE,
-            _dtype_code(q), RING_FUSE[fuse], _stream()))
+            _dtype_code(q), RING_FUSE[fuse], _stream())
+    with _on(q.device):
+        if static_scratch:
+            _lib.check(lib.spa_ring_fwd_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), *tail))
+        else:
+            _lib.check(lib.spa_ring_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                                        workspace.data_ptr() if workspace is not None else None, *tail))
     return out, lse
 
 

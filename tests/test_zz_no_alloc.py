@@ -80,3 +80,36 @@ def test_static_scratch_rejects_sizes_beyond_the_buffer():
                                  _lib.SPA_RING_PER_STEP, None)
     assert rc == -1 and b"built-in buffer" in lib.spa_last_error()
     torch.cuda.synchronize()
+
+
+def test_static_scratch_entry_under_graph_capture():
+    """What the entry point is for: a per-step ring forward captured in a graph without any
+    workspace tensor; every replay (eager work and synchronisations in between) must equal the
+    eager result of spa_ring_fwd."""
+    from sp_aurora_amd import ops
+    B, S, H, D, P = 1, 1024, 4, 128, 4
+    q, k, v = (t.to(DEV) for t in rand_qkv((B, S, H, D), 310, torch.bfloat16))
+    want_out, want_lse = ops.ring_fwd(q, k, v, P, None, True, fuse="step")
+    out = torch.empty_like(q)
+    lse = torch.empty((B, H, S), dtype=torch.float32, device=DEV)
+    run = lambda: ops.ring_fwd(q, k, v, P, None, True, out=out, lse=lse, fuse="step", static_scratch=True)
+    run()  # the first call on a device looks the buffer's address up: outside the capture
+    torch.cuda.synchronize()
+    assert torch.equal(out, want_out) and torch.equal(lse, want_lse)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run()
+    for rep in range(3):
+        out.fill_(7)
+        lse.fill_(7)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want_out) and torch.equal(lse, want_lse), f"replay {rep} differs"
+        q.mul_(-1)
+        torch.cuda.synchronize()
+        q.mul_(-1)
