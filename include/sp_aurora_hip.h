@@ -148,6 +148,22 @@ int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* 
                  float scale, int mask_mode, int dtype, int fuse, void* stream);
 
 /*
+ * spa_ring_fwd with e4m3 K / V as in spa_flash_fwd_fp8kv: k8, v8 [B,H,S,D] by strides in bytes,
+ * k_scale / v_scale fp32 contiguous [B,H] — one scale per (batch, head) for the whole sequence, i.e.
+ * every ring chunk quantised on the same grid (a ring whose ranks quantise their chunks on their
+ * own would rescale to a common scale before the exchange).  q / out bf16 or fp16, D in {64, 128};
+ * all three `fuse` modes; workspace as for spa_ring_fwd.  Same call sites as spa_flash_fwd_fp8kv,
+ * seen from the ring loop (sp_aurora/intel_ring_flash_attn.py:72-148).
+ */
+int spa_ring_fwd_fp8kv(const void* q, const void* k8, const void* v8,
+                       const float* k_scale, const float* v_scale,
+                       void* out, float* lse, void* workspace,
+                       int B, int H, int S, int D, int P, int rank,
+                       const int64_t q_strides[3], const int64_t k_strides[3],
+                       const int64_t v_strides[3], const int64_t o_strides[3],
+                       float scale, int mask_mode, int dtype, int fuse, void* stream);
+
+/*
  * spa_ring_fwd for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc): the same call without the workspace
  * argument.  The scratch is a fixed buffer of SPA_STATIC_SCRATCH_BYTES inside the library's

@@ -215,7 +215,9 @@ int static_scratch(void** ptr) {
 }
 
 // `what` names the entry point in messages; `ws_bytes` < 0: the caller vouches for the workspace size.
-int ring_fwd(const char* what, const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
+// k_scale / v_scale non-null: K and V are e4m3 bytes with one scale per (batch, head) for the whole sequence.
+int ring_fwd(const char* what, const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
+             void* out, float* lse, void* workspace,
              int64_t ws_bytes, int B, int H, int S, int D, int P, int rank, const int64_t q_strides[3],
              const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3], float scale,
              int mask_mode, int dtype, int fuse, void* stream) {
@@ -229,11 +231,17 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, void
   if (fuse < SPA_RING_PER_STEP || fuse > SPA_RING_ALL_RANKS) return fail(SPA_EINVAL, "%s: bad fuse mode %d", what, fuse);
   if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "%s: softmax scale must be positive and finite", what);
   if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "%s: head dim %d not in {32,64,128}", what, D);
-  const int esz = elem_size(dtype);
-  if (!aligned16(q, q_strides, esz) || !aligned16(k, k_strides, esz) || !aligned16(v, v_strides, esz) ||
+  const bool kv8 = k_scale || v_scale;
+  if (kv8 && (!k_scale || !v_scale)) return fail(SPA_EINVAL, "%s: null scale pointer", what);
+  if (kv8 && dtype == SPA_F32) return fail(SPA_EUNSUPPORTED, "%s: e4m3 K/V go with bf16 or fp16 queries", what);
+  if (kv8 && D == 32) return fail(SPA_EUNSUPPORTED, "%s: e4m3 K/V need head dim 64 or 128", what);
+  const int esz = elem_size(dtype), kesz = kv8 ? 1 : esz;
+  const bool kv_aligned = kv8 ? aligned8(k, k_strides, 3) && aligned8(v, v_strides, 3) && (((uintptr_t)k_scale | (uintptr_t)v_scale) & 3) == 0
+                              : aligned16(k, k_strides, esz) && aligned16(v, v_strides, esz);
+  if (!aligned16(q, q_strides, esz) || !kv_aligned ||
       !aligned16(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0 || ((uintptr_t)workspace & 15) != 0)
-    return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned", what);
-  if (!span_ok(S, k_strides[2], D, esz) || !span_ok(S, v_strides[2], D, esz))
+    return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned (8-byte for e4m3 K/V)", what);
+  if (!span_ok(S, k_strides[2], D, kesz) || !span_ok(S, v_strides[2], D, kesz))
     return fail(SPA_EUNSUPPORTED, "%s: K/V of one (batch, head) span more than 2 GiB", what);
   const bool causal = mask_mode == SPA_MASK_CAUSAL;
   const int s = S / P;
@@ -270,7 +278,7 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, void
   p.P = P;
   p.epi = SPA_EPI_PLAIN;
   p.cu_q = nullptr; p.cu_k = nullptr;
-  p.k_scale = nullptr; p.v_scale = nullptr;
+  p.k_scale = k_scale; p.v_scale = v_scale;
 
   if (fuse == SPA_RING_ALL_RANKS) {  // one launch: every requested rank, every step
     p.rank0 = r_lo; p.nranks = r_hi - r_lo; p.t_begin = 0; p.t_count = -1;
@@ -334,8 +342,17 @@ int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* 
                  int H, int S, int D, int P, int rank, const int64_t q_strides[3], const int64_t k_strides[3],
                  const int64_t v_strides[3], const int64_t o_strides[3], float scale, int mask_mode, int dtype,
                  int fuse, void* stream) {
-  return ring_fwd("spa_ring_fwd", q, k, v, out, lse, workspace, -1, B, H, S, D, P, rank, q_strides, k_strides,
+  return ring_fwd("spa_ring_fwd", q, k, v, nullptr, nullptr, out, lse, workspace, -1, B, H, S, D, P, rank, q_strides, k_strides,
                   v_strides, o_strides, scale, mask_mode, dtype, fuse, stream);
+}
+
+int spa_ring_fwd_fp8kv(const void* q, const void* k8, const void* v8, const float* k_scale, const float* v_scale,
+                       void* out, float* lse, void* workspace, int B, int H, int S, int D, int P, int rank,
+                       const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                       const int64_t o_strides[3], float scale, int mask_mode, int dtype, int fuse, void* stream) {
+  if (!k_scale || !v_scale) return fail(SPA_EINVAL, "spa_ring_fwd_fp8kv: null scale pointer");
+  return ring_fwd("spa_ring_fwd_fp8kv", q, k8, v8, k_scale, v_scale, out, lse, workspace, -1, B, H, S, D, P, rank, q_strides,
+                  k_strides, v_strides, o_strides, scale, mask_mode, dtype, fuse, stream);
 }
 
 int64_t spa_static_scratch_bytes(void) { return (int64_t)SPA_STATIC_SCRATCH_BYTES; }
@@ -347,7 +364,7 @@ int spa_ring_fwd_static(const void* q, const void* k, const void* v, void* out, 
   void* ws = nullptr;
   const int rc = static_scratch(&ws);
   if (rc != SPA_OK) return rc;
-  return ring_fwd("spa_ring_fwd_static", q, k, v, out, lse, ws, (int64_t)SPA_STATIC_SCRATCH_BYTES, B, H, S, D, P,
+  return ring_fwd("spa_ring_fwd_static", q, k, v, nullptr, nullptr, out, lse, ws, (int64_t)SPA_STATIC_SCRATCH_BYTES, B, H, S, D, P,
                   rank, q_strides, k_strides, v_strides, o_strides, scale, mask_mode, dtype, fuse, stream);
 }
 

@@ -176,18 +176,28 @@ RING_FUSE = {"step": _lib.SPA_RING_PER_STEP, "rank": _lib.SPA_RING_PER_RANK, "al
 
 
 def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layout="bshd", out=None, lse=None,
-             workspace=None, fuse="rank", static_scratch=False):
+             workspace=None, fuse="rank", static_scratch=False, k_scale=None, v_scale=None):
     """Simulated ring forward of one rank (or all, rank=-1) over the full-sequence q,k,v: one C call
     that enqueues the kernels in ring order.  Calls spa_ring_fwd.  `fuse`: "step" = one launch per
     (q chunk, kv chunk) pair, "rank" = one launch per rank walking its chunks, "all" = one launch.
     Returns (out like q, lse fp32 [B,H,S]); with rank >= 0 only that rank's rows are written.
+    k, v may be torch.float8_e4m3fn with k_scale, v_scale fp32 [B,H] (spa_ring_fwd_fp8kv).
     static_scratch=True calls spa_ring_fwd_static instead: no workspace tensor, the library's built-in
     32 MiB buffer holds the running output between step launches (for callers that must not allocate;
     calls that overlap on one device race)."""
     lib = _lib.load()
-    q, k, v = _prep(q), _prep(k), _prep(v)
-    if not (q.dtype == k.dtype == v.dtype):
-        raise TypeError("q, k, v must share a dtype")
+    fp8 = k.dtype == FP8 or v.dtype == FP8
+    if fp8:
+        if static_scratch:
+            raise ValueError("static_scratch=True has no e4m3 K/V form")
+        q = _prep(q)
+        k, v = [t if t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1]) and t.data_ptr() % 8 == 0 else t.contiguous() for t in (k, v)]
+        if not k.is_cuda or not v.is_cuda:
+            raise ValueError("sp_aurora_amd kernels need tensors on a HIP device (got a CPU tensor)")
+    else:
+        q, k, v = _prep(q), _prep(k), _prep(v)
+        if not (q.dtype == k.dtype == v.dtype):
+            raise TypeError("q, k, v must share a dtype")
     (B, H, S, D), qs = _bhs(q, layout)
     shp_k, ks = _bhs(k, layout)
     shp_v, vs = _bhs(v, layout)
@@ -211,7 +221,12 @@ def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layo
             float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE,
             _dtype_code(q), RING_FUSE[fuse], _stream())
     with _on(q.device):
-        if static_scratch:
+        if fp8:
+            ksc, vsc = _fp8_scales(k, v, k_scale, v_scale, B, H)
+            _lib.check(lib.spa_ring_fwd_fp8kv(q.data_ptr(), k.data_ptr(), v.data_ptr(), ksc.data_ptr(), vsc.data_ptr(),
+                                              out.data_ptr(), lse.data_ptr(),
+                                              workspace.data_ptr() if workspace is not None else None, *tail))
+        elif static_scratch:
             _lib.check(lib.spa_ring_fwd_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), *tail))
         else:
             _lib.check(lib.spa_ring_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),

@@ -119,6 +119,20 @@ def test_varlen_forward_with_e4m3_kv(lengths, H, D, causal):
     check_lse(lse, want_lse)
 
 
+@pytest.mark.parametrize("fuse", ["step", "rank", "all"])
+@pytest.mark.parametrize("B,S,H,D,P,causal", [(1, 512, 2, 128, 4, True), (2, 384, 3, 64, 3, False), (1, 1024, 4, 128, 8, True)])
+def test_ring_forward_with_e4m3_kv(B, S, H, D, P, causal, fuse):
+    """The three ring schedules over e4m3 K / V (one scale per (batch, head) for the whole sequence)
+    against full attention on the dequantised tensors."""
+    q = rand((B, S, H, D), 560, torch.bfloat16)
+    k8, ksc, k_deq = quantised((B, S, H, D), 561, "bshd", spread=1.2)
+    v8, vsc, v_deq = quantised((B, S, H, D), 562, "bshd")
+    want_out, want_lse = O.full_attention(q, k_deq, v_deq, None, causal)
+    out, lse = ops.ring_fwd(q.to(DEV), k8.to(DEV), v8.to(DEV), P, None, causal, fuse=fuse, k_scale=ksc, v_scale=vsc)
+    check_out(out, want_out, torch.bfloat16)
+    check_lse(lse, want_lse)
+
+
 def test_e4m3_kv_argument_checks():
     q = rand((1, 2, 64, 64), 550, torch.bfloat16).to(DEV)
     k8 = torch.zeros((1, 2, 64, 64), dtype=torch.float8_e4m3fn, device=DEV)
