@@ -71,7 +71,8 @@ int spa_device_info(char* buf, int n);
  *  sp_aurora/intel_flash_attn_optimized.py:95-225) and the native
  * `forward(...)` of the reference plugin (sp_aurora/sycl_bindings/bindings.cpp:50-272).
  * q: [B,H,Sq,D] by strides, k,v: [B,H,Sk,D] by strides, out: like q.
- * D in {32, 64, 128}.  scale must be > 0.  Any Sq, Sk >= 1.
+ * D in {32, 64, 128}.  Any finite scale (negative and zero included, as in the reference).
+ * Any Sq, Sk >= 1.
  */
 int spa_flash_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
                   int B, int H, int Sq, int Sk, int D,

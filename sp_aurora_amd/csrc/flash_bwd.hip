@@ -242,6 +242,7 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
   const float l2 = p.lse[li] * 1.4426950408889634f;
   const float dl = p.delta[li];
   const float c = p.scale_log2;
+  const float hidden = c < 0.f ? INFINITY : -INFINITY;  // a hidden score: exp2(hidden * c - lse) = 0 for either sign of the scale
   const int lim = p.causal ? (qrow < p.Sk - 1 ? qrow : p.Sk - 1) : p.Sk - 1;  // last visible key
 
   const int kv_end = p.causal ? (q0 + NW * 32 < p.Sk ? q0 + NW * 32 : p.Sk) : p.Sk;
@@ -358,7 +359,7 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
       if ((p.causal && key0 + 31 > qw0) || key0 + 31 >= p.Sk) {
 #pragma unroll
         for (int v = 0; v < 16; ++v)
-          if (key0 + 8 * (v >> 2) + 4 * hh + (v & 3) > lim) sc[v] = -INFINITY;
+          if (key0 + 8 * (v >> 2) + 4 * hh + (v & 3) > lim) sc[v] = hidden;
       }
       if (!MIXED) {
         zero16(sn);
@@ -486,6 +487,7 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
     vf[ks] = as_frag<frag>(*(const u32x4*)(vp + (int64_t)krow_c * p.vs.s + ks * 16 + hh * 8));
   }
   const float c = p.scale_log2;
+  const float hidden = c < 0.f ? INFINITY : -INFINITY;  // a hidden score: exp2(hidden * c - lse) = 0 for either sign of the scale
 
   // causal: query rows before the first key of this workgroup see none of its keys
   const int it0 = p.causal ? k0 / BWD_ROWS : 0;
@@ -606,7 +608,7 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
         if (p.causal && kw0 + 31 > r0) {     // diagonal: a key sees only the queries at or after it
 #pragma unroll
           for (int v = 0; v < 16; ++v)
-            if (krow > r0 + 8 * (v >> 2) + 4 * hh + (v & 3)) sc[v] = -INFINITY;
+            if (krow > r0 + 8 * (v >> 2) + 4 * hh + (v & 3)) sc[v] = hidden;
         }
         // lse (times -log2 e) and delta of this lane's 16 query rows
         float nl[16], de[16];

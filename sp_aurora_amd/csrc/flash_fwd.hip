@@ -154,9 +154,13 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const int qrow_c = qrow < p.Sq ? qrow : p.Sq - 1;
 
   frag qf[D / 16];
+  const unsigned qsign = p.negq ? 0x80008000u : 0u;  // negative softmax scale: -q with |scale|
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks)
-    qf[ks] = as_frag<frag>(*(const u32x4*)(qp + (int64_t)qrow_c * p.qs.s + ks * 16 + hh * 8));
+  for (int ks = 0; ks < D / 16; ++ks) {
+    u32x4 x = *(const u32x4*)(qp + (int64_t)qrow_c * p.qs.s + ks * 16 + hh * 8);
+    x[0] ^= qsign; x[1] ^= qsign; x[2] ^= qsign; x[3] ^= qsign;
+    qf[ks] = as_frag<frag>(x);
+  }
 
   // ---- the schedule of this workgroup ----
   // K/V hold P chunks of Sk keys.  Ring step t of rank r uses chunk (r - t) mod P; a causal ring
@@ -828,8 +832,10 @@ __global__ void __launch_bounds__(FWD_THREADS, 1) flash_fwd32_kernel(const FwdPa
   // 8*(u/4) + 4*hh + (u%4): a lane's dims come as 16-byte groups.
   f32x4 qf[D / 8];
 #pragma unroll
-  for (int g = 0; g < D / 8; ++g)
+  for (int g = 0; g < D / 8; ++g) {
     qf[g] = *(const f32x4*)(qp + (int64_t)qrow_c * p.qs.s + 8 * g + 4 * hh);
+    if (p.negq) qf[g] = -qf[g];  // negative softmax scale: -q with |scale|
+  }
 
   const int kv_end = p.causal ? (q0 + FWD_BM < p.Sk ? q0 + FWD_BM : p.Sk) : p.Sk;
   const int nt = (kv_end + F32_BN - 1) / F32_BN;

@@ -68,6 +68,12 @@ bool span_ok(int64_t rows, int64_t row_stride, int D, int esz) {
   return ((rows - 1) * row_stride + D) * esz < 0x7fffffffLL;
 }
 
+// Any finite softmax scale, as in the reference.  Zero is carried as 1e-30: every finite score then
+// scales to (practically) zero while a hidden score stays at -inf instead of becoming inf * 0;
+// the results differ from exact arithmetic by less than 1e-25.
+bool scale_ok(float scale) { return scale == scale && scale > -INFINITY && scale < INFINITY; }
+float scale_eff(float scale) { return scale == 0.f ? 1e-30f : scale; }
+
 int launch_result(hipError_t e, const char* what) {
   if (e == hipSuccess) return SPA_OK;
   if (e == hipErrorInvalidValue) return fail(SPA_EUNSUPPORTED, "%s: no kernel for this head dim / dtype", what);
@@ -120,7 +126,7 @@ int flash_fwd(const char* what, const void* q, const void* k, const void* v, con
   if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "%s: bad dtype %d", what, dtype);
   if (kv8 && dtype == SPA_F32) return fail(SPA_EUNSUPPORTED, "%s: e4m3 K/V go with bf16 or fp16 queries", what);
   if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "%s: bad mask_mode %d", what, mask_mode);
-  if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "%s: softmax scale must be positive and finite", what);
+  if (!scale_ok(scale)) return fail(SPA_EINVAL, "%s: softmax scale must be finite", what);
   if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "%s: head dim %d not in {32,64,128}", what, D);
   if (kv8 && D == 32) return fail(SPA_EUNSUPPORTED, "%s: e4m3 K/V need head dim 64 or 128", what);
   const int esz = elem_size(dtype), kesz = kv8 ? 1 : esz;
@@ -135,8 +141,9 @@ int flash_fwd(const char* what, const void* q, const void* k, const void* v, con
   p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
   p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
   p.qs = S3(q_strides); p.ks = S3(k_strides); p.vs = S3(v_strides); p.os = S3(o_strides);
-  p.scale = scale;
-  p.scale_log2 = scale * 1.4426950408889634f;
+  p.scale = scale_eff(scale);
+  p.scale_log2 = fabsf(scale_eff(scale)) * 1.4426950408889634f;
+  p.negq = scale < 0.f;
   p.causal = mask_mode == SPA_MASK_CAUSAL;
   p.nqt = 0;
   p.lse_bh = Sq;
@@ -229,7 +236,7 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "%s: bad dtype %d", what, dtype);
   if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "%s: bad mask_mode %d", what, mask_mode);
   if (fuse < SPA_RING_PER_STEP || fuse > SPA_RING_ALL_RANKS) return fail(SPA_EINVAL, "%s: bad fuse mode %d", what, fuse);
-  if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "%s: softmax scale must be positive and finite", what);
+  if (!scale_ok(scale)) return fail(SPA_EINVAL, "%s: softmax scale must be finite", what);
   if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "%s: head dim %d not in {32,64,128}", what, D);
   const bool kv8 = k_scale || v_scale;
   if (kv8 && (!k_scale || !v_scale)) return fail(SPA_EINVAL, "%s: null scale pointer", what);
@@ -268,8 +275,9 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
   p.B = B; p.H = H; p.Sq = s; p.Sk = s;
   p.qs = S3(q_strides); p.ks = S3(k_strides); p.vs = S3(v_strides); p.os = S3(o_strides);
-  p.scale = scale;
-  p.scale_log2 = scale * 1.4426950408889634f;
+  p.scale = scale_eff(scale);
+  p.scale_log2 = fabsf(scale_eff(scale)) * 1.4426950408889634f;
+  p.negq = scale < 0.f;
   p.causal = causal;
   p.nqt = 0;
   p.lse_bh = S;
@@ -438,7 +446,7 @@ int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout,
   if (!dims_ok(B, H, Sq, D) || Sk <= 0) return fail(SPA_EINVAL, "spa_flash_bwd: sizes must be positive");
   if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "spa_flash_bwd: bad dtype %d", dtype);
   if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "spa_flash_bwd: bad mask_mode %d", mask_mode);
-  if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "spa_flash_bwd: softmax scale must be positive and finite");
+  if (!scale_ok(scale)) return fail(SPA_EINVAL, "spa_flash_bwd: softmax scale must be finite");
   if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "spa_flash_bwd: head dim %d not in {32,64,128}", D);
   const int esz = elem_size(dtype);
   if (!aligned16(q, q_strides, esz) || !aligned16(k, k_strides, esz) || !aligned16(v, v_strides, esz) ||
@@ -456,8 +464,8 @@ int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout,
   p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
   p.qs = S3(q_strides); p.ks = S3(k_strides); p.vs = S3(v_strides); p.dos = S3(do_strides);
   p.dqs = S3(dq_strides); p.dks = S3(dk_strides); p.dvs = S3(dv_strides);
-  p.scale = scale;
-  p.scale_log2 = scale * 1.4426950408889634f;
+  p.scale = scale_eff(scale);
+  p.scale_log2 = scale_eff(scale) * 1.4426950408889634f;
   p.causal = mask_mode == SPA_MASK_CAUSAL;
   p.nqt = 0;
   p.nkt = 0;
@@ -485,7 +493,7 @@ int varlen_sizes_ok(const char* what, const void* cu_q, const void* cu_k, int ns
                 what, nseq, H, total_q, total_k, max_sq, max_sk);
   if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "%s: bad dtype %d", what, dtype);
   if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "%s: bad mask_mode %d", what, mask_mode);
-  if (!(scale > 0.f) || !(scale < INFINITY)) return fail(SPA_EINVAL, "%s: softmax scale must be positive and finite", what);
+  if (!scale_ok(scale)) return fail(SPA_EINVAL, "%s: softmax scale must be finite", what);
   if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "%s: head dim %d not in {32,64,128}", what, D);
   if ((max_sq + 127) / 128 > 65535 || (int64_t)nseq * H * ((max_sq + 127) / 128) > 0x7fffffffLL ||
       (int64_t)nseq * H * ((max_sk + 127) / 128) > 0x7fffffffLL)
@@ -522,8 +530,9 @@ int flash_fwd_varlen(const char* what, const void* q, const void* k, const void*
   p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
   p.B = nseq; p.H = H; p.Sq = max_sq; p.Sk = max_sk;
   p.qs = S2(q_strides); p.ks = S2(k_strides); p.vs = S2(v_strides); p.os = S2(o_strides);
-  p.scale = scale;
-  p.scale_log2 = scale * 1.4426950408889634f;
+  p.scale = scale_eff(scale);
+  p.scale_log2 = fabsf(scale_eff(scale)) * 1.4426950408889634f;
+  p.negq = scale < 0.f;
   p.causal = mask_mode == SPA_MASK_CAUSAL;
   p.nqt = 0;
   p.lse_bh = total_q;
@@ -589,8 +598,8 @@ int spa_flash_bwd_varlen(const void* q, const void* k, const void* v, const void
   p.B = nseq; p.H = H; p.Sq = max_sq; p.Sk = max_sk;
   p.qs = S2(q_strides); p.ks = S2(k_strides); p.vs = S2(v_strides); p.dos = S2(do_strides);
   p.dqs = S2(dq_strides); p.dks = S2(dk_strides); p.dvs = S2(dv_strides);
-  p.scale = scale;
-  p.scale_log2 = scale * 1.4426950408889634f;
+  p.scale = scale_eff(scale);
+  p.scale_log2 = scale_eff(scale) * 1.4426950408889634f;
   p.causal = mask_mode == SPA_MASK_CAUSAL;
   p.nqt = 0;
   p.nkt = 0;

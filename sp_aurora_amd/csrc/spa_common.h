@@ -23,7 +23,9 @@ struct FwdParams {
   int B, H, Sq, Sk;
   Strides3 qs, ks, vs, os;
   float scale;       // softmax scale
-  float scale_log2;  // scale * log2(e)
+  float scale_log2;  // |scale| * log2(e): the forward kernels take the row max on raw scores, so a
+                     // negative scale travels as negq (q is negated on its way into registers)
+  int negq;
   int causal;        // 1: query row i sees keys j <= i (top-left aligned)
   int nqt;           // number of query tiles per (batch, head)
   int64_t lse_bh;    // elements between consecutive (batch, head) rows of lse

@@ -47,8 +47,9 @@ def test_bad_arguments_return_codes_without_touching_a_device():
     p = ctypes.c_void_p(4096)  # aligned, never dereferenced: every check below fails before a launch
     # unsupported head dim
     assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 8, 8, 48, st, st, st, st, 1.0, 0, 1, None) == -2
-    # non-positive scale
-    assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 8, 8, 64, st, st, st, st, 0.0, 0, 1, None) == -1
+    # a scale that is not finite (any finite one is accepted, negative and zero included)
+    assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 8, 8, 64, st, st, st, st, float("nan"), 0, 1, None) == -1
+    assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 8, 8, 64, st, st, st, st, float("inf"), 0, 1, None) == -1
     # bad dtype / mask
     assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 8, 8, 64, st, st, st, st, 1.0, 0, 7, None) == -1
     assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 8, 8, 64, st, st, st, st, 1.0, 5, 1, None) == -1

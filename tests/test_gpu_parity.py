@@ -627,3 +627,32 @@ def test_prepared_calls_replay_the_recorded_sequence():
     run, _ = ops.prepared(lambda: (ops.relayout_s2h(x, 2, out=y), ops.relayout_h2s(y, 2, out=back)))
     run()
     assert torch.equal(back, x) and torch.equal(y, ops.relayout_s2h(x, 2))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("scale", [-0.25, 0.0, -1.0 / 8])
+@pytest.mark.parametrize("causal", [False, True])
+def test_any_finite_softmax_scale_forward_and_backward(scale, causal, dtype):
+    """The reference takes whatever softmax_scale it is given (sp_aurora/intel_flash_attn.py:46-47,
+    a plain multiplication); so does the HIP path: negative scales, and zero (uniform attention
+    over the visible keys, lse = log of their number, zero gradients for q and k)."""
+    B, S, H, D, P = 1, 200, 2, 64, 1
+    q, k, v, dout = rand_qkv((B, S, H, D), 170, dtype, n=4)
+    want_out, want_lse = O.full_attention(q, k, v, scale, causal)
+    want = O.attn_backward_autograd(q, k, v, dout, scale, causal)
+    xs = [t.to(DEV).requires_grad_(True) for t in (q, k, v)]
+    out, lse, _ = spa.ring_flash_attn_func(*xs, softmax_scale=scale, causal=causal, return_attn_probs=True)
+    check_out(out, want_out, dtype)
+    check_lse(lse, want_lse)
+    out.backward(dout.to(DEV))
+    for x, w, name in zip(xs, want, "qkv"):
+        if w.abs().max() == 0:
+            assert x.grad.abs().max() < 1e-20, f"d{name} should vanish"
+        else:
+            check_grad(x.grad, w, dtype, "d" + name)
+    # the ring schedules take the same scale
+    P = 4
+    for fuse in ("step", "rank", "all"):
+        o2, l2 = spa.ring.ring_flash_attn_forward(q.to(DEV), k.to(DEV), v.to(DEV), scale, causal, P, fuse=fuse)
+        check_out(o2, want_out, dtype)
+        check_lse(l2, want_lse)
