@@ -262,6 +262,13 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
 #pragma unroll
     for (int q = 0; q < C::NDMA; ++q) vld.load(q, i < nt, i * BWD_ROWS, dst + C::TILEB);
   };
+  auto issue_one = [&](int i, int n) {  // load n of tile i's G::NL, in issue_tile's order
+    const unsigned dst = stage_of(i) + w * 1024;
+    if (n < C::NDMA)
+      kld.load(n, i < nt, i * BWD_ROWS, dst);
+    else
+      vld.load(n - C::NDMA, i < nt, i * BWD_ROWS, dst + C::TILEB);
+  };
 
   f32x16 dq[D / 32];
 #pragma unroll
@@ -344,11 +351,13 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
   set_addresses(0);
 #pragma unroll
   for (int j = 0; j < BWD_LOOK; ++j) win[j] = fetch(j);
+  // The loads of tile i + 3 go out one at a time between the MFMAs of the pass: issued in one burst
+  // after the barrier, they hold up the wave's instruction stream while the memory pipeline takes them in.
+  constexpr int LOAD_GAP = NBODY / G::NL;
   for (int i = 0; i < nt; ++i) {
     // tile i+1 must have landed before this body reads it; tile i-1 is free for tile i+3
     wait_loads_but<G::NL>();
     __syncthreads();
-    issue_tile(i + 3);
     set_addresses(i);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -403,6 +412,7 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
           else
             dq[db] = M::run(a, dsf[u], dq[db]);
         }
+        if (J % LOAD_GAP == LOAD_GAP / 2 && J / LOAD_GAP < G::NL) issue_one(i + 3, J / LOAD_GAP);
         __builtin_amdgcn_sched_barrier(0);
       }
       sc = sn;
@@ -513,6 +523,17 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
     load_to_lds_b32(stat_rsrc, i < nt ? (unsigned)(i * BWD_ROWS + lane) * 4u : OFF_NONE,
                     st + 2 * C::TILEB + (w & 1) * (BWD_ROWS * 4));
   };
+  auto issue_one = [&](int i, int n) {  // load n of tile i's G::NL, in issue_tile's order
+    const unsigned st = stage_of(i);
+    const unsigned dst = st + w * 1024;
+    if (n < C::NDMA)
+      qld.load(n, i < nt, i * BWD_ROWS, dst);
+    else if (n < 2 * C::NDMA)
+      dold.load(n - C::NDMA, i < nt, i * BWD_ROWS, dst + C::TILEB);
+    else
+      load_to_lds_b32(stat_rsrc, i < nt ? (unsigned)(i * BWD_ROWS + lane) * 4u : OFF_NONE,
+                      st + 2 * C::TILEB + (w & 1) * (BWD_ROWS * 4));
+  };
 
   f32x16 dk[D / 32], dv[D / 32];
 #pragma unroll
@@ -596,10 +617,13 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
     set_addresses(it0);
 #pragma unroll
     for (int j = 0; j < BWD_LOOK; ++j) win[j] = fetch(j);
+    // The loads of tile i + 3 go out one at a time between the MFMAs of the pass: issued in one
+    // burst after the barrier, they hold up the wave's instruction stream while the memory pipeline
+    // takes them in.
+    constexpr int LOAD_GAP = NBODY / G::NL;
     for (int i = it0; i < nt; ++i) {
       wait_loads_but<G::NL>();
       __syncthreads();
-      issue_tile(i + 3);
       set_addresses(i);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -675,6 +699,7 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
               MA::acc_a(dv[db], a, pf[u]);
             }
           }
+          if (J % LOAD_GAP == LOAD_GAP / 2 && J / LOAD_GAP < G::NL) issue_one(i + 3, J / LOAD_GAP);
           __builtin_amdgcn_sched_barrier(0);
         }
         sc = sn;
