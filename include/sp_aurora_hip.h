@@ -127,7 +127,10 @@ int spa_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* 
  * between steps).
  * `fuse` chooses how the schedule maps onto launches (the results agree to rounding):
  *   SPA_RING_PER_STEP   one block-attention launch per visited (q chunk, kv chunk) pair, as a
- *                       multi-GPU ring would issue them; needs the workspace.
+ *                       multi-GPU ring would issue them; needs the workspace.  Every step but a
+ *                       rank's last leaves its block output (in q's type, as the reference's
+ *                       block_out) and lse there; the last step's epilogue applies
+ *                       update_out_and_lse to all of them and its own block in one pass.
  *   SPA_RING_PER_RANK   one launch per rank: a workgroup keeps its query tile and its output
  *                       accumulators in registers and walks the rank's KV chunks in ring order,
  *                       so the merge is the online softmax itself and no accumulator leaves the CU.
@@ -135,7 +138,9 @@ int spa_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* 
  * fp32 always runs per step, whatever `fuse` says.  No collectives: the "ring" is the order in
  * which chunks are visited.
  * workspace: device scratch of spa_ring_fwd_workspace_bytes() bytes (16-byte aligned), owned
- * by the caller; it holds the fp32 running output of one rank between separate step launches.
+ * by the caller; between separate step launches it holds one rank's earlier block results (16-bit
+ * types: P - 1 outputs [B,S/P,H,D] in q's type and their lse; fp32: the running output, one block's
+ * output and lse).
  * It may be NULL only when no launch needs it: 16-bit types in the fused modes, or a schedule in
  * which no rank visits more than one block (P = 1; causal rank 0).  fp32 inputs with more than
  * one block per rank always need it (SPA_EINVAL otherwise).

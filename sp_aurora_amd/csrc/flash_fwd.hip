@@ -87,9 +87,12 @@ __device__ __forceinline__ int v_swizzle(int row) {
 // global -> registers -> LDS and are widened to T on the way (every e4m3 value is exact in bf16 and
 // fp16), once per workgroup, so LDS holds the same swizzled 16-bit tiles as without KV8 and both
 // contractions run unchanged; k_scale folds into the softmax scale, v_scale into the final 1 / l.
-template <typename T, int D, int NG, bool SHARE, bool KV8 = false>
+// FINALN: the variant for a rank's last ring step (epilogue SPA_EPI_FINALN); the others write a
+// block result as it is (SPA_EPI_PLAIN / SPA_EPI_PART).
+template <typename T, int D, int NG, bool SHARE, bool KV8 = false, bool FINALN = false>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams pk) {
   static_assert(!(KV8 && SHARE), "e4m3 K/V tiles are staged through registers per wave group");
+  static_assert(!(FINALN && SHARE), "the merging epilogue goes with 128-row workgroups");
   typedef typename std::conditional<KV8, unsigned char, T>::type KVT;  // element type of K / V in memory
   typedef Fwd16Cfg<D, NG, SHARE> C;
   FwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
@@ -599,17 +602,36 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // exp2((m - m_all) c) / l_all and stages it as fp32 rows in LDS (free now); then all
   // waves walk the 128 x D tile row-major, add the groups' partials and write full rows:
   // 16-byte coalesced stores instead of 8-byte pieces scattered over 32 rows per wave.
-  // A ring step's merge with the running (acc, lse) happens in the same pass (p.epi).
-  if (SHARE && p.epi == SPA_EPI_PLAIN) {
+  // A rank's last ring step merges the earlier steps' results in the same pass (p.epi).
+  // Where the block result goes: the caller's out / lse (rows of this rank), or, for a ring step
+  // that is not the rank's last, the step's slot (in q's element type, as the reference keeps a
+  // block's output: sp_aurora/intel_ring_flash_attn.py:96-108).
+  // The fields only this epilogue needs are read from the kernel-argument segment HERE (the pointer
+  // passes through an empty asm): read through `p`, they are fetched before the loop and held in
+  // scalar registers across it, which the loop has none to spare for.
+  typedef const __attribute__((address_space(4))) FwdParams* LateParams;
+  LateParams late = (LateParams)__builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(late));
+  void* const part = late->part;
+  const int part_slot = late->part_slot, npart = late->npart;
+  const bool to_slot = late->epi == SPA_EPI_PART;
+  const RingSlots slots(p.B, p.H, p.Sq, D);
+  const int64_t slot_rs = (int64_t)p.H * D;                          // a slot is contiguous [B, Sq, H, D]
+  const int64_t slot_bh = (int64_t)b * p.Sq * slot_rs + h * D;
+  T* const out_bh = to_slot ? slots.template out<T>(part, part_slot) + slot_bh
+                            : (T*)p.out + b * p.os.b + h * p.os.h + qoff * p.os.s;
+  const int64_t out_rs = to_slot ? slot_rs : p.os.s;
+  float* const lse_bh = to_slot ? slots.lse(part, p.P, part_slot) + ((int64_t)b * p.H + h) * p.Sq
+                                : p.lse + ((int64_t)b * p.H + h) * p.lse_bh + qoff;
+  if constexpr (SHARE) {
     // A wave's rows are complete and nothing is merged: straight from the registers.  A lane holds
     // 4 consecutive head dims per register group and its partner 32 lanes on the next 4; one
     // v_permlane32_swap per dword pairs them up so that every lane stores 16-byte pieces, the two
     // lanes of a row side by side.  No LDS round trip, no barrier.
     const float l_tot = halves_sum(l_run);
-    const float inv = 1.f / l_tot;
-    if (hh == 0 && qrow < p.Sq)
-      p.lse[((int64_t)b * p.H + h) * p.lse_bh + qoff + qrow] = (m_run * c + fast_log2(l_tot)) * 0.6931471805599453f;
-    T* const orow = (T*)p.out + b * p.os.b + h * p.os.h + (qoff + qrow_c) * p.os.s;
+    const float inv = vsc / l_tot;
+    if (hh == 0 && qrow < p.Sq) lse_bh[qrow] = (m_run * c + fast_log2(l_tot)) * 0.6931471805599453f;
+    T* const orow = out_bh + qrow_c * out_rs;
 #pragma unroll
     for (int db = 0; db < D / 32; ++db)
 #pragma unroll
@@ -630,135 +652,156 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         if (qrow < p.Sq) *(u32x4*)(orow + db * 32 + 8 * (2 * gp + hh)) = st;
       }
     return;
-  }
-  constexpr int TP = D + 4;  // floats per staged row
-  float* const tile = (float*)smem + grp * (FWD_BM * TP);
-  float* const ml = (float*)smem + NG * FWD_BM * TP;  // [NG][128](m, l), then lse_b[rows of the workgroup]
-  float* const lsb = ml + NG * FWD_BM * 2;
-  const int rloc = w * 32 + ln;
-  // The final pass walks the tile row-major, a thread owning 8 head dims of NIT rows; the CH lanes of
-  // a row share a wave.  A merging step fetches its pieces of the running (acc, lse) NOW, so that
-  // their latency passes under the exchange and the staging below instead of after them.
-  constexpr int CH = D / 8;                                   // 8-element chunks per row
-  constexpr int NIT = C::BMW * CH / (FWD_THREADS * NG);       // chunks per thread
-  constexpr int NPRE = NIT < 4 ? NIT : 4;                     // of which fetched before the staging
-  static_assert(NIT * FWD_THREADS * NG == C::BMW * CH, "the final pass must tile the workgroup's rows");
-  const int epi = p.epi;
-  const bool merging = epi >= SPA_EPI_MERGE;
-  f32x4 pa[NIT][2];
-  float pl[NIT];
-  auto acc_ptr = [&](int it, int& grow, int& ch) -> float* {
-    const int cidx = tid + it * (FWD_THREADS * NG);
-    const int row = cidx / CH;
-    ch = cidx % CH;
-    grow = q0 + row;
-    return p.acc + b * p.as.b + h * p.as.h + (int64_t)grow * p.as.s + ch * 8;
-  };
-  auto fetch_acc = [&](int it) {
-    int grow, ch;
-    const float* ap = acc_ptr(it, grow, ch);
-    if (merging && grow < p.Sq) {
-      pa[it][0] = *(const f32x4*)ap;
-      pa[it][1] = *(const f32x4*)(ap + 4);
-      pl[it] = p.lse[((int64_t)b * p.H + h) * p.lse_bh + qoff + grow];
-    }
-  };
-#pragma unroll
-  for (int it = 0; it < NPRE; ++it) fetch_acc(it);
-  const float l_own = halves_sum(l_run);
-  float scale, lse_b;
-  if (NG > 1 && !SHARE) {
-    if (hh == 0) {
-      ml[(grp * FWD_BM + rloc) * 2] = m_run;
-      ml[(grp * FWD_BM + rloc) * 2 + 1] = l_own;
-    }
-    __syncthreads();
-    const float m2 = ml[((grp ^ 1) * FWD_BM + rloc) * 2];
-    const float l2 = ml[((grp ^ 1) * FWD_BM + rloc) * 2 + 1];
-    const float m_all = fmaxf(m_run, m2);  // finite: some group has seen key 0 of the first chunk
-    const float a1 = fast_exp2((m_run - m_all) * c);
-    const float a2 = fast_exp2((m2 - m_all) * c);
-    const float l_all = l_own * a1 + l2 * a2;
-    scale = a1 * vsc / l_all;
-    lse_b = (m_all * c + fast_log2(l_all)) * 0.6931471805599453f;
   } else {
-    scale = vsc / l_own;
-    lse_b = (m_run * c + fast_log2(l_own)) * 0.6931471805599453f;
-  }
-#pragma unroll
-  for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      f32x4 st;
-      st[0] = o[db][4 * g + 0] * scale;
-      st[1] = o[db][4 * g + 1] * scale;
-      st[2] = o[db][4 * g + 2] * scale;
-      st[3] = o[db][4 * g + 3] * scale;
-      *(f32x4*)(tile + rloc * TP + db * 32 + 8 * g + 4 * hh) = st;
-    }
-  if ((SHARE || grp == 0) && hh == 0) lsb[(SHARE ? grp * FWD_BM : 0) + rloc] = lse_b;
-  __syncthreads();
-#pragma unroll
-  for (int it = NPRE; it < NIT; ++it) fetch_acc(it);  // the accumulators are staged: registers are free for the rest
-  {
-    const float* t0 = (const float*)smem;
+    constexpr int TP = D + 4;  // floats per staged row
+    float* const tile = (float*)smem + grp * (FWD_BM * TP);
+    float* const ml = (float*)smem + NG * FWD_BM * TP;  // [NG][128](m, l), then lse_b[rows of the workgroup]
+    float* const lsb = ml + NG * FWD_BM * 2;
+    const int rloc = w * 32 + ln;
+    // The final pass walks the tile row-major, a thread owning 8 head dims of NIT rows; the CH lanes of
+    // a row share a wave.
+    constexpr int CH = D / 8;                                   // 8-element chunks per row
+    constexpr int NIT = C::BMW * CH / (FWD_THREADS * NG);       // chunks per thread
+    static_assert(NIT * FWD_THREADS * NG == C::BMW * CH, "the final pass must tile the workgroup's rows");
+    int crow[NIT], cch[NIT];
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
-      int grow, ch;
-      float* ap = acc_ptr(it, grow, ch);
-      const int row = grow - q0;
-      if (grow >= p.Sq) continue;
-      float x[8];
-      {
-        const f32x4 a = *(const f32x4*)(t0 + row * TP + ch * 8);
-        const f32x4 bq = *(const f32x4*)(t0 + row * TP + ch * 8 + 4);
-        x[0] = a[0]; x[1] = a[1]; x[2] = a[2]; x[3] = a[3];
-        x[4] = bq[0]; x[5] = bq[1]; x[6] = bq[2]; x[7] = bq[3];
-      }
-      if (NG > 1 && !SHARE) {
-        const float* t1 = t0 + FWD_BM * TP;
-        const f32x4 a = *(const f32x4*)(t1 + row * TP + ch * 8);
-        const f32x4 bq = *(const f32x4*)(t1 + row * TP + ch * 8 + 4);
-        x[0] += a[0]; x[1] += a[1]; x[2] += a[2]; x[3] += a[3];
-        x[4] += bq[0]; x[5] += bq[1]; x[6] += bq[2]; x[7] += bq[3];
-      }
-      float lb = lsb[row];
-      const int64_t li = ((int64_t)b * p.H + h) * p.lse_bh + qoff + grow;
-      if (merging) {  // merge with the running accumulators (sp_aurora/utils.py:103-104)
-        const float la = pl[it];
-        const f32x4 a = pa[it][0];
-        const f32x4 bq = pa[it][1];
-        const float xa[8] = {a[0], a[1], a[2], a[3], bq[0], bq[1], bq[2], bq[3]};
-        const float d = lb - la;
-        float wgt, ln_;
-        if (d == d) {
-          const float e = __expf(-fabsf(d));
-          const float inv = 1.f / (1.f + e);
-          wgt = d >= 0.f ? inv : e * inv;  // sigmoid(lb - la)
-          ln_ = fmaxf(la, lb) + log1pf(e);
-        } else {
-          wgt = 0.f;
-          ln_ = la;
-        }
+      const int cidx = tid + it * (FWD_THREADS * NG);
+      crow[it] = cidx / CH;
+      cch[it] = cidx % CH;
+    }
+    // The rank's last step fetches the first slots NOW, so that their latency passes under the
+    // exchange and the staging below; NB slots are in flight at a time.
+    constexpr int NB = 2;
+    u32x4 raw[NB][NIT];
+    float rl[NB][NIT];
+    auto fetch_slots = [&](int j0) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = xa[e] - wgt * (xa[e] - x[e]);
-        lb = ln_;
+      for (int jj = 0; jj < NB; ++jj)
+        if (j0 + jj < npart) {
+          const T* so = slots.template out<T>(part, j0 + jj) + slot_bh;
+          const float* sl = slots.lse(part, p.P, j0 + jj) + ((int64_t)b * p.H + h) * p.Sq;
+#pragma unroll
+          for (int it = 0; it < NIT; ++it) {
+            const int grow = q0 + crow[it];
+            if (grow < p.Sq) {
+              raw[jj][it] = *(const u32x4*)(so + (int64_t)grow * slot_rs + cch[it] * 8);
+              rl[jj][it] = sl[grow];
+            }
+          }
+        }
+    };
+    if constexpr (FINALN) fetch_slots(0);
+    const float l_own = halves_sum(l_run);
+    float scale, lse_b;
+    if (NG > 1) {
+      if (hh == 0) {
+        ml[(grp * FWD_BM + rloc) * 2] = m_run;
+        ml[(grp * FWD_BM + rloc) * 2 + 1] = l_own;
       }
-      if (epi == SPA_EPI_INIT || epi == SPA_EPI_MERGE) {
-        f32x4 a, bq;
-        a[0] = x[0]; a[1] = x[1]; a[2] = x[2]; a[3] = x[3];
-        bq[0] = x[4]; bq[1] = x[5]; bq[2] = x[6]; bq[3] = x[7];
-        *(f32x4*)ap = a;
-        *(f32x4*)(ap + 4) = bq;
-      } else {
-        u32x4 st;
-        st[0] = M::pack2(x[0], x[1]);
-        st[1] = M::pack2(x[2], x[3]);
-        st[2] = M::pack2(x[4], x[5]);
-        st[3] = M::pack2(x[6], x[7]);
-        *(u32x4*)((T*)p.out + b * p.os.b + h * p.os.h + (qoff + grow) * p.os.s + ch * 8) = st;
+      __syncthreads();
+      const float m2 = ml[((grp ^ 1) * FWD_BM + rloc) * 2];
+      const float l2 = ml[((grp ^ 1) * FWD_BM + rloc) * 2 + 1];
+      const float m_all = fmaxf(m_run, m2);  // finite: some group has seen key 0 of the first chunk
+      const float a1 = fast_exp2((m_run - m_all) * c);
+      const float a2 = fast_exp2((m2 - m_all) * c);
+      const float l_all = l_own * a1 + l2 * a2;
+      scale = a1 * vsc / l_all;
+      lse_b = (m_all * c + fast_log2(l_all)) * 0.6931471805599453f;
+    } else {
+      scale = vsc / l_own;
+      lse_b = (m_run * c + fast_log2(l_own)) * 0.6931471805599453f;
+    }
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 st;
+        st[0] = o[db][4 * g + 0] * scale;
+        st[1] = o[db][4 * g + 1] * scale;
+        st[2] = o[db][4 * g + 2] * scale;
+        st[3] = o[db][4 * g + 3] * scale;
+        *(f32x4*)(tile + rloc * TP + db * 32 + 8 * g + 4 * hh) = st;
       }
-      if (ch == 0) p.lse[li] = lb;
+    if (grp == 0 && hh == 0) lsb[rloc] = lse_b;
+    __syncthreads();
+    const float* t0 = (const float*)smem;
+    float x[NIT][8], lb[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int row = crow[it], ch = cch[it];
+      const f32x4 a = *(const f32x4*)(t0 + row * TP + ch * 8);
+      const f32x4 bq = *(const f32x4*)(t0 + row * TP + ch * 8 + 4);
+      x[it][0] = a[0]; x[it][1] = a[1]; x[it][2] = a[2]; x[it][3] = a[3];
+      x[it][4] = bq[0]; x[it][5] = bq[1]; x[it][6] = bq[2]; x[it][7] = bq[3];
+      if (NG > 1) {
+        const float* t1 = t0 + FWD_BM * TP;
+        const f32x4 a2 = *(const f32x4*)(t1 + row * TP + ch * 8);
+        const f32x4 b2 = *(const f32x4*)(t1 + row * TP + ch * 8 + 4);
+        x[it][0] += a2[0]; x[it][1] += a2[1]; x[it][2] += a2[2]; x[it][3] += a2[3];
+        x[it][4] += b2[0]; x[it][5] += b2[1]; x[it][6] += b2[2]; x[it][7] += b2[3];
+      }
+      lb[it] = lsb[row];
+    }
+    if constexpr (FINALN) {
+      // update_out_and_lse over all of the rank's steps at once (sp_aurora/utils.py:103-104 applied
+      // npart times): out = sum_j e^(lse_j - L) out_j, L = log sum_j e^(lse_j), carried as a running
+      // (weighted sum, weight sum) relative to the largest lse so far, starting from this step's block.
+      constexpr float LOG2E = 1.4426950408889634f;
+      float wsum[NIT];
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) wsum[it] = 1.f;
+      for (int j0 = 0; j0 < npart; j0 += NB) {
+        u32x4 cur[NB][NIT];
+        float cul[NB][NIT];
+#pragma unroll
+        for (int jj = 0; jj < NB; ++jj)
+#pragma unroll
+          for (int it = 0; it < NIT; ++it) {
+            cur[jj][it] = raw[jj][it];
+            cul[jj][it] = rl[jj][it];
+          }
+        fetch_slots(j0 + NB);
+#pragma unroll
+        for (int jj = 0; jj < NB; ++jj)
+          if (j0 + jj < npart) {
+#pragma unroll
+            for (int it = 0; it < NIT; ++it) {
+              const float lj = cul[jj][it];
+              const float mx = fmaxf(lb[it], lj);  // lb is finite: the last step's block hides no key of a row
+              const float wa = fast_exp2((lb[it] - mx) * LOG2E);
+              const float wb = fast_exp2((lj - mx) * LOG2E);
+              wsum[it] = wsum[it] * wa + wb;
+              lb[it] = mx;
+#pragma unroll
+              for (int k = 0; k < 4; ++k) {
+                float lo, hi;
+                M::unpack2(cur[jj][it][k], lo, hi);
+                x[it][2 * k] = x[it][2 * k] * wa + lo * wb;
+                x[it][2 * k + 1] = x[it][2 * k + 1] * wa + hi * wb;
+              }
+            }
+          }
+      }
+#pragma unroll
+      for (int it = 0; it < NIT; ++it) {
+        const float inv = 1.f / wsum[it];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) x[it][k] *= inv;
+        lb[it] += fast_log2(wsum[it]) * 0.6931471805599453f;
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      const int grow = q0 + crow[it];
+      if (grow >= p.Sq) continue;
+      u32x4 st;
+      st[0] = M::pack2(x[it][0], x[it][1]);
+      st[1] = M::pack2(x[it][2], x[it][3]);
+      st[2] = M::pack2(x[it][4], x[it][5]);
+      st[3] = M::pack2(x[it][6], x[it][7]);
+      *(u32x4*)(out_bh + (int64_t)grow * out_rs + cch[it] * 8) = st;
+      if (cch[it] == 0) lse_bh[grow] = lb[it];
     }
   }
 }
@@ -994,6 +1037,10 @@ hipError_t launch16(FwdParams p, hipStream_t stream) {
   const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
   const int force_share = spa_knob(SPA_KNOB_FWD_SHARE);
   const bool two = force ? force == 2 : p.Sk > fwd_bn<D>();
+  if (p.epi == SPA_EPI_FINALN) {
+    if (two) return launch<flash_fwd16_kernel<T, D, 2, false, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+    return launch<flash_fwd16_kernel<T, D, 1, false, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+  }
   if (two && D >= 64) {
     const int nqt2 = (p.Sq + 2 * FWD_BM - 1) / (2 * FWD_BM);
     const int64_t wgs = (int64_t)p.B * p.H * nqt2 * p.nranks;
@@ -1012,6 +1059,10 @@ template <typename T, int D>
 hipError_t launch16_kv8(FwdParams p, hipStream_t stream) {
   const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
   const bool two = force ? force == 2 : p.Sk > fwd_bn<D>();
+  if (p.epi == SPA_EPI_FINALN) {
+    if (two) return launch<flash_fwd16_kernel<T, D, 2, false, true, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+    return launch<flash_fwd16_kernel<T, D, 1, false, true, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+  }
   if (two) return launch<flash_fwd16_kernel<T, D, 2, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
   return launch<flash_fwd16_kernel<T, D, 1, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
 }

@@ -147,8 +147,7 @@ int flash_fwd(const char* what, const void* q, const void* k, const void* v, con
   p.causal = mask_mode == SPA_MASK_CAUSAL;
   p.nqt = 0;
   p.lse_bh = Sq;
-  p.acc = nullptr;
-  p.as = S3(o_strides);
+  p.part = nullptr; p.part_slot = 0; p.npart = 0;
   p.epi = SPA_EPI_PLAIN;
   p.P = 1; p.rank0 = 0; p.nranks = 1; p.t_begin = 0; p.t_count = -1;
   p.cu_q = nullptr; p.cu_k = nullptr;
@@ -197,7 +196,8 @@ int64_t spa_ring_fwd_workspace_bytes(int B, int H, int S, int D, int P, int dtyp
   if (B <= 0 || H <= 0 || S <= 0 || D <= 0 || P <= 0 || S % P != 0 || !dtype_ok(dtype)) return -1;
   const int64_t s = S / P;
   const int64_t acc = (int64_t)B * s * H * D * 4;
-  if (dtype != SPA_F32) return acc;
+  // 16-bit: one slot per step but a rank's last: the block's output in q's type and its lse
+  if (dtype != SPA_F32) return RingSlots(B, H, s, D).total(P);
   // fp32: running output, one block's output, one block's lse
   return 2 * acc + (int64_t)B * H * s * 4;
 }
@@ -263,8 +263,8 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   if ((int64_t)B * H > 0x7fffffffLL || (s + 127) / 128 > 65535 || r_hi - r_lo > 65535) return fail(SPA_EINVAL, "%s: grid too large", what);
   hipStream_t st = (hipStream_t)stream;
 
-  // workspace carve-up; the running output of one rank is laid out [B, s, H, D]
-  float* acc = (float*)workspace;
+  // workspace carve-up; one rank's block output (or, fp32, its running output) is laid out [B, s, H, D]
+  float* acc = (float*)workspace;        // fp32 path only
   const int64_t acc_elems = (int64_t)B * s * H * D;
   Strides3 as;
   as.b = (int64_t)s * H * D; as.h = D; as.s = (int64_t)H * D;
@@ -281,8 +281,8 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   p.causal = causal;
   p.nqt = 0;
   p.lse_bh = S;
-  p.acc = acc;
-  p.as = as;
+  p.part = workspace;  // 16-bit path: the steps' slots (RingSlots)
+  p.part_slot = 0; p.npart = 0;
   p.P = P;
   p.epi = SPA_EPI_PLAIN;
   p.cu_q = nullptr; p.cu_k = nullptr;
@@ -305,7 +305,10 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
       hipError_t e;
       if (dtype != SPA_F32) {
         p.t_begin = t; p.t_count = 1;
-        p.epi = nsteps == 1 ? SPA_EPI_PLAIN : t == 0 ? SPA_EPI_INIT : t + 1 == nsteps ? SPA_EPI_FINAL : SPA_EPI_MERGE;
+        // every step but the last leaves its block in slot t; the last merges them in ring order and adds its own
+        p.epi = nsteps == 1 ? SPA_EPI_PLAIN : t + 1 == nsteps ? SPA_EPI_FINALN : SPA_EPI_PART;
+        p.part_slot = t;
+        p.npart = nsteps - 1;
         e = spa_launch_flash_fwd(p, D, dtype, st);
       } else {
         // fp32: one plain block pair per launch on explicit chunk pointers, merged by the stand-alone kernels
@@ -536,8 +539,7 @@ int flash_fwd_varlen(const char* what, const void* q, const void* k, const void*
   p.causal = mask_mode == SPA_MASK_CAUSAL;
   p.nqt = 0;
   p.lse_bh = total_q;
-  p.acc = nullptr;
-  p.as = S2(o_strides);
+  p.part = nullptr; p.part_slot = 0; p.npart = 0;
   p.epi = SPA_EPI_PLAIN;
   p.P = 1; p.rank0 = 0; p.nranks = 1; p.t_begin = 0; p.t_count = -1;
   p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;

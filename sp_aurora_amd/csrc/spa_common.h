@@ -33,9 +33,12 @@ struct FwdParams {
   // rows; the launch runs ranks rank0 .. rank0+nranks-1, each over steps [t_begin, t_begin+t_count)
   // of its schedule (t_count < 0: to the end).  A plain block call is P = 1, rank 0, all steps.
   int P, rank0, nranks, t_begin, t_count;
-  // ring-step epilogue (16-bit kernels): what happens to the block result
-  float* acc;        // fp32 running output, [B,H,Sq,D] by `as` (SPA_EPI_INIT/MERGE/FINAL)
-  Strides3 as;
+  // ring-step epilogue (16-bit kernels): what happens to the block result.  The results of a
+  // rank's earlier steps wait in slots at `part` (see RingSlots): slot j holds step j's block
+  // output in q's element type, contiguous [B,Sq,H,D], and its lse, [B*H,Sq] fp32.
+  void* part;
+  int part_slot;     // SPA_EPI_PART: the slot this step fills
+  int npart;         // SPA_EPI_FINALN: slots 0 .. npart-1 are merged, in that order, then this step's block
   int epi;
   // variable-length batch (null: every sequence has Sq queries and Sk keys): sequence b owns rows
   // cu_q[b] .. cu_q[b+1] of q/out/lse and cu_k[b] .. cu_k[b+1] of k/v, batch strides are unused,
@@ -48,11 +51,24 @@ struct FwdParams {
   const float* v_scale;
 };
 
+// Layout of the ring-step slots of one rank in the caller's workspace (16-bit inputs, ring of P):
+// P - 1 output slots of out_bytes each, then P - 1 lse slots of lse_bytes each; host and kernels
+// derive it from the sizes, so that it costs the kernels no arguments.
+struct RingSlots {
+  int64_t out_bytes, lse_bytes;
+  __host__ __device__ RingSlots(int B, int H, int64_t s, int D)
+      : out_bytes(((int64_t)B * s * H * D * 2 + 255) / 256 * 256), lse_bytes(((int64_t)B * H * s * 4 + 255) / 256 * 256) {}
+  __host__ __device__ int64_t total(int P) const { return (int64_t)(P - 1) * (out_bytes + lse_bytes); }
+  template <typename T>
+  __device__ T* out(void* part, int j) const { return (T*)((char*)part + j * out_bytes); }
+  __device__ float* lse(void* part, int P, int j) const { return (float*)((char*)part + (P - 1) * out_bytes + j * lse_bytes); }
+};
+
 enum {
-  SPA_EPI_PLAIN = 0,  // out <- block, lse <- block lse
-  SPA_EPI_INIT = 1,   // acc <- block (fp32), lse <- block lse            (first of several steps)
-  SPA_EPI_MERGE = 2,  // (acc, lse) <- merge((acc, lse), block)            (middle step)
-  SPA_EPI_FINAL = 3   // out <- cast(merge((acc, lse), block)), lse <- merged lse (last step)
+  SPA_EPI_PLAIN = 0,   // out <- block, lse <- block lse
+  SPA_EPI_PART = 1,    // slot part_slot <- (block rounded to q's type, block lse): a step that is not the rank's last
+  SPA_EPI_FINALN = 2   // (out, lse) <- the slots merged one after the other (fp32, sp_aurora/utils.py:103-104), then
+                       // this step's block: the rank's last step
 };
 
 struct BwdParams {
@@ -102,6 +118,10 @@ struct Mma16<__bf16> {
     r[0] = (__bf16)lo; r[1] = (__bf16)hi;
     return __builtin_bit_cast(unsigned, r);
   }
+  static __device__ __forceinline__ void unpack2(unsigned x, float& lo, float& hi) {
+    lo = __builtin_bit_cast(float, x << 16);
+    hi = __builtin_bit_cast(float, x & 0xffff0000u);
+  }
 };
 
 template <>
@@ -122,6 +142,12 @@ struct Mma16<_Float16> {
     f16x2 r;
     r[0] = (_Float16)lo; r[1] = (_Float16)hi;
     return __builtin_bit_cast(unsigned, r);
+  }
+  static __device__ __forceinline__ void unpack2(unsigned x, float& lo, float& hi) {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    const f16x2 r = __builtin_bit_cast(f16x2, x);
+    lo = (float)r[0];
+    hi = (float)r[1];
   }
 };
 

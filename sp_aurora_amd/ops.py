@@ -183,7 +183,7 @@ def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layo
     Returns (out like q, lse fp32 [B,H,S]); with rank >= 0 only that rank's rows are written.
     k, v may be torch.float8_e4m3fn with k_scale, v_scale fp32 [B,H] (spa_ring_fwd_fp8kv).
     static_scratch=True calls spa_ring_fwd_static instead: no workspace tensor, the library's built-in
-    32 MiB buffer holds the running output between step launches (for callers that must not allocate;
+    32 MiB buffer holds a rank's earlier block results between step launches (for callers that must not allocate;
     calls that overlap on one device race)."""
     lib = _lib.load()
     fp8 = k.dtype == FP8 or v.dtype == FP8

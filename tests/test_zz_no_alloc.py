@@ -1,7 +1,7 @@
 """spa_ring_fwd_static — the ring forward for callers that cannot allocate — against spa_ring_fwd.
 
-Both entry points run the same kernels; the only difference is where the fp32 running output of a
-rank lives between step launches (the caller's workspace / the library's built-in buffer).  The
+Both entry points run the same kernels; the only difference is where the earlier block results of a
+rank live between step launches (the caller's workspace / the library's built-in buffer).  The
 results must therefore be bit-identical, on two calls in a row, the second one smaller (the buffer
 keeps the first call's contents).  Called through the C ABI directly.
 """
@@ -71,7 +71,7 @@ def test_static_scratch_matches_caller_workspace_twice_in_a_row(dtype):
 
 def test_static_scratch_rejects_sizes_beyond_the_buffer():
     lib = _lib.load()
-    B, S, H, D, P = 1, 8192, 64, 128, 2   # one rank's fp32 running output: 128 MiB
+    B, S, H, D, P = 1, 8192, 64, 128, 2   # one block output of a rank: 64 MiB
     assert lib.spa_ring_fwd_workspace_bytes(B, H, S, D, P, _lib.SPA_BF16) > lib.spa_static_scratch_bytes()
     x = torch.empty((16,), dtype=torch.bfloat16, device=DEV)   # never dereferenced: the size check comes first
     st = _lib.strides3((S * H * D, D, H * D))
