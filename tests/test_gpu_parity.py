@@ -529,9 +529,11 @@ def test_ring_driver_matches_stepwise_path_and_oracle(causal, dtype):
 
 @pytest.mark.parametrize("fuse", ["step", "rank", "all"])
 @pytest.mark.parametrize("P,B,s,H,D,causal", [(8, 1, 128, 2, 128, True), (3, 2, 200, 2, 64, True), (4, 1, 72, 3, 32, False),
-                                              (2, 1, 1024, 2, 128, True), (5, 1, 64, 1, 128, True)])
+                                              (2, 1, 1024, 2, 128, True), (5, 1, 64, 1, 128, True),
+                                              (16, 1, 40, 2, 64, False), (12, 2, 136, 1, 128, True)])
 def test_ring_driver_modes_on_awkward_shapes(P, B, s, H, D, causal, fuse):
-    """Chunk lengths that are not multiples of the key tile, odd ring sizes, many ranks."""
+    """Chunk lengths that are not multiples of the key tile, odd ring sizes, many ranks (in the per-step
+    schedule a rank's last step then merges up to 15 earlier results)."""
     q, k, v = rand_qkv((B, P * s, H, D), 111, torch.bfloat16)
     want_out, want_lse = O.full_attention(q, k, v, None, causal)
     out, lse = ops.ring_fwd(q.to(DEV), k.to(DEV), v.to(DEV), P, None, causal, fuse=fuse)
