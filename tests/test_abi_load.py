@@ -34,6 +34,20 @@ def test_abi_version_and_error_string():
     assert isinstance(lib.spa_last_error(), bytes)
 
 
+def test_ring_workspace_sizes():
+    """16-bit inputs: one slot per step but a rank's last (a block output in q's type and its fp32 lse, each a
+    multiple of 256 bytes); fp32: the running output, one block's output and its lse."""
+    lib = _lib.load()
+    up = lambda n: (n + 255) // 256 * 256
+    for B, H, S, D, P in [(1, 32, 8192, 128, 8), (2, 3, 600, 64, 3), (1, 1, 64, 32, 1), (2, 16, 32768, 128, 16)]:
+        s = S // P
+        for dt in (_lib.SPA_BF16, _lib.SPA_F16):
+            assert lib.spa_ring_fwd_workspace_bytes(B, H, S, D, P, dt) == (P - 1) * (up(B * s * H * D * 2) + up(B * H * s * 4))
+        assert lib.spa_ring_fwd_workspace_bytes(B, H, S, D, P, _lib.SPA_F32) == 2 * B * s * H * D * 4 + B * H * s * 4
+    assert lib.spa_ring_fwd_workspace_bytes(1, 1, 100, 64, 3, _lib.SPA_BF16) == -1   # the ring must divide the sequence
+    assert lib.spa_ring_fwd_workspace_bytes(1, 1, 64, 64, 2, 7) == -1                 # no such dtype
+
+
 def _s3(*v):
     return _lib.strides3(v)
 
