@@ -608,7 +608,8 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // block's output: sp_aurora/intel_ring_flash_attn.py:96-108).
   // The fields only this epilogue needs are read from the kernel-argument segment HERE (the pointer
   // passes through an empty asm): read through `p`, they are fetched before the loop and held in
-  // scalar registers across it, which the loop has none to spare for.
+  // scalar registers across it, which the loop has none to spare for.  (FwdParams is the kernel's
+  // only argument, so the segment begins with it.)
   typedef const __attribute__((address_space(4))) FwdParams* LateParams;
   LateParams late = (LateParams)__builtin_amdgcn_kernarg_segment_ptr();
   asm volatile("" : "+s"(late));
