@@ -602,28 +602,13 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // exp2((m - m_all) c) / l_all and stages it as fp32 rows in LDS (free now); then all
   // waves walk the 128 x D tile row-major, add the groups' partials and write full rows:
   // 16-byte coalesced stores instead of 8-byte pieces scattered over 32 rows per wave.
-  // A rank's last ring step merges the earlier steps' results in the same pass (p.epi).
-  // Where the block result goes: the caller's out / lse (rows of this rank), or, for a ring step
-  // that is not the rank's last, the step's slot (in q's element type, as the reference keeps a
-  // block's output: sp_aurora/intel_ring_flash_attn.py:96-108).
-  // The fields only this epilogue needs are read from the kernel-argument segment HERE (the pointer
-  // passes through an empty asm): read through `p`, they are fetched before the loop and held in
-  // scalar registers across it, which the loop has none to spare for.  (FwdParams is the kernel's
-  // only argument, so the segment begins with it.)
-  typedef const __attribute__((address_space(4))) FwdParams* LateParams;
-  LateParams late = (LateParams)__builtin_amdgcn_kernarg_segment_ptr();
-  asm volatile("" : "+s"(late));
-  void* const part = late->part;
-  const int part_slot = late->part_slot, npart = late->npart;
-  const bool to_slot = late->epi == SPA_EPI_PART;
-  const RingSlots slots(p.B, p.H, p.Sq, D);
-  const int64_t slot_rs = (int64_t)p.H * D;                          // a slot is contiguous [B, Sq, H, D]
-  const int64_t slot_bh = (int64_t)b * p.Sq * slot_rs + h * D;
-  T* const out_bh = to_slot ? slots.template out<T>(part, part_slot) + slot_bh
-                            : (T*)p.out + b * p.os.b + h * p.os.h + qoff * p.os.s;
-  const int64_t out_rs = to_slot ? slot_rs : p.os.s;
-  float* const lse_bh = to_slot ? slots.lse(part, p.P, part_slot) + ((int64_t)b * p.H + h) * p.Sq
-                                : p.lse + ((int64_t)b * p.H + h) * p.lse_bh + qoff;
+  // A rank's last ring step (the FINALN variants) merges the earlier steps' results, which lie in the
+  // slots of p.part, in the same pass.  A step that is not the rank's last needs nothing of its own:
+  // the host points out / lse and their strides at the step's slot (in q's element type, as the
+  // reference keeps a block's output: sp_aurora/intel_ring_flash_attn.py:96-108).
+  T* const out_bh = (T*)p.out + b * p.os.b + h * p.os.h + qoff * p.os.s;
+  const int64_t out_rs = p.os.s;
+  float* const lse_bh = p.lse + ((int64_t)b * p.H + h) * p.lse_bh + qoff;
   if constexpr (SHARE) {
     // A wave's rows are complete and nothing is merged: straight from the registers.  A lane holds
     // 4 consecutive head dims per register group and its partner 32 lanes on the next 4; one
@@ -674,6 +659,11 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     // The rank's last step fetches the first slots NOW, so that their latency passes under the
     // exchange and the staging below; NB slots are in flight at a time.
     constexpr int NB = 2;
+    void* const part = FINALN ? p.part : nullptr;
+    const int npart = FINALN ? p.npart : 0;
+    const RingSlots slots(p.B, p.H, p.Sq, D);
+    const int64_t slot_rs = (int64_t)p.H * D;  // a slot is contiguous [B, Sq, H, D]
+    const int64_t slot_bh = (int64_t)b * p.Sq * slot_rs + h * D;
     u32x4 raw[NB][NIT];
     float rl[NB][NIT];
     auto fetch_slots = [&](int j0) {
@@ -1073,6 +1063,18 @@ hipError_t launch16_kv8(FwdParams p, hipStream_t stream) {
 // Returns hipSuccess, or hipErrorInvalidValue for an unsupported (dtype, D).
 hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream) {
   p.nqt = (p.Sq + FWD_BM - 1) / FWD_BM;
+  if (p.epi == SPA_EPI_PART) {
+    // A ring step that is not the rank's last: the kernel writes the block as it would write any
+    // result, and out / lse are pointed at the step's slot here.  The kernel adds the rank's row
+    // offset (rank0 * Sq rows) to both, so the slot's addresses go in with that offset taken off.
+    if (dtype == 0 || p.nranks != 1 || !p.part) return hipErrorInvalidValue;
+    const RingSlots slots(p.B, p.H, p.Sq, D);
+    p.os.b = (int64_t)p.Sq * p.H * D; p.os.s = (int64_t)p.H * D; p.os.h = D;
+    p.lse_bh = p.Sq;
+    const int64_t row0 = (int64_t)p.rank0 * p.Sq;
+    p.out = (char*)slots.out<char>(p.part, p.part_slot) - row0 * p.os.s * 2;
+    p.lse = slots.lse(p.part, p.P, p.part_slot) - row0;
+  }
   if (p.k_scale) {  // K / V are e4m3 bytes, q / out of type `dtype`
     if (!p.v_scale) return hipErrorInvalidValue;
     if (dtype == 1) {

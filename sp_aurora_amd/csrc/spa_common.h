@@ -36,8 +36,9 @@ struct FwdParams {
   // ring-step epilogue (16-bit kernels): what happens to the block result.  The results of a
   // rank's earlier steps wait in slots at `part` (see RingSlots): slot j holds step j's block
   // output in q's element type, contiguous [B,Sq,H,D], and its lse, [B*H,Sq] fp32.
+  // Only the kernels for a rank's last step read part and npart; part_slot and epi are for the host.
   void* part;
-  int part_slot;     // SPA_EPI_PART: the slot this step fills
+  int part_slot;     // SPA_EPI_PART: the slot this step fills (the launcher points out / lse at it)
   int npart;         // SPA_EPI_FINALN: slots 0 .. npart-1 are merged, in that order, then this step's block
   int epi;
   // variable-length batch (null: every sequence has Sq queries and Sk keys): sequence b owns rows
@@ -53,15 +54,15 @@ struct FwdParams {
 
 // Layout of the ring-step slots of one rank in the caller's workspace (16-bit inputs, ring of P):
 // P - 1 output slots of out_bytes each, then P - 1 lse slots of lse_bytes each; host and kernels
-// derive it from the sizes, so that it costs the kernels no arguments.
+// derive it from the sizes.
 struct RingSlots {
   int64_t out_bytes, lse_bytes;
   __host__ __device__ RingSlots(int B, int H, int64_t s, int D)
       : out_bytes(((int64_t)B * s * H * D * 2 + 255) / 256 * 256), lse_bytes(((int64_t)B * H * s * 4 + 255) / 256 * 256) {}
   __host__ __device__ int64_t total(int P) const { return (int64_t)(P - 1) * (out_bytes + lse_bytes); }
   template <typename T>
-  __device__ T* out(void* part, int j) const { return (T*)((char*)part + j * out_bytes); }
-  __device__ float* lse(void* part, int P, int j) const { return (float*)((char*)part + (P - 1) * out_bytes + j * lse_bytes); }
+  __host__ __device__ T* out(void* part, int j) const { return (T*)((char*)part + j * out_bytes); }
+  __host__ __device__ float* lse(void* part, int P, int j) const { return (float*)((char*)part + (P - 1) * out_bytes + j * lse_bytes); }
 };
 
 enum {
