@@ -87,11 +87,12 @@ __device__ __forceinline__ int v_swizzle(int row) {
 // global -> registers -> LDS and are widened to T on the way (every e4m3 value is exact in bf16 and
 // fp16), once per workgroup, so LDS holds the same swizzled 16-bit tiles as without KV8 and both
 // contractions run unchanged; k_scale folds into the softmax scale, v_scale into the final 1 / l.
+// (With shared buffers every thread of the workgroup stages its share of a tile and writes it before
+// the barrier at which the direct loads of the 16-bit form are waited for.)
 // FINALN: the variant for a rank's last ring step (epilogue SPA_EPI_FINALN); the others write a
 // block result as it is (SPA_EPI_PLAIN / SPA_EPI_PART).
 template <typename T, int D, int NG, bool SHARE, bool KV8 = false, bool FINALN = false>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams pk) {
-  static_assert(!(KV8 && SHARE), "e4m3 K/V tiles are staged through registers per wave group");
   static_assert(!(FINALN && SHARE), "the merging epilogue goes with 128-row workgroups");
   typedef typename std::conditional<KV8, unsigned char, T>::type KVT;  // element type of K / V in memory
   typedef Fwd16Cfg<D, NG, SHARE> C;
@@ -527,6 +528,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   __syncthreads();
   if (NG > 1 && grp == 1) {  // group 1 runs one phase behind group 0
     loads_landed();          // (with shared buffers group 0 reads this group's share of V(0), K(1) after this barrier)
+    if constexpr (SHARE) store_staged(k_lds(1), v_lds(0));
     __syncthreads();
   }
 
@@ -559,8 +561,10 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     // Shared buffers need one barrier per step and group (after the wait for the loads: group 0
     // at the end of its VALU phase, group 1 at the end of its MFMA phase, the same physical
     // barrier); the other one only holds the two groups in step, and they drift little without it.
-    if (!early) loads_landed();
-    store_staged((unsigned)((PAR ^ 1) * C::TILEB), (unsigned)(2 * C::TILEB + PAR * C::TILEB));  // K(i + 1), V(i)
+    if (!early) {
+      loads_landed();
+      store_staged((unsigned)((PAR ^ 1) * C::TILEB), (unsigned)(2 * C::TILEB + PAR * C::TILEB));  // K(i + 1), V(i)
+    }
     if (!SHARE || !early) __syncthreads();
     __builtin_amdgcn_s_setprio(3);
     mfma_phase(std::true_type{}, std::true_type{}, va, ka, pf, [&](int j) {
@@ -573,7 +577,10 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     cursor_next(cs);
     cursor_next(cv);
     cursor_next(ck);
-    if (early) loads_landed();
+    if (early) {
+      loads_landed();
+      store_staged(kb, vb);  // this group's share of K(i + 2), V(i + 1), loaded at the top of the step
+    }
     if (!SHARE || early) __syncthreads();
   };
   {
@@ -590,7 +597,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     unsigned va[D / 32], ka[D / 16];
     operand_addresses(n - 1, va, ka);
     loads_landed();
-    store_staged(k_lds(n), v_lds(n - 1));  // V(n - 1) (and whatever K(n) stands for: never read)
+    if (!early) store_staged(k_lds(n), v_lds(n - 1));  // V(n - 1) (and whatever K(n) stands for: never read)
     if (!SHARE || !early) __syncthreads();
     mfma_phase(std::true_type{}, std::false_type{}, va, ka, pf, [](int) {});
     if (!SHARE || early) __syncthreads();
@@ -1045,14 +1052,24 @@ hipError_t launch16(FwdParams p, hipStream_t stream) {
   return launch<flash_fwd16_kernel<T, D, 1, false>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
 }
 
-// e4m3 K/V: the register-staged variants (no shared-buffer form).
+// e4m3 K/V: the register-staged variants, chosen like the 16-bit ones.
 template <typename T, int D>
 hipError_t launch16_kv8(FwdParams p, hipStream_t stream) {
   const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
+  const int force_share = spa_knob(SPA_KNOB_FWD_SHARE);
   const bool two = force ? force == 2 : p.Sk > fwd_bn<D>();
   if (p.epi == SPA_EPI_FINALN) {
     if (two) return launch<flash_fwd16_kernel<T, D, 2, false, true, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
     return launch<flash_fwd16_kernel<T, D, 1, false, true, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+  }
+  if (two) {
+    const int nqt2 = (p.Sq + 2 * FWD_BM - 1) / (2 * FWD_BM);
+    const int64_t wgs = (int64_t)p.B * p.H * nqt2 * p.nranks;
+    const bool share = force_share ? force_share == 2 : wgs >= 2 * (int64_t)spa_device_cus();
+    if (share) {
+      p.nqt = nqt2;
+      return launch<flash_fwd16_kernel<T, D, 2, true, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, true>::SMEM, p, stream);
+    }
   }
   if (two) return launch<flash_fwd16_kernel<T, D, 2, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
   return launch<flash_fwd16_kernel<T, D, 1, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);

@@ -89,6 +89,50 @@ def test_e4m3_kv_with_one_and_two_wave_groups(groups):
     check_lse(lse, want_lse)
 
 
+@pytest.mark.parametrize("B,H,Sq,Sk,D,causal,dtype", [(1, 2, 512, 512, 128, True, torch.bfloat16),
+                                                      (2, 3, 300, 333, 128, False, torch.bfloat16),
+                                                      (1, 2, 256, 130, 128, True, torch.float16),
+                                                      (1, 4, 640, 640, 64, True, torch.bfloat16),
+                                                      (1, 2, 77, 1000, 64, False, torch.float16)])
+def test_e4m3_kv_with_shared_buffers(B, H, Sq, Sk, D, causal, dtype):
+    """The 256-row workgroups whose two wave groups stage one set of K/V tiles together (large launches pick
+    them; here forced), against the oracle, and within rounding of the 128-row form (which sums the keys in
+    another order)."""
+    from sp_aurora_amd import _lib
+    q = rand((B, H, Sq, D), 560, dtype)
+    k8, ksc, k_deq = quantised((B, H, Sk, D), 561, "bhsd")
+    v8, vsc, v_deq = quantised((B, H, Sk, D), 562, "bhsd")
+    want_out, want_lse = O.attn_block(q, k_deq, v_deq, None, causal)
+    got = {}
+    try:
+        for share in (2, 1):
+            _lib.tune("fwd_share", share)
+            got[share] = ops.flash_fwd(q.to(DEV), k8.to(DEV), v8.to(DEV), None, causal, layout="bhsd", k_scale=ksc, v_scale=vsc)
+    finally:
+        _lib.tune("fwd_share", 0)
+    check_out(got[2][0], want_out, dtype)
+    check_lse(got[2][1], want_lse)
+    check_out(got[2][0], got[1][0].double().cpu(), dtype)
+    check_lse(got[2][1], got[1][1].double().cpu())
+
+
+def test_ring_all_ranks_with_e4m3_kv_and_shared_buffers():
+    """One launch for every rank of a causal ring (the schedule the shared-buffer form serves), forced onto it."""
+    from sp_aurora_amd import _lib
+    B, S, H, D, P = 1, 1024, 2, 128, 4
+    q = rand((B, S, H, D), 570, torch.bfloat16)
+    k8, ksc, k_deq = quantised((B, S, H, D), 571, "bshd")
+    v8, vsc, v_deq = quantised((B, S, H, D), 572, "bshd")
+    want_out, want_lse = O.full_attention(q, k_deq, v_deq, None, True)
+    try:
+        _lib.tune("fwd_share", 2)
+        out, lse = ops.ring_fwd(q.to(DEV), k8.to(DEV), v8.to(DEV), ring_size=P, causal=True, rank=-1, fuse="all", k_scale=ksc, v_scale=vsc)
+    finally:
+        _lib.tune("fwd_share", 0)
+    check_out(out, want_out, torch.bfloat16)
+    check_lse(lse, want_lse)
+
+
 @pytest.mark.parametrize("lengths,H,D,causal", [([128, 256, 128], 8, 64, True), ([1, 77, 300, 5, 129], 3, 128, False),
                                                 ([1, 77, 300, 5, 129], 3, 128, True)])
 def test_varlen_forward_with_e4m3_kv(lengths, H, D, causal):
