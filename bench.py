@@ -378,14 +378,20 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
         y = ys[0]
         del ys, backs
         scale = Dn ** -0.5
-        fn = lambda: spa.intel_ulysses_flash_attn_forward(None, q, k, v, scale, causal=True)
+        fn = lambda: spa.intel_ulysses_flash_attn_forward(None, q, k, v, scale, causal=True, relayout="kernels")
         fn()
         m = measure(torch, fn, 5, 2, **light)
         flops = 4.0 * Bn * Hn * (Pn * sn) ** 2 * Dn / 2
         tf = flops / (m["ms_per_step"] * 1e-3) / 1e12
+        # the same result with head groups read and written in place (B = 1: no re-layout pass at all)
+        fv = lambda: spa.intel_ulysses_flash_attn_forward(None, q, k, v, scale, causal=True, relayout="views")
+        fv()
+        mv = measure(torch, fv, 5, 2, **light)
         finish("config4_ulysses_forward", m,
                {"workload": "config 4: q,k,v [P=8,B=1,s=2048,H=32,D=128] bf16 -> head-sharded [8,1,16384,4,128], full causal attention per head group, "
-                            "inverse re-layout of out (3 re-layouts in, attention, 1 out; output allocation included)", "flops_per_step": flops},
+                            "inverse re-layout of out (3 re-layouts in, attention, 1 out; output allocation included)", "flops_per_step": flops,
+                "same_result_through_strided_views": {"ms_per_step": round(mv["ms_per_step"], 4),
+                                                      "tflops": round(flops / (mv["ms_per_step"] * 1e-3) / 1e12, 2)}},
                tf, "TFLOP/s", roof("mfma", "relayout_kernel x4 + flash_fwd16_kernel<bf16,128,2>", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
         del q, k, v, y, xs
     if "fp8kv" in which:

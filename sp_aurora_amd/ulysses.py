@@ -115,18 +115,36 @@ class SeqAllToAll5D(torch.autograd.Function):
 
 
 def intel_ulysses_flash_attn_forward(process_group, q, k, v, softmax_scale, dropout_p=0.0, causal=False,
-                                     window_size=(-1, -1), alibi_slopes=None, deterministic=False):
+                                     window_size=(-1, -1), alibi_slopes=None, deterministic=False, *, relayout="auto"):
     """Ulysses forward for all ranks: re-layout q,k,v, attention over the full sequence on
     H/P heads per rank, inverse re-layout of out (sp_aurora/intel_ulysses_attn.py:233-287).
 
     q,k,v: rank-stacked [P,B,s,H,D] (or a single rank's [B,S,H,D], P = 1).
     Returns out like q and lse fp32 [P,B,H/P,P*s] — head-sharded, as the reference leaves it
-    (:284-287)."""
+    (:284-287).
+
+    relayout (not in the reference): "kernels" runs the four re-layout passes; "views" runs none -
+    with B = 1 the rank-stacked tensor IS the full sequence [P*s, H, D], head group r is a strided
+    view of it (heads r*h .. r*h+h-1), and the attention kernel reads and writes such views as they
+    are, which on one GPU is what peer writes into the head-sharded layout are across GPUs;
+    "auto" = "views" where it applies (B = 1, compact tensors), else "kernels"."""
     _no_multi_gpu(process_group)
     _check_unsupported(dropout_p, window_size, alibi_slopes)
+    if relayout not in ("auto", "views", "kernels"):
+        raise ValueError(f"relayout must be 'auto', 'views' or 'kernels', got {relayout!r}")
     if q.dim() == 4:
         return ops.flash_fwd(q, k, v, softmax_scale, causal, layout="bshd")
     P, B, s, H, D = q.shape
+    views_ok = B == 1 and H % P == 0 and all(t.is_contiguous() for t in (q, k, v)) and q.shape == k.shape == v.shape
+    if relayout == "views" and not views_ok:
+        raise ValueError("relayout='views' needs B = 1 and compact q, k, v of one shape")
+    if relayout != "kernels" and views_ok:
+        h = H // P
+        out = torch.empty_like(q)
+        # group r as a batch entry: [P groups, P*s rows, h heads, D] over the [P*s, H, D] sequence
+        grp = lambda t: t.as_strided((P, P * s, h, D), (h * D, H * D, D, 1), t.storage_offset())
+        _, lse = ops.flash_fwd(grp(q), grp(k), grp(v), softmax_scale, causal, layout="bshd", out=grp(out))
+        return out, lse.view(P, B, h, P * s)
     yq, yk, yv = ops.relayout_s2h(q, P), ops.relayout_s2h(k, P), ops.relayout_s2h(v, P)
     h = H // P
     # the P head groups are independent: fold the rank axis into the batch axis

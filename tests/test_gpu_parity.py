@@ -321,6 +321,28 @@ def test_ulysses_equals_full_attention(causal):
     assert torch.equal(spa.ulysses_flash_attn_qkvpacked_func(qkv, causal=causal), out)
 
 
+@pytest.mark.parametrize("P,s,H,D,dtype,causal", [(4, 64, 8, 64, torch.float16, True), (2, 100, 4, 128, torch.bfloat16, True),
+                                                  (8, 40, 8, 128, torch.bfloat16, False), (3, 130, 6, 32, torch.float16, True)])
+def test_ulysses_through_views_equals_ulysses_through_relayout_kernels(P, s, H, D, dtype, causal):
+    """B = 1: head group r read and written in place as a strided view, no re-layout pass, against the four
+    re-layout passes around the same attention call (bit for bit) and against the oracle."""
+    B = 1
+    q, k, v = rand_qkv((B, P * s, H, D), 95, dtype)
+    want_out, want_lse = O.full_attention(q, k, v, None, causal)
+    stack = lambda t: torch.stack(t.chunk(P, 1)).contiguous().to(DEV)
+    xq, xk, xv = stack(q), stack(k), stack(v)
+    out_v, lse_v = spa.intel_ulysses_flash_attn_forward(None, xq, xk, xv, D ** -0.5, causal=causal, relayout="views")
+    out_k, lse_k = spa.intel_ulysses_flash_attn_forward(None, xq, xk, xv, D ** -0.5, causal=causal, relayout="kernels")
+    assert torch.equal(out_v, out_k) and torch.equal(lse_v, lse_k)
+    check_out(torch.cat(list(out_v), 1), want_out, dtype)
+    check_lse(torch.cat(list(lse_v), 1), want_lse)
+    out_a, _ = spa.intel_ulysses_flash_attn_forward(None, xq, xk, xv, D ** -0.5, causal=causal)
+    assert torch.equal(out_a, out_v)
+    with pytest.raises(ValueError):
+        spa.intel_ulysses_flash_attn_forward(None, torch.cat([xq, xq], 1), torch.cat([xk, xk], 1), torch.cat([xv, xv], 1),
+                                             D ** -0.5, causal=causal, relayout="views")
+
+
 # ------------------------------------------------------------------ backward
 GRAD_TOL = {torch.bfloat16: dict(atol=3e-2, rtol=3e-2), torch.float16: dict(atol=4e-3, rtol=1e-2),
             torch.float32: dict(atol=2e-5, rtol=1e-4)}
