@@ -343,6 +343,22 @@ def test_ulysses_through_views_equals_ulysses_through_relayout_kernels(P, s, H, 
                                              D ** -0.5, causal=causal, relayout="views")
 
 
+@pytest.mark.parametrize("P,B,s,H,D,dtype,causal", [(4, 1, 64, 8, 64, torch.bfloat16, True), (2, 1, 100, 4, 128, torch.float16, False),
+                                                    (4, 2, 48, 4, 64, torch.bfloat16, True)])
+def test_ulysses_gradients(P, B, s, H, D, dtype, causal):
+    """Backward of the Ulysses function on rank-stacked tensors against the oracle's autograd through full
+    attention: B = 1 runs on strided views of the stacked tensors, B = 2 through the re-layout passes."""
+    q, k, v, dout = rand_qkv((B, P * s, H, D), 97, dtype, n=4)
+    want = O.attn_backward_autograd(q, k, v, dout, None, causal)
+    stack = lambda t: torch.stack(t.chunk(P, 1)).contiguous().to(DEV)
+    xs = [stack(t).requires_grad_(True) for t in (q, k, v)]
+    out = spa.ulysses_flash_attn_func(*xs, causal=causal)
+    out.backward(stack(dout))
+    for x, w, name in zip(xs, want, "qkv"):
+        assert x.grad.shape == (P, B, s, H, D) and x.grad.dtype == dtype
+        check_grad(torch.cat(list(x.grad), 1), w, dtype, "d" + name)
+
+
 # ------------------------------------------------------------------ backward
 GRAD_TOL = {torch.bfloat16: dict(atol=3e-2, rtol=3e-2), torch.float16: dict(atol=4e-3, rtol=1e-2),
             torch.float32: dict(atol=2e-5, rtol=1e-4)}
