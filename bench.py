@@ -471,7 +471,7 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
         tf = bwd_flops / (m["ms_per_step"] * 1e-3) / 1e12
         finish("config5_ring_backward", m,
                {"workload": "config 5 backward: dq/dk/dv by block-wise recompute with the global lse over the same 136 block pairs, one launch per kernel "
-                            "(delta pre-pass, fp32 accumulator zeroing and final casts included); 5-GEMM FLOP count (the two kernels execute 7)",
+                            "(delta pre-pass and output allocation included; the kernels write the gradients in bf16: spa_flash_bwd_out); 5-GEMM FLOP count (the two kernels execute 7)",
                 "flops_per_step": bwd_flops},
                tf, "TFLOP/s", roof("mfma", "flash_bwd_dq_kernel + flash_bwd_dkdv_kernel", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
         del qkv, dout, out, lse

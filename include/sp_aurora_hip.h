@@ -244,6 +244,23 @@ int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout,
                   float scale, int mask_mode, int dtype, void* stream);
 
 /*
+ * spa_flash_bwd for a gradient that ONE call computes in full (a whole block, or a whole simulated
+ * ring over the full-sequence tensors): dq [B,H,Sq,D], dk / dv [B,H,Sk,D] have the inputs' element
+ * type `dtype` and are WRITTEN, not added to - no fp32 accumulators to zero, read back and cast.
+ * The values are those of spa_flash_bwd into zeroed accumulators followed by the reference's final
+ * cast to q's type (sp_aurora/intel_ring_flash_attn.py:250-271), bit for bit.
+ */
+int spa_flash_bwd_out(const void* q, const void* k, const void* v, const void* dout,
+                      const float* lse, const float* delta,
+                      void* dq, void* dk, void* dv,
+                      int B, int H, int Sq, int Sk, int D,
+                      const int64_t q_strides[3], const int64_t k_strides[3],
+                      const int64_t v_strides[3], const int64_t do_strides[3],
+                      const int64_t dq_strides[3], const int64_t dk_strides[3],
+                      const int64_t dv_strides[3],
+                      float scale, int mask_mode, int dtype, void* stream);
+
+/*
  * Block attention over a batch of sequences of different lengths packed back
  * to back (no padding): q / out are [total_q, H, D], k / v [total_k, H, D];
  * sequence b owns query rows cu_seqlens_q[b] .. cu_seqlens_q[b+1] and key rows

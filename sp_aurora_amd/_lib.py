@@ -39,6 +39,7 @@ SIGNATURES = {
     "spa_relayout_h2s": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "spa_bwd_delta": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _s3, _s3, _i, _vp]),
     "spa_flash_bwd": (_i, [_vp] * 9 + [_i] * 5 + [_s3] * 7 + [_f, _i, _i, _vp]),
+    "spa_flash_bwd_out": (_i, [_vp] * 9 + [_i] * 5 + [_s3] * 7 + [_f, _i, _i, _vp]),
     "spa_flash_fwd_varlen": (_i, [_vp] * 7 + [_i] * 7 + [_s3] * 4 + [_f, _i, _i, _vp]),
     "spa_flash_bwd_varlen": (_i, [_vp] * 11 + [_i] * 7 + [_s3] * 7 + [_f, _i, _i, _vp]),
 }

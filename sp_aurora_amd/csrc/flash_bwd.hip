@@ -424,7 +424,19 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
   // wait, so no read of them can be scheduled above it.
   if constexpr (MIXED) asm volatile("s_nop 15\n s_nop 15" : "+a"(dq[0]), "+a"(dq[1]), "+a"(dq[2]), "+a"(dq[3])::"memory");
 
-  if (qrow < p.Sq) {
+  if (qrow < p.Sq && p.grads_in_t) {
+    // the whole gradient of the row: written in q's element type, nothing read
+    T* dqp = (T*)p.dq + b * p.dqs.b + h * p.dqs.h + (int64_t)qrow * p.dqs.s;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 st;
+        st[0] = Mma16<T>::pack2(dq[db][4 * g + 0] * p.scale, dq[db][4 * g + 1] * p.scale);
+        st[1] = Mma16<T>::pack2(dq[db][4 * g + 2] * p.scale, dq[db][4 * g + 3] * p.scale);
+        *(u32x2*)(dqp + db * 32 + 8 * g + 4 * hh) = st;
+      }
+  } else if (qrow < p.Sq) {
     float* dqp = p.dq + b * p.dqs.b + h * p.dqs.h + (int64_t)qrow * p.dqs.s;
 #pragma unroll
     for (int db = 0; db < D / 32; ++db)
@@ -714,7 +726,22 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
     asm volatile("s_nop 15\n s_nop 15"
                  : "+a"(dk[0]), "+a"(dk[1]), "+a"(dk[2]), "+a"(dk[3]), "+a"(dv[0]), "+a"(dv[1]), "+a"(dv[2]), "+a"(dv[3])::"memory");
 
-  if (krow < p.Sk) {
+  if (krow < p.Sk && p.grads_in_t) {
+    T* dkp = (T*)p.dk + b * p.dks.b + h * p.dks.h + (int64_t)krow * p.dks.s;
+    T* dvp = (T*)p.dv + b * p.dvs.b + h * p.dvs.h + (int64_t)krow * p.dvs.s;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 x, y;
+        x[0] = Mma16<T>::pack2(dk[db][4 * g + 0] * p.scale, dk[db][4 * g + 1] * p.scale);
+        x[1] = Mma16<T>::pack2(dk[db][4 * g + 2] * p.scale, dk[db][4 * g + 3] * p.scale);
+        y[0] = Mma16<T>::pack2(dv[db][4 * g + 0], dv[db][4 * g + 1]);
+        y[1] = Mma16<T>::pack2(dv[db][4 * g + 2], dv[db][4 * g + 3]);
+        *(u32x2*)(dkp + db * 32 + 8 * g + 4 * hh) = x;
+        *(u32x2*)(dvp + db * 32 + 8 * g + 4 * hh) = y;
+      }
+  } else if (krow < p.Sk) {
     float* dkp = p.dk + b * p.dks.b + h * p.dks.h + (int64_t)krow * p.dks.s;
     float* dvp = p.dv + b * p.dvs.b + h * p.dvs.h + (int64_t)krow * p.dvs.s;
 #pragma unroll
@@ -883,7 +910,8 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dq_kernel(const Bw
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         f32x4* dst = (f32x4*)(dqp + db * 32 + 8 * g + 4 * hh);
-        f32x4 x = *dst;
+        f32x4 x = {0.f, 0.f, 0.f, 0.f};
+        if (!p.grads_in_t) x = *dst;
 #pragma unroll
         for (int e = 0; e < 4; ++e) x[e] += dq[db][4 * g + e] * p.scale;
         *dst = x;
@@ -1009,7 +1037,23 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dkdv_kernel(const 
     __syncthreads();
   }
 
-  if (krow < p.Sk) {
+  if (krow < p.Sk && p.grads_in_t) {
+    float* dkp = p.dk + b * p.dks.b + h * p.dks.h + (int64_t)krow * p.dks.s;
+    float* dvp = p.dv + b * p.dvs.b + h * p.dvs.h + (int64_t)krow * p.dvs.s;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 x, y;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          x[e] = dk[db][4 * g + e] * p.scale;
+          y[e] = dv[db][4 * g + e];
+        }
+        *(f32x4*)(dkp + db * 32 + 8 * g + 4 * hh) = x;
+        *(f32x4*)(dvp + db * 32 + 8 * g + 4 * hh) = y;
+      }
+  } else if (krow < p.Sk) {
     float* dkp = p.dk + b * p.dks.b + h * p.dks.h + (int64_t)krow * p.dks.s;
     float* dvp = p.dv + b * p.dvs.b + h * p.dvs.h + (int64_t)krow * p.dvs.s;
 #pragma unroll

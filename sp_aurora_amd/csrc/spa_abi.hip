@@ -437,33 +437,36 @@ int spa_bwd_delta(const void* out, const void* dout, float* delta, int B, int H,
                        "spa_bwd_delta");
 }
 
-int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
-                  const float* delta, float* dq_acc, float* dk_acc, float* dv_acc, int B, int H, int Sq, int Sk,
-                  int D, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
-                  const int64_t do_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
-                  const int64_t dv_strides[3], float scale, int mask_mode, int dtype, void* stream) {
-  if (!q || !k || !v || !dout || !lse || !delta || !dq_acc || !dk_acc || !dv_acc)
-    return fail(SPA_EINVAL, "spa_flash_bwd: null pointer");
+namespace {
+// grads_in_t: dq / dk / dv are tensors of the inputs' element type and are written (spa_flash_bwd_out);
+// else fp32 accumulators that are added to (spa_flash_bwd).
+int flash_bwd(const char* what, const void* q, const void* k, const void* v, const void* dout, const float* lse,
+              const float* delta, void* dq, void* dk, void* dv, bool grads_in_t, int B, int H, int Sq, int Sk,
+              int D, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+              const int64_t do_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+              const int64_t dv_strides[3], float scale, int mask_mode, int dtype, void* stream) {
+  if (!q || !k || !v || !dout || !lse || !delta || !dq || !dk || !dv) return fail(SPA_EINVAL, "%s: null pointer", what);
   if (!q_strides || !k_strides || !v_strides || !do_strides || !dq_strides || !dk_strides || !dv_strides)
-    return fail(SPA_EINVAL, "spa_flash_bwd: null strides");
-  if (!dims_ok(B, H, Sq, D) || Sk <= 0) return fail(SPA_EINVAL, "spa_flash_bwd: sizes must be positive");
-  if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "spa_flash_bwd: bad dtype %d", dtype);
-  if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "spa_flash_bwd: bad mask_mode %d", mask_mode);
-  if (!scale_ok(scale)) return fail(SPA_EINVAL, "spa_flash_bwd: softmax scale must be finite");
-  if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "spa_flash_bwd: head dim %d not in {32,64,128}", D);
-  const int esz = elem_size(dtype);
+    return fail(SPA_EINVAL, "%s: null strides", what);
+  if (!dims_ok(B, H, Sq, D) || Sk <= 0) return fail(SPA_EINVAL, "%s: sizes must be positive", what);
+  if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "%s: bad dtype %d", what, dtype);
+  if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "%s: bad mask_mode %d", what, mask_mode);
+  if (!scale_ok(scale)) return fail(SPA_EINVAL, "%s: softmax scale must be finite", what);
+  if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "%s: head dim %d not in {32,64,128}", what, D);
+  const int esz = elem_size(dtype), gsz = grads_in_t ? esz : 4;
   if (!aligned16(q, q_strides, esz) || !aligned16(k, k_strides, esz) || !aligned16(v, v_strides, esz) ||
-      !aligned16(dout, do_strides, esz) || !aligned16(dq_acc, dq_strides, 4) || !aligned16(dk_acc, dk_strides, 4) ||
-      !aligned16(dv_acc, dv_strides, 4))
-    return fail(SPA_EALIGN, "spa_flash_bwd: pointers and row strides must be 16-byte aligned");
+      !aligned16(dout, do_strides, esz) || !aligned16(dq, dq_strides, gsz) || !aligned16(dk, dk_strides, gsz) ||
+      !aligned16(dv, dv_strides, gsz))
+    return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned", what);
   if (!span_ok(Sq, q_strides[2], D, esz) || !span_ok(Sk, k_strides[2], D, esz) || !span_ok(Sk, v_strides[2], D, esz) ||
       !span_ok(Sq, do_strides[2], D, esz))
-    return fail(SPA_EUNSUPPORTED, "spa_flash_bwd: a tensor of one (batch, head) spans more than 2 GiB");
+    return fail(SPA_EUNSUPPORTED, "%s: a tensor of one (batch, head) spans more than 2 GiB", what);
   if ((int64_t)B * H * ((Sq + 127) / 128) > 0x7fffffffLL || (int64_t)B * H * ((Sk + 127) / 128) > 0x7fffffffLL)
-    return fail(SPA_EINVAL, "spa_flash_bwd: grid too large");
+    return fail(SPA_EINVAL, "%s: grid too large", what);
   BwdParams p;
   p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta;
-  p.dq = dq_acc; p.dk = dk_acc; p.dv = dv_acc;
+  p.dq = (float*)dq; p.dk = (float*)dk; p.dv = (float*)dv;
+  p.grads_in_t = grads_in_t;
   p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
   p.qs = S3(q_strides); p.ks = S3(k_strides); p.vs = S3(v_strides); p.dos = S3(do_strides);
   p.dqs = S3(dq_strides); p.dks = S3(dk_strides); p.dvs = S3(dv_strides);
@@ -474,7 +477,26 @@ int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout,
   p.nkt = 0;
   p.lse_bh = Sq;
   p.cu_q = nullptr; p.cu_k = nullptr;
-  return launch_result(spa_launch_flash_bwd(p, D, dtype, (hipStream_t)stream), "spa_flash_bwd");
+  return launch_result(spa_launch_flash_bwd(p, D, dtype, (hipStream_t)stream), what);
+}
+}  // namespace
+
+int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                  const float* delta, float* dq_acc, float* dk_acc, float* dv_acc, int B, int H, int Sq, int Sk,
+                  int D, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                  const int64_t do_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                  const int64_t dv_strides[3], float scale, int mask_mode, int dtype, void* stream) {
+  return flash_bwd("spa_flash_bwd", q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, false, B, H, Sq, Sk, D, q_strides, k_strides,
+                   v_strides, do_strides, dq_strides, dk_strides, dv_strides, scale, mask_mode, dtype, stream);
+}
+
+int spa_flash_bwd_out(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                      const float* delta, void* dq, void* dk, void* dv, int B, int H, int Sq, int Sk,
+                      int D, const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                      const int64_t do_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                      const int64_t dv_strides[3], float scale, int mask_mode, int dtype, void* stream) {
+  return flash_bwd("spa_flash_bwd_out", q, k, v, dout, lse, delta, dq, dk, dv, true, B, H, Sq, Sk, D, q_strides, k_strides,
+                   v_strides, do_strides, dq_strides, dk_strides, dv_strides, scale, mask_mode, dtype, stream);
 }
 
 namespace {
@@ -597,6 +619,7 @@ int spa_flash_bwd_varlen(const void* q, const void* k, const void* v, const void
   BwdParams p;
   p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta;
   p.dq = dq_acc; p.dk = dk_acc; p.dv = dv_acc;
+  p.grads_in_t = 0;
   p.B = nseq; p.H = H; p.Sq = max_sq; p.Sk = max_sk;
   p.qs = S2(q_strides); p.ks = S2(k_strides); p.vs = S2(v_strides); p.dos = S2(do_strides);
   p.dqs = S2(dq_strides); p.dks = S2(dk_strides); p.dvs = S2(dv_strides);

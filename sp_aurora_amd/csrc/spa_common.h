@@ -94,6 +94,9 @@ struct BwdParams {
   // cu_k[b] .. cu_k[b+1] of k/v/dk/dv belong to sequence b; lse and delta are [H][lse_bh]
   const int* cu_q;
   const int* cu_k;
+  // 0: dq/dk/dv are fp32 accumulators, added to; 1: they are tensors of q's element type (strides in
+  // those elements) and are WRITTEN: the whole gradient comes from this one launch
+  int grads_in_t;
 };
 
 // 16-bit element traits: MFMA 32x32x16 with 8 elements per lane per operand.

@@ -401,6 +401,44 @@ def _cu(cu, device, what):
     return cu
 
 
+def flash_bwd_out(q, k, v, dout, lse, delta, softmax_scale=None, causal=False, layout="bshd", dq=None, dk=None, dv=None):
+    """Backward that one call computes in full: returns (dq, dk, dv) in q's dtype, written by the kernels
+    (no fp32 accumulators).  dq, dk, dv may be given (views of q's / k's shape and dtype).  Calls spa_flash_bwd_out."""
+    if not (q.dtype == k.dtype == v.dtype == dout.dtype):
+        raise TypeError("flash_bwd_out: q, k, v, dout must share a dtype")
+    (B, H, Sq, D), _ = _bhs(q, layout)
+    shp_k, shp_v, shp_do = _bhs(k, layout)[0], _bhs(v, layout)[0], _bhs(dout, layout)[0]
+    Sk = shp_k[2]
+    if shp_k != (B, H, Sk, D) or shp_v != shp_k or shp_do != (B, H, Sq, D):
+        raise ValueError(f"flash_bwd_out: shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)} dout {tuple(dout.shape)}")
+    if tuple(lse.shape) != (B, H, Sq) or tuple(delta.shape) != (B, H, Sq):
+        raise ValueError(f"flash_bwd_out: lse {tuple(lse.shape)} and delta {tuple(delta.shape)} must be [B,H,Sq] = {(B, H, Sq)}")
+    for t in (lse, delta):
+        if t.dtype != torch.float32 or not t.is_contiguous() or t.device != q.device:
+            raise ValueError("flash_bwd_out: lse and delta must be contiguous float32 tensors on q's device")
+    q, k, v, dout = _prep(q), _prep(k), _prep(v), _prep(dout)
+    dq = torch.empty(q.shape, dtype=q.dtype, device=q.device) if dq is None else dq
+    dk = torch.empty(k.shape, dtype=q.dtype, device=q.device) if dk is None else dk
+    dv = torch.empty(v.shape, dtype=q.dtype, device=q.device) if dv is None else dv
+    for g, like, name in ((dq, q, "dq"), (dk, k, "dk"), (dv, v, "dv")):
+        # the kernels index the gradients with q's / k's sizes: a mismatch would be an out-of-bounds access
+        if tuple(g.shape) != tuple(like.shape) or g.dtype != q.dtype or g.device != q.device or not _rows_ok(g, g.element_size()):
+            raise ValueError(f"flash_bwd_out: {name} must have the shape, dtype and device of its input, inner stride 1 and 16-byte aligned rows")
+    if softmax_scale is None:
+        softmax_scale = D ** (-0.5)
+    lib = _lib.load()
+    qs, ks, vs, dos = _bhs(q, layout)[1], _bhs(k, layout)[1], _bhs(v, layout)[1], _bhs(dout, layout)[1]
+    dqs, dks, dvs = _bhs(dq, layout)[1], _bhs(dk, layout)[1], _bhs(dv, layout)[1]
+    with _on(q.device):
+        _lib.check(lib.spa_flash_bwd_out(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, Sq, Sk, D,
+            _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(dos),
+            _lib.strides3(dqs), _lib.strides3(dks), _lib.strides3(dvs),
+            float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(q), _stream()))
+    return dq, dk, dv
+
+
 def flash_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale=None,
                      causal=False, out=None, lse=None, k_scale=None, v_scale=None):
     """Attention inside each sequence of a packed batch: q [total_q,H,D], k,v [total_k,H,D],

@@ -135,24 +135,24 @@ def ring_flash_attn_backward(dout, q, k, v, out, softmax_lse, softmax_scale=None
     P = int(ring_size)
     lse = softmax_lse if softmax_lse.is_contiguous() else softmax_lse.contiguous()
     delta = ops.bwd_delta(out, dout, layout="bshd")
+    if P == 1 or fuse == "all":
+        # one launch of each kernel computes the whole gradient: written in q's dtype, no fp32 accumulators
+        return ops.flash_bwd_out(q, k, v, dout, lse, delta, softmax_scale, causal, layout="bshd")
     dq = torch.zeros((B, S, H, D), dtype=torch.float32, device=q.device)
     dk = torch.zeros((B, k.shape[1], H, D), dtype=torch.float32, device=q.device)
     dv = torch.zeros((B, k.shape[1], H, D), dtype=torch.float32, device=q.device)
-    if P == 1 or fuse == "all":
-        ops.flash_bwd(q, k, v, dout, lse, delta, dq, dk, dv, softmax_scale, causal, layout="bshd")
-    else:
-        s = S // P
-        for r in range(P):
-            rs = slice(r * s, (r + 1) * s)
-            lse_r = lse[:, :, rs].contiguous()
-            delta_r = delta[:, :, rs].contiguous()
-            for t in range(P):
-                if causal and t > r:
-                    continue
-                c = (r - t) % P
-                cs = slice(c * s, (c + 1) * s)
-                ops.flash_bwd(q[:, rs], k[:, cs], v[:, cs], dout[:, rs], lse_r, delta_r,
-                              dq[:, rs], dk[:, cs], dv[:, cs], softmax_scale, causal and t == 0, layout="bshd")
+    s = S // P
+    for r in range(P):
+        rs = slice(r * s, (r + 1) * s)
+        lse_r = lse[:, :, rs].contiguous()
+        delta_r = delta[:, :, rs].contiguous()
+        for t in range(P):
+            if causal and t > r:
+                continue
+            c = (r - t) % P
+            cs = slice(c * s, (c + 1) * s)
+            ops.flash_bwd(q[:, rs], k[:, cs], v[:, cs], dout[:, rs], lse_r, delta_r,
+                          dq[:, rs], dk[:, cs], dv[:, cs], softmax_scale, causal and t == 0, layout="bshd")
     return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype)
 
 

@@ -181,15 +181,15 @@ class UlyssesFlashAttnFunc(torch.autograd.Function):
             P, B, s, H, D = q.shape
             h = H // P
             if B == 1 and all(t.is_contiguous() for t in (q, k, v, out)):
-                # as in the forward: head groups are strided views of the stacked tensors, and the fp32
-                # gradient accumulators are views of stacked buffers, so nothing is re-laid
+                # as in the forward: head groups are strided views of the stacked tensors, and the kernels
+                # write the gradients through such views of stacked tensors, so nothing is re-laid
                 grp = lambda t: t.as_strided((P, P * s, h, D), (h * D, H * D, D, 1), t.storage_offset())
                 dout = dout.contiguous()
                 delta = ops.bwd_delta(grp(out), grp(dout), layout="bshd")
-                acc = [torch.zeros(q.shape, dtype=torch.float32, device=q.device) for _ in range(3)]
-                ops.flash_bwd(grp(q), grp(k), grp(v), grp(dout), lse.view(P, h, P * s), delta, grp(acc[0]), grp(acc[1]), grp(acc[2]),
-                              ctx.softmax_scale, ctx.causal, layout="bshd")
-                return (acc[0].to(q.dtype), acc[1].to(k.dtype), acc[2].to(v.dtype)) + (None,) * 8
+                grads = [torch.empty_like(q) for _ in range(3)]
+                ops.flash_bwd_out(grp(q), grp(k), grp(v), grp(dout), lse.view(P, h, P * s), delta, ctx.softmax_scale, ctx.causal,
+                                  layout="bshd", dq=grp(grads[0]), dk=grp(grads[1]), dv=grp(grads[2]))
+                return tuple(grads) + (None,) * 8
             fold = lambda t: ops.relayout_s2h(t.contiguous(), P).view(P * B, P * s, h, D)
             gq, gk, gv = ring_flash_attn_backward(fold(dout), fold(q), fold(k), fold(v), fold(out),
                                                   lse.view(P * B, h, P * s), ctx.softmax_scale, ctx.causal, 1)

@@ -388,6 +388,35 @@ def test_backward_matches_autograd_of_full_attention(B, S, H, D, causal, P, dtyp
         check_grad(got, w, dtype, "d" + name)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("B,Sq,Sk,H,D,causal", [(1, 300, 300, 2, 128, True), (2, 130, 257, 3, 64, False), (1, 64, 64, 1, 32, True),
+                                                (1, 1000, 1000, 2, 128, True)])
+def test_backward_written_in_the_inputs_type_equals_accumulate_then_cast(B, Sq, Sk, H, D, causal, dtype):
+    """spa_flash_bwd_out against spa_flash_bwd into zeroed fp32 accumulators followed by the cast
+    (sp_aurora/intel_ring_flash_attn.py:250-271): bit for bit, also through strided gradient views."""
+    g = torch.Generator().manual_seed(160)
+    q, dout = [(torch.randn(B, Sq, H, D, generator=g) * 0.5).to(dtype).to(DEV) for _ in range(2)]
+    k, v = [(torch.randn(B, Sk, H, D, generator=g) * 0.5).to(dtype).to(DEV) for _ in range(2)]
+    out, lse = ops.flash_fwd(q, k, v, None, causal, layout="bshd")
+    delta = ops.bwd_delta(out, dout, layout="bshd")
+    acc = [torch.zeros(t.shape, dtype=torch.float32, device=DEV) for t in (q, k, v)]
+    ops.flash_bwd(q, k, v, dout, lse, delta, *acc, None, causal, layout="bshd")
+    want = [a.to(dtype) for a in acc]
+    got = ops.flash_bwd_out(q, k, v, dout, lse, delta, None, causal, layout="bshd")
+    for gt, w, name in zip(got, want, "qkv"):
+        assert gt.dtype == dtype and torch.equal(gt, w), f"d{name}"
+    # gradients written into the halves of packed buffers (row stride 2 H D)
+    pq = torch.full((B, Sq, 2, H, D), 7.0, dtype=dtype, device=DEV)
+    pkv = torch.full((B, Sk, 2, H, D), 7.0, dtype=dtype, device=DEV)
+    ops.flash_bwd_out(q, k, v, dout, lse, delta, None, causal, layout="bshd", dq=pq[:, :, 1], dk=pkv[:, :, 0], dv=pkv[:, :, 1])
+    assert torch.equal(pq[:, :, 1], want[0]) and torch.equal(pkv[:, :, 0], want[1]) and torch.equal(pkv[:, :, 1], want[2])
+    assert (pq[:, :, 0] == 7.0).all()
+    with pytest.raises(ValueError):
+        ops.flash_bwd_out(q, k, v, dout, lse, delta, None, causal, layout="bshd", dq=torch.empty_like(k[:, :1]))
+    with pytest.raises(ValueError):
+        ops.flash_bwd_out(q, k, v, dout, lse, delta, None, causal, layout="bshd", dk=torch.empty(k.shape, dtype=torch.float64, device=DEV))
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("Sq,Sk,causal", [(96, 100, False), (130, 70, False), (100, 100, True)])
 def test_backward_with_strongly_negative_scores_and_ragged_keys(Sq, Sk, causal, dtype):
