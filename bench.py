@@ -683,7 +683,7 @@ def main():
     if os.path.exists(TRAFFIC_JSON):
         try:
             traffic = json.load(open(TRAFFIC_JSON)).get("hbm_bytes_per_launch")
-            traffic_src = ("profiles/flash_fwd_traffic.json: two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of an earlier build of this "
+            traffic_src = ("profiles/flash_fwd_traffic.json: two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of this "
                            "kernel, scaled by a 1 GiB copy; a recorded constant, not measured in this run")
         except (ValueError, OSError):
             traffic = None
