@@ -248,7 +248,8 @@ int spa_flash_bwd(const void* q, const void* k, const void* v, const void* dout,
  * ring over the full-sequence tensors): dq [B,H,Sq,D], dk / dv [B,H,Sk,D] have the inputs' element
  * type `dtype` and are WRITTEN, not added to - no fp32 accumulators to zero, read back and cast.
  * The values are those of spa_flash_bwd into zeroed accumulators followed by the reference's final
- * cast to q's type (sp_aurora/intel_ring_flash_attn.py:250-271), bit for bit.
+ * cast to q's type (sp_aurora/intel_ring_flash_attn.py:250-271), bit for bit; rows of dk / dv that
+ * no query sees (causal with Sk > Sq) are written as zeros.
  */
 int spa_flash_bwd_out(const void* q, const void* k, const void* v, const void* dout,
                       const float* lse, const float* delta,
@@ -315,6 +316,24 @@ int spa_flash_bwd_varlen(const void* q, const void* k, const void* v, const void
                          const int64_t dq_strides[2], const int64_t dk_strides[2],
                          const int64_t dv_strides[2],
                          float scale, int mask_mode, int dtype, void* stream);
+
+/*
+ * spa_flash_bwd_varlen for the whole gradient in one call, as spa_flash_bwd_out is to spa_flash_bwd:
+ * dq [total_q, H, D], dk / dv [total_k, H, D] have the inputs' element type and are WRITTEN (zeros
+ * where a sequence has queries but no keys, or keys that no query sees).  Rows that belong to no
+ * sequence, or that lie past max_sq / max_sk of a longer sequence, are left untouched.  Same
+ * call site as spa_flash_bwd_varlen (test_intel_ring_flash_attn_varlen.py:85-91).
+ */
+int spa_flash_bwd_varlen_out(const void* q, const void* k, const void* v, const void* dout,
+                             const float* lse, const float* delta,
+                             void* dq, void* dk, void* dv,
+                             const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                             int nseq, int H, int total_q, int total_k, int max_sq, int max_sk, int D,
+                             const int64_t q_strides[2], const int64_t k_strides[2],
+                             const int64_t v_strides[2], const int64_t do_strides[2],
+                             const int64_t dq_strides[2], const int64_t dk_strides[2],
+                             const int64_t dv_strides[2],
+                             float scale, int mask_mode, int dtype, void* stream);
 
 /*
  * Kernel-variant override for experiments and tests; no counterpart in the reference and not

@@ -188,12 +188,31 @@ __device__ __forceinline__ void select_sequence(BwdParams& p, int& b) {
   p.dout = (const T*)p.dout + (int64_t)q_lo * p.dos.s;
   p.k = (const T*)p.k + (int64_t)k_lo * p.ks.s;
   p.v = (const T*)p.v + (int64_t)k_lo * p.vs.s;
-  p.dq += (int64_t)q_lo * p.dqs.s;
-  p.dk += (int64_t)k_lo * p.dks.s;
-  p.dv += (int64_t)k_lo * p.dvs.s;
+  const int64_t gsz = p.grads_in_t ? (int64_t)sizeof(T) : 4;  // gradients written in T, or fp32 accumulators
+  p.dq = (float*)((char*)p.dq + q_lo * p.dqs.s * gsz);
+  p.dk = (float*)((char*)p.dk + k_lo * p.dks.s * gsz);
+  p.dv = (float*)((char*)p.dv + k_lo * p.dvs.s * gsz);
   p.lse += q_lo;
   p.delta += q_lo;
   b = 0;
+}
+
+// A row of a gradient that is written (BwdParams::grads_in_t) and that no tile contributes to: the
+// lane's share of the row (the columns the epilogues give it) is set to zero.
+template <typename E, int D>
+__device__ __forceinline__ void zero_grad_row(E* rowp, int hh) {
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      if constexpr (sizeof(E) == 2) {
+        const u32x2 z = {0u, 0u};
+        *(u32x2*)(rowp + db * 32 + 8 * g + 4 * hh) = z;
+      } else {
+        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+        *(f32x4*)(rowp + db * 32 + 8 * g + 4 * hh) = z;
+      }
+    }
 }
 
 template <typename T, int D, int NW>
@@ -222,7 +241,11 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
   const int q0 = qt * (NW * 32);
   const int qw0 = q0 + w * 32;
   select_sequence<T>(p, b);
-  if (q0 >= p.Sq || p.Sk <= 0) return;  // (variable-length batches only) nothing to add to dq
+  if (q0 >= p.Sq || p.Sk <= 0) {  // (variable-length batches only) no keys: nothing to add to dq, a written dq is zero
+    if (p.grads_in_t && qw0 + ln < p.Sq)
+      zero_grad_row<T, D>((T*)p.dq + b * p.dqs.b + h * p.dqs.h + (int64_t)(qw0 + ln) * p.dqs.s, hh);
+    return;
+  }
 
   const T* qp = (const T*)p.q + b * p.qs.b + h * p.qs.h;
   const T* kp = (const T*)p.k + b * p.ks.b + h * p.ks.h;
@@ -490,7 +513,13 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
   const int k0 = kt * 128;
   const int kw0 = k0 + w * 32;
   select_sequence<T>(p, b);
-  if (k0 >= p.Sk || p.Sq <= 0 || (p.causal && k0 >= p.Sq)) return;  // no query sees these keys: nothing to add to dk, dv
+  if (k0 >= p.Sk || p.Sq <= 0 || (p.causal && k0 >= p.Sq)) {  // no query sees these keys: nothing to add to dk, dv
+    if (p.grads_in_t && kw0 + ln < p.Sk) {                     // written gradients of such keys are zero
+      zero_grad_row<T, D>((T*)p.dk + b * p.dks.b + h * p.dks.h + (int64_t)(kw0 + ln) * p.dks.s, hh);
+      zero_grad_row<T, D>((T*)p.dv + b * p.dvs.b + h * p.dvs.h + (int64_t)(kw0 + ln) * p.dvs.s, hh);
+    }
+    return;
+  }
 
   const T* qp = (const T*)p.q + b * p.qs.b + h * p.qs.h;
   const T* kp = (const T*)p.k + b * p.ks.b + h * p.ks.h;
@@ -830,7 +859,11 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dq_kernel(const Bw
   const int q0 = qt * 128;
   const int qw0 = q0 + w * 32;
   select_sequence<float>(p, b);
-  if (q0 >= p.Sq || p.Sk <= 0) return;  // (variable-length batches only) nothing to add to dq
+  if (q0 >= p.Sq || p.Sk <= 0) {  // (variable-length batches only) no keys: nothing to add to dq, a written dq is zero
+    if (p.grads_in_t && qw0 + ln < p.Sq)
+      zero_grad_row<float, D>(p.dq + b * p.dqs.b + h * p.dqs.h + (int64_t)(qw0 + ln) * p.dqs.s, hh);
+    return;
+  }
 
   const float* qp = (const float*)p.q + b * p.qs.b + h * p.qs.h;
   const float* kp = (const float*)p.k + b * p.ks.b + h * p.ks.h;
@@ -936,7 +969,13 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd32_dkdv_kernel(const 
   const int k0 = kt * 128;
   const int kw0 = k0 + w * 32;
   select_sequence<float>(p, b);
-  if (k0 >= p.Sk || p.Sq <= 0 || (p.causal && k0 >= p.Sq)) return;  // no query sees these keys: nothing to add to dk, dv
+  if (k0 >= p.Sk || p.Sq <= 0 || (p.causal && k0 >= p.Sq)) {  // no query sees these keys: nothing to add to dk, dv
+    if (p.grads_in_t && kw0 + ln < p.Sk) {                     // written gradients of such keys are zero
+      zero_grad_row<float, D>(p.dk + b * p.dks.b + h * p.dks.h + (int64_t)(kw0 + ln) * p.dks.s, hh);
+      zero_grad_row<float, D>(p.dv + b * p.dvs.b + h * p.dvs.h + (int64_t)(kw0 + ln) * p.dvs.s, hh);
+    }
+    return;
+  }
 
   const float* qp = (const float*)p.q + b * p.qs.b + h * p.qs.h;
   const float* kp = (const float*)p.k + b * p.ks.b + h * p.ks.h;

@@ -568,6 +568,44 @@ int flash_fwd_varlen(const char* what, const void* q, const void* k, const void*
   p.k_scale = k_scale; p.v_scale = v_scale;
   return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), what);
 }
+
+// grads_in_t: as in flash_bwd above.
+int flash_bwd_varlen(const char* what, const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                     const float* delta, void* dq, void* dk, void* dv, bool grads_in_t, const int32_t* cu_seqlens_q,
+                     const int32_t* cu_seqlens_k, int nseq, int H, int total_q, int total_k, int max_sq, int max_sk,
+                     int D, const int64_t q_strides[2], const int64_t k_strides[2], const int64_t v_strides[2],
+                     const int64_t do_strides[2], const int64_t dq_strides[2], const int64_t dk_strides[2],
+                     const int64_t dv_strides[2], float scale, int mask_mode, int dtype, void* stream) {
+  if (!q || !k || !v || !dout || !lse || !delta || !dq || !dk || !dv) return fail(SPA_EINVAL, "%s: null pointer", what);
+  if (!q_strides || !k_strides || !v_strides || !do_strides || !dq_strides || !dk_strides || !dv_strides)
+    return fail(SPA_EINVAL, "%s: null strides", what);
+  const int rc = varlen_sizes_ok(what, cu_seqlens_q, cu_seqlens_k, nseq, H, total_q, total_k, max_sq, max_sk, D, dtype,
+                                 mask_mode, scale);
+  if (rc != SPA_OK) return rc;
+  const int esz = elem_size(dtype), gsz = grads_in_t ? esz : 4;
+  if (!aligned16v(q, q_strides, esz) || !aligned16v(k, k_strides, esz) || !aligned16v(v, v_strides, esz) ||
+      !aligned16v(dout, do_strides, esz) || !aligned16v(dq, dq_strides, gsz) || !aligned16v(dk, dk_strides, gsz) ||
+      !aligned16v(dv, dv_strides, gsz) || (((uintptr_t)lse | (uintptr_t)delta) & 3) != 0)
+    return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned", what);
+  if (!span_ok(max_sq, q_strides[1], D, esz) || !span_ok(max_sk, k_strides[1], D, esz) ||
+      !span_ok(max_sk, v_strides[1], D, esz) || !span_ok(max_sq, do_strides[1], D, esz))
+    return fail(SPA_EUNSUPPORTED, "%s: a tensor of one (sequence, head) spans more than 2 GiB", what);
+  BwdParams p;
+  p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta;
+  p.dq = (float*)dq; p.dk = (float*)dk; p.dv = (float*)dv;
+  p.grads_in_t = grads_in_t;
+  p.B = nseq; p.H = H; p.Sq = max_sq; p.Sk = max_sk;
+  p.qs = S2(q_strides); p.ks = S2(k_strides); p.vs = S2(v_strides); p.dos = S2(do_strides);
+  p.dqs = S2(dq_strides); p.dks = S2(dk_strides); p.dvs = S2(dv_strides);
+  p.scale = scale_eff(scale);
+  p.scale_log2 = scale_eff(scale) * 1.4426950408889634f;
+  p.causal = mask_mode == SPA_MASK_CAUSAL;
+  p.nqt = 0;
+  p.nkt = 0;
+  p.lse_bh = total_q;
+  p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
+  return launch_result(spa_launch_flash_bwd(p, D, dtype, (hipStream_t)stream), what);
+}
 }  // namespace
 
 extern "C" {
@@ -601,36 +639,21 @@ int spa_flash_bwd_varlen(const void* q, const void* k, const void* v, const void
                          const int64_t k_strides[2], const int64_t v_strides[2], const int64_t do_strides[2],
                          const int64_t dq_strides[2], const int64_t dk_strides[2], const int64_t dv_strides[2],
                          float scale, int mask_mode, int dtype, void* stream) {
-  if (!q || !k || !v || !dout || !lse || !delta || !dq_acc || !dk_acc || !dv_acc)
-    return fail(SPA_EINVAL, "spa_flash_bwd_varlen: null pointer");
-  if (!q_strides || !k_strides || !v_strides || !do_strides || !dq_strides || !dk_strides || !dv_strides)
-    return fail(SPA_EINVAL, "spa_flash_bwd_varlen: null strides");
-  const int rc = varlen_sizes_ok("spa_flash_bwd_varlen", cu_seqlens_q, cu_seqlens_k, nseq, H, total_q, total_k, max_sq,
-                                 max_sk, D, dtype, mask_mode, scale);
-  if (rc != SPA_OK) return rc;
-  const int esz = elem_size(dtype);
-  if (!aligned16v(q, q_strides, esz) || !aligned16v(k, k_strides, esz) || !aligned16v(v, v_strides, esz) ||
-      !aligned16v(dout, do_strides, esz) || !aligned16v(dq_acc, dq_strides, 4) || !aligned16v(dk_acc, dk_strides, 4) ||
-      !aligned16v(dv_acc, dv_strides, 4) || (((uintptr_t)lse | (uintptr_t)delta) & 3) != 0)
-    return fail(SPA_EALIGN, "spa_flash_bwd_varlen: pointers and row strides must be 16-byte aligned");
-  if (!span_ok(max_sq, q_strides[1], D, esz) || !span_ok(max_sk, k_strides[1], D, esz) ||
-      !span_ok(max_sk, v_strides[1], D, esz) || !span_ok(max_sq, do_strides[1], D, esz))
-    return fail(SPA_EUNSUPPORTED, "spa_flash_bwd_varlen: a tensor of one (sequence, head) spans more than 2 GiB");
-  BwdParams p;
-  p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta;
-  p.dq = dq_acc; p.dk = dk_acc; p.dv = dv_acc;
-  p.grads_in_t = 0;
-  p.B = nseq; p.H = H; p.Sq = max_sq; p.Sk = max_sk;
-  p.qs = S2(q_strides); p.ks = S2(k_strides); p.vs = S2(v_strides); p.dos = S2(do_strides);
-  p.dqs = S2(dq_strides); p.dks = S2(dk_strides); p.dvs = S2(dv_strides);
-  p.scale = scale_eff(scale);
-  p.scale_log2 = scale_eff(scale) * 1.4426950408889634f;
-  p.causal = mask_mode == SPA_MASK_CAUSAL;
-  p.nqt = 0;
-  p.nkt = 0;
-  p.lse_bh = total_q;
-  p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
-  return launch_result(spa_launch_flash_bwd(p, D, dtype, (hipStream_t)stream), "spa_flash_bwd_varlen");
+  return flash_bwd_varlen("spa_flash_bwd_varlen", q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, false, cu_seqlens_q,
+                          cu_seqlens_k, nseq, H, total_q, total_k, max_sq, max_sk, D, q_strides, k_strides, v_strides,
+                          do_strides, dq_strides, dk_strides, dv_strides, scale, mask_mode, dtype, stream);
+}
+
+int spa_flash_bwd_varlen_out(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                             const float* delta, void* dq, void* dk, void* dv, const int32_t* cu_seqlens_q,
+                             const int32_t* cu_seqlens_k, int nseq, int H, int total_q, int total_k, int max_sq,
+                             int max_sk, int D, const int64_t q_strides[2], const int64_t k_strides[2],
+                             const int64_t v_strides[2], const int64_t do_strides[2], const int64_t dq_strides[2],
+                             const int64_t dk_strides[2], const int64_t dv_strides[2], float scale, int mask_mode,
+                             int dtype, void* stream) {
+  return flash_bwd_varlen("spa_flash_bwd_varlen_out", q, k, v, dout, lse, delta, dq, dk, dv, true, cu_seqlens_q,
+                          cu_seqlens_k, nseq, H, total_q, total_k, max_sq, max_sk, D, q_strides, k_strides, v_strides,
+                          do_strides, dq_strides, dk_strides, dv_strides, scale, mask_mode, dtype, stream);
 }
 
 }  // extern "C"

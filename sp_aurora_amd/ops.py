@@ -484,27 +484,30 @@ def flash_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
     return out, lse
 
 
-def flash_bwd_varlen(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
-                     max_seqlen_k, softmax_scale=None, causal=False):
-    """Backward of flash_fwd_varlen; adds into the fp32 accumulators dq [total_q,H,D], dk, dv
-    [total_k,H,D].  lse, delta: fp32 [H,total_q].  Calls spa_flash_bwd_varlen."""
+def _flash_bwd_varlen(name, q, k, v, dout, lse, delta, dq, dk, dv, grad_dtype, cu_seqlens_q, cu_seqlens_k,
+                      max_seqlen_q, max_seqlen_k, softmax_scale, causal):
     if not (q.dtype == k.dtype == v.dtype == dout.dtype):
-        raise TypeError("flash_bwd_varlen: q, k, v, dout must share a dtype")
+        raise TypeError(f"{name}: q, k, v, dout must share a dtype")
     (Tq, H, D), _ = _thd(q, "q")
     shp_k, shp_v, shp_do = _thd(k, "k")[0], _thd(v, "v")[0], _thd(dout, "dout")[0]
-    shp_dq, dqs = _thd(dq_acc, "dq_acc")
-    shp_dk, dks = _thd(dk_acc, "dk_acc")
-    shp_dv, dvs = _thd(dv_acc, "dv_acc")
+    shp_dq, dqs = _thd(dq, "dq")
+    shp_dk, dks = _thd(dk, "dk")
+    shp_dv, dvs = _thd(dv, "dv")
     Tk = shp_k[0]
+    # the kernels index the gradients with q's / k's sizes: a mismatch would be an out-of-bounds access
     if shp_k != (Tk, H, D) or shp_v != shp_k or shp_dk != shp_k or shp_dv != shp_k:
-        raise ValueError(f"flash_bwd_varlen: k {shp_k}, v {shp_v}, dk_acc {shp_dk}, dv_acc {shp_dv} must agree (heads and head dim as q {tuple(q.shape)})")
+        raise ValueError(f"{name}: k {shp_k}, v {shp_v}, dk {shp_dk}, dv {shp_dv} must agree (heads and head dim as q {tuple(q.shape)})")
     if shp_do != (Tq, H, D) or shp_dq != (Tq, H, D):
-        raise ValueError(f"flash_bwd_varlen: dout {shp_do} and dq_acc {shp_dq} must have q's shape {tuple(q.shape)}")
-    for t in (dq_acc, dk_acc, dv_acc, lse, delta):
+        raise ValueError(f"{name}: dout {shp_do} and dq {shp_dq} must have q's shape {tuple(q.shape)}")
+    for t in (lse, delta):
         if t.dtype != torch.float32:
-            raise TypeError("accumulators, lse and delta must be float32")
+            raise TypeError(f"{name}: lse and delta must be float32")
+    for t in (dq, dk, dv):
+        if t.dtype != grad_dtype:
+            raise TypeError(f"{name}: dq, dk, dv must be {grad_dtype}")
+    for t in (dq, dk, dv, lse, delta):
         if t.device != q.device:
-            raise ValueError("flash_bwd_varlen: every tensor must live on q's device")
+            raise ValueError(f"{name}: every tensor must live on q's device")
     if tuple(lse.shape) != (H, Tq) or tuple(delta.shape) != (H, Tq) or not lse.is_contiguous() or not delta.is_contiguous():
         raise ValueError("lse and delta must be contiguous [H, total_q]")
     if cu_seqlens_q.numel() != cu_seqlens_k.numel():
@@ -512,16 +515,38 @@ def flash_bwd_varlen(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, cu_seqle
     lib = _lib.load()
     q, k, v, dout = _prep(q), _prep(k), _prep(v), _prep(dout)
     qs, ks, vs, dos = _thd(q, "q")[1], _thd(k, "k")[1], _thd(v, "v")[1], _thd(dout, "dout")[1]
-    if not (_rows_ok(dq_acc, 4) and _rows_ok(dk_acc, 4) and _rows_ok(dv_acc, 4)):
-        raise ValueError("flash_bwd_varlen: accumulators need an inner stride of 1 and 16-byte aligned rows")
+    gsz = dq.element_size()
+    if not (_rows_ok(dq, gsz) and _rows_ok(dk, gsz) and _rows_ok(dv, gsz)):
+        raise ValueError(f"{name}: dq, dk, dv need an inner stride of 1 and 16-byte aligned rows")
     cu_q, cu_k = _cu(cu_seqlens_q, q.device, "cu_seqlens_q"), _cu(cu_seqlens_k, q.device, "cu_seqlens_k")
     if softmax_scale is None:
         softmax_scale = D ** (-0.5)
     with _on(q.device):
-        _lib.check(lib.spa_flash_bwd_varlen(
+        _lib.check(getattr(lib, name)(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(), delta.data_ptr(),
-            dq_acc.data_ptr(), dk_acc.data_ptr(), dv_acc.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), cu_q.data_ptr(), cu_k.data_ptr(),
             cu_q.numel() - 1, H, Tq, Tk, int(max_seqlen_q), int(max_seqlen_k), D,
             _lib.strides2(qs), _lib.strides2(ks), _lib.strides2(vs), _lib.strides2(dos), _lib.strides2(dqs),
             _lib.strides2(dks), _lib.strides2(dvs),
             float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(q), _stream()))
+
+
+def flash_bwd_varlen(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
+                     max_seqlen_k, softmax_scale=None, causal=False):
+    """Backward of flash_fwd_varlen; adds into the fp32 accumulators dq [total_q,H,D], dk, dv
+    [total_k,H,D].  lse, delta: fp32 [H,total_q].  Calls spa_flash_bwd_varlen."""
+    _flash_bwd_varlen("spa_flash_bwd_varlen", q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, torch.float32,
+                      cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, causal)
+
+
+def flash_bwd_varlen_out(q, k, v, dout, lse, delta, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                         softmax_scale=None, causal=False, dq=None, dk=None, dv=None):
+    """Backward of flash_fwd_varlen in one call: returns (dq, dk, dv) in q's dtype, written by the
+    kernels (no fp32 accumulators).  cu_seqlens must cover every row of the packed tensors: rows of
+    no sequence are not written.  Calls spa_flash_bwd_varlen_out."""
+    dq = torch.empty(q.shape, dtype=q.dtype, device=q.device) if dq is None else dq
+    dk = torch.empty(k.shape, dtype=q.dtype, device=q.device) if dk is None else dk
+    dv = torch.empty(v.shape, dtype=q.dtype, device=q.device) if dv is None else dv
+    _flash_bwd_varlen("spa_flash_bwd_varlen_out", q, k, v, dout, lse, delta, dq, dk, dv, q.dtype,
+                      cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, causal)
+    return dq, dk, dv

@@ -37,11 +37,9 @@ class VarlenFlashAttnFunc(torch.autograd.Function):
         max_q, max_k, scale, causal = ctx.args
         # delta = rowsum(dout * out) per (row, head): the packed tensors are one batch of total_q rows
         delta = ops.bwd_delta(out.unsqueeze(0), dout.unsqueeze(0), layout="bshd")[0]
-        dq = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
-        dk = torch.zeros(k.shape, dtype=torch.float32, device=q.device)
-        dv = torch.zeros(v.shape, dtype=torch.float32, device=q.device)
-        ops.flash_bwd_varlen(q, k, v, dout, lse, delta, dq, dk, dv, cu_q, cu_k, max_q, max_k, scale, causal)
-        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None, None, None, None, None
+        # one call computes the whole gradient: the kernels write it in q's dtype
+        dq, dk, dv = ops.flash_bwd_varlen_out(q, k, v, dout, lse, delta, cu_q, cu_k, max_q, max_k, scale, causal)
+        return dq, dk, dv, None, None, None, None, None, None, None
 
 
 def sp_aurora_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k=None, max_seqlen=None, dropout_p=0.0,

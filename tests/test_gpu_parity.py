@@ -390,7 +390,9 @@ def test_backward_matches_autograd_of_full_attention(B, S, H, D, causal, P, dtyp
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("B,Sq,Sk,H,D,causal", [(1, 300, 300, 2, 128, True), (2, 130, 257, 3, 64, False), (1, 64, 64, 1, 32, True),
-                                                (1, 1000, 1000, 2, 128, True)])
+                                                (1, 1000, 1000, 2, 128, True),
+                                                # causal with keys that no query sees: whole tiles of zeros
+                                                (1, 100, 400, 2, 64, True), (2, 130, 300, 1, 128, True)])
 def test_backward_written_in_the_inputs_type_equals_accumulate_then_cast(B, Sq, Sk, H, D, causal, dtype):
     """spa_flash_bwd_out against spa_flash_bwd into zeroed fp32 accumulators followed by the cast
     (sp_aurora/intel_ring_flash_attn.py:250-271): bit for bit, also through strided gradient views."""

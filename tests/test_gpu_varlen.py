@@ -111,6 +111,40 @@ def test_varlen_with_different_query_and_key_lengths_and_empty_sequences(causal)
         k0 += lk
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("D,causal", [(64, True), (128, False), (32, True)])
+def test_varlen_backward_written_in_the_inputs_type_equals_accumulate_then_cast(D, causal, dtype):
+    """spa_flash_bwd_varlen_out against spa_flash_bwd_varlen into zeroed fp32 accumulators followed
+    by the cast, bit for bit, into buffers that start out poisoned: every row of every sequence must
+    be written, with zeros where a sequence has no keys or keys that no query sees."""
+    lens_q = [50, 0, 130, 20, 64, 300]
+    lens_k = [70, 40, 0, 300, 10, 300]
+    H = 2
+    Tq, Tk = sum(lens_q), sum(lens_k)
+    q, dout = (rand((Tq, H, D), 430 + i, dtype).to(DEV) for i in range(2))
+    k, v = (rand((Tk, H, D), 432 + i, dtype).to(DEV) for i in range(2))
+    cu_q, cu_k = cu_of(lens_q).to(DEV), cu_of(lens_k).to(DEV)
+    out, lse = ops.flash_fwd_varlen(q, k, v, cu_q, cu_k, max(lens_q), max(lens_k), None, causal)
+    delta = ops.bwd_delta(out.unsqueeze(0), dout.unsqueeze(0), layout="bshd")[0]
+    acc = [torch.zeros(t.shape, dtype=torch.float32, device=DEV) for t in (q, k, v)]
+    ops.flash_bwd_varlen(q, k, v, dout, lse, delta, *acc, cu_q, cu_k, max(lens_q), max(lens_k), None, causal)
+    want = [a.to(dtype) for a in acc]
+    # gradients written into the halves of packed buffers (row stride 2 H D) that hold a marker value
+    pq = torch.full((Tq, 2, H, D), 7.0, dtype=dtype, device=DEV)
+    pkv = torch.full((Tk, 2, H, D), 7.0, dtype=dtype, device=DEV)
+    ops.flash_bwd_varlen_out(q, k, v, dout, lse, delta, cu_q, cu_k, max(lens_q), max(lens_k), None, causal,
+                             dq=pq[:, 1], dk=pkv[:, 0], dv=pkv[:, 1])
+    for gt, w, name in zip((pq[:, 1], pkv[:, 0], pkv[:, 1]), want, "qkv"):
+        assert torch.equal(gt, w), f"d{name}"
+    assert (pq[:, 0] == 7.0).all()
+    with pytest.raises(TypeError):
+        ops.flash_bwd_varlen_out(q, k, v, dout, lse, delta, cu_q, cu_k, max(lens_q), max(lens_k), None, causal,
+                                 dq=torch.empty(q.shape, dtype=torch.float64, device=DEV))
+    with pytest.raises(ValueError):
+        ops.flash_bwd_varlen_out(q, k, v, dout, lse, delta, cu_q, cu_k, max(lens_q), max(lens_k), None, causal,
+                                 dk=torch.empty_like(k[:1]))
+
+
 def test_varlen_large_batch_matches_the_fixed_length_kernels():
     """Enough workgroups for the shared-buffer forward variant; equal lengths make the padded
     batch call a second opinion, the ragged tail a check that short sequences leave their
