@@ -112,6 +112,12 @@ def test_bad_arguments_return_codes_without_touching_a_device():
     assert lib.spa_flash_bwd_varlen(*bad) == -1
     bad = list(okb); bad[-2] = 9  # dtype
     assert lib.spa_flash_bwd_varlen(*bad) == -1
+    # gradients written in the inputs' type: their rows are 16-byte aligned in that type
+    bad = list(okb); bad[6] = None  # dq
+    assert lib.spa_flash_bwd_varlen_out(*bad) == -1 and b"spa_flash_bwd_varlen_out" in lib.spa_last_error()
+    bad = list(okb); bad[24] = _lib.strides2((64, 68))  # dv rows: 136 bytes in bf16
+    assert lib.spa_flash_bwd_varlen_out(*bad) == -3
+    assert lib.spa_flash_bwd_varlen(*bad) != -3  # 272 bytes as fp32 accumulators: aligned
 
 
 def test_python_wrappers_refuse_cpu_tensors():
@@ -210,6 +216,23 @@ def test_backward_wrappers_check_shapes_before_any_launch():
     for name, t in vbad.items():
         with pytest.raises(ValueError):
             ops.flash_bwd_varlen(**{**vgood, name: t})
+
+    # the same tensors with the gradients written in q's dtype
+    ogood = {k: v for k, v in good.items() if not k.endswith("_acc")}
+    with pytest.raises(ValueError, match="HIP device"):
+        ops.flash_bwd_out(**ogood)
+    for name, t in (("dq", mk(B, Sq - 8, H, D)), ("dk", mk(B, Sk, H + 1, D)), ("dv", mk(B, Sk, H, D, dt=torch.float32)),
+                    ("lse", mk(B, H, Sq + 1, dt=torch.float32))):
+        with pytest.raises(ValueError):
+            ops.flash_bwd_out(**{**ogood, name: t})
+    vogood = {k: v for k, v in vgood.items() if not k.endswith("_acc")}
+    with pytest.raises(ValueError, match="HIP device"):
+        ops.flash_bwd_varlen_out(**vogood)
+    for name, t in (("dq", mk(Tq + 1, H, D)), ("dk", mk(Tk - 8, H, D)), ("delta", mk(H, Tq + 4, dt=torch.float32))):
+        with pytest.raises(ValueError):
+            ops.flash_bwd_varlen_out(**{**vogood, name: t})
+    with pytest.raises(TypeError):
+        ops.flash_bwd_varlen_out(**{**vogood, "dv": mk(Tk, H, D, dt=torch.float32)})
 
 
 def test_cu_seqlens_are_checked_on_the_host():
