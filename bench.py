@@ -15,12 +15,16 @@ The sweep runs through the C entry point spa_ring_fwd in three schedules, same (
   step  one launch per (rank, ring step), the running (out, lse) in HBM, the update_out_and_lse
         merge in the kernel's epilogue: what a rank runs while chunks arrive over the wire.
 `other_schedules` holds rank and step; `ring_step` repeats the step figure as the per-ring-step
-number.
+number; `roofline` carries both again as `rank_tflops` / `step_tflops`.  The line is kept below
+7.5 KB (long texts live in this docstring and in ROW_NOTES, not in the line), with `rows` ahead of
+`other_schedules`, `ring_step` and `protocol`, so that a reader who keeps only the end of the
+output still has them; the host's core counts appear once, as `host`.
 
-Timing protocol.  (1) settle: the same launch repeated until 10 consecutive launches agree within
-2 % or 0.3 s have passed (after an idle period the first ~40 launches run 5-25 % slower while the
-power management answers the load step; reported as `settle_launches`, `settle_ms`,
-`cold_ms_per_step` = mean of the first 5 launches).  (2) `--warmup` untimed steps.  (3) the timed
+Timing protocol.  (1) settle: the same launch repeated in groups of 10 until the median of a group
+is within 2 % of the median of the group before it (40 launches at least), or 0.3 s have passed (after an idle period the
+first ~40 launches run 5-25 % slower while the power management answers the load step; reported
+as `settle_launches`, `settle_ms`, `settle_ended_by` = "converged" or "cap", `cold_ms_per_step` =
+mean of the first 5 launches).  (2) `--warmup` untimed steps.  (3) the timed
 region: blocks of exactly `--steps` steps, each block bracketed by events on the launch stream and
 a synchronize, repeated until >= 0.2 s are covered; `ms_per_step` is the MEDIAN block
 (`timed_blocks`, `block_ms_min`, `block_ms_max` beside it).
@@ -109,11 +113,14 @@ def timed_block(torch, fn, iters):
     return start.elapsed_time(end) / iters
 
 
-def settle(torch, fn, max_s=0.3, need=10, tol=0.02):
-    """Repeats fn until `need` consecutive launches agree within `tol`, or max_s have passed.
-    Returns (launches, ms spent, mean ms of the first 5 launches)."""
+def settle(torch, fn, max_s=0.3, need=10, tol=0.02, min_launches=40):
+    """Repeats fn in groups of `need` launches until the median of a group is within `tol` of the
+    median of the group before it (and at least min_launches have run: the slow stretch after an
+    idle period lasts about 30), or max_s have passed.
+    Returns (launches, ms spent, mean ms of the first 5 launches, "converged" | "cap")."""
     t0 = time.perf_counter()
     times = []
+    prev = None
     while True:
         chunk = []
         for _ in range(need):
@@ -124,20 +131,26 @@ def settle(torch, fn, max_s=0.3, need=10, tol=0.02):
             b.record()
             chunk.append((a, b))
         torch.cuda.synchronize()
-        times += [a.elapsed_time(b) for a, b in chunk]
-        last = times[-need:]
+        last = [a.elapsed_time(b) for a, b in chunk]
+        times += last
+        med = statistics.median(last)
         spent = time.perf_counter() - t0
-        if max(last) <= min(last) * (1.0 + tol) or spent >= max_s:
+        if prev is not None and len(times) >= min_launches and abs(med - prev) <= tol * prev:
+            ended = "converged"
             break
-    return len(times), spent * 1e3, sum(times[:5]) / min(5, len(times))
+        if spent >= max_s:
+            ended = "cap"
+            break
+        prev = med
+    return len(times), spent * 1e3, sum(times[:5]) / min(5, len(times)), ended
 
 
 def measure(torch, fn, steps, warmup, min_s=MIN_TIMED_S, do_settle=True):
     """The protocol of the module docstring for one callable.  Returns a dict."""
     res = {}
     if do_settle:
-        n, ms, cold = settle(torch, fn)
-        res.update(settle_launches=n, settle_ms=round(ms, 2), cold_ms_per_step=round(cold, 4))
+        n, ms, cold, ended = settle(torch, fn)
+        res.update(settle_launches=n, settle_ms=round(ms, 2), settle_ended_by=ended, cold_ms_per_step=round(cold, 4))
     for _ in range(warmup):
         fn()
     blocks = []
@@ -196,7 +209,14 @@ def cpu_time(fn, warm=2, timed=5):
 
 class CpuLegs:
     """The reference's op sequence per row on the host cores (oracle restatements, fp32 torch;
-    bf16 inputs are up-cast to fp32: no fast bf16 GEMM is assumed on the host)."""
+    bf16 inputs are up-cast to fp32: no fast bf16 GEMM is assumed on the host).  `sample` texts are
+    short on purpose (the whole line must stay below 7.5 KB); what each leg runs:
+      pairs   one diagonal and one full block pair [B,H,s,D] through torch CPU SDPA plus a second
+              q k^T / logsumexp for the lse, median of 5 after 2 warm-up, extrapolated to the row's
+              pair counts (d = diagonal, f = full)
+      full    the row's whole workload, median of 5 (re-layout: of 3)
+      backward  the same pairs through torch CPU autograd of softmax(q k^T) v (forward recompute
+              included, as in the reference), median of 3, 5-GEMM FLOP count"""
 
     def __init__(self, torch):
         from oracle import attn_oracle as O
@@ -207,7 +227,7 @@ class CpuLegs:
         self._pair_cache = {}
 
     def _entry(self, value, unit, sample, kind="port"):
-        return {"value": value, "unit": unit, "cores": self.threads, "kind": kind, "sample": sample, "host": self.host}
+        return {"value": float(f"{value:.4g}"), "unit": unit, "cores": self.threads, "kind": kind, "sample": sample}
 
     def pair_times(self, Bn, Hn, sn, Dn, seed):
         """seconds for one diagonal and one full block pair [Bn,Hn,sn,Dn] (SDPA + second QK^T/logsumexp)."""
@@ -219,23 +239,20 @@ class CpuLegs:
             self._pair_cache[key] = (cpu_time(lambda: f(True)), cpu_time(lambda: f(False)))
         return self._pair_cache[key]
 
-    def ring_forward(self, Bn, Hn, sn, Dn, n_diag, n_full, seed, what):
+    def ring_forward(self, Bn, Hn, sn, Dn, n_diag, n_full, seed):
         """Extrapolation from one measured diagonal and one measured full pair."""
         t_d, t_f = self.pair_times(Bn, Hn, sn, Dn, seed)
         full = 4.0 * Bn * Hn * sn * sn * Dn
         flops = n_full * full + n_diag * full / 2
         secs = n_diag * t_d + n_full * t_f
         return self._entry(flops / secs / 1e12, "TFLOP/s",
-                           f"{what}: measured 1 diagonal ({t_d * 1e3:.1f} ms) + 1 full ({t_f * 1e3:.1f} ms) block pair "
-                           f"[B{Bn},H{Hn},s{sn},D{Dn}] (median of 5 after 2 warm-up), extrapolated to {n_diag} diagonal + "
-                           f"{n_full} full pairs = {secs * 1e3:.0f} ms; bf16 inputs up-cast to fp32, torch CPU SDPA + second QK^T/logsumexp")
+                           f"pairs [B{Bn},H{Hn},s{sn},D{Dn}]: 1 d {t_d * 1e3:.0f} ms + 1 f {t_f * 1e3:.0f} ms measured, x {n_diag} d + {n_full} f = {secs * 1e3:.0f} ms")
 
     def config1(self):
         torch, O = self.torch, self.O
         q, k, v = rand_tensors(torch, (1, 8, 512, 64), 0, 3, 1.0, torch.float32)
         t = cpu_time(lambda: O.attn_block_sdpa(q, k, v, 0.125, False, compute_dtype=torch.float32))
-        return self._entry(4.0 * 8 * 512 * 512 * 64 / t / 1e12, "TFLOP/s",
-                           f"config 1 in full: fp32 [1,8,512,64] non-causal, SDPA + second QK^T/logsumexp, {t * 1e3:.2f} ms (median of 5)")
+        return self._entry(4.0 * 8 * 512 * 512 * 64 / t / 1e12, "TFLOP/s", f"full: {t * 1e3:.2f} ms")
 
     def config2(self):
         """Rank 2 of the P=4 ring in full: 3 block pairs + 1 init, 2 merges (sigmoid / logsigmoid form)."""
@@ -257,9 +274,7 @@ class CpuLegs:
 
         t = cpu_time(run)
         flops = 2.5 * 4.0 * Bn * Hn * sn * sn * Dn
-        return self._entry(flops / t / 1e12, "TFLOP/s",
-                           f"config 2 in full: rank 2 of P=4, [B2,H32,s1024,D64], 1 diagonal + 2 full pairs + merges, {t * 1e3:.0f} ms (median of 5); "
-                           "bf16 inputs up-cast to fp32")
+        return self._entry(flops / t / 1e12, "TFLOP/s", f"full (3 pairs + merges): {t * 1e3:.0f} ms")
 
     def relayout(self):
         torch, O = self.torch, self.O
@@ -269,9 +284,8 @@ class CpuLegs:
         ys = O.all_to_all_4d_s2h(xs)
         t_h2s = cpu_time(lambda: O.all_to_all_4d_h2s(ys), 1, 3)
         nbytes = 2 * x.numel() * 2
-        mk = lambda t, d: self._entry(nbytes / t / 1e9, "GB/s", f"config 4 tensor [8,1,2048,32,128] bf16 in full, {d}: the reference's "
-                                      f"reshape/transpose/contiguous chains around the exchange, {t * 1e3:.0f} ms (median of 3)")
-        return mk(t_s2h, "s2h"), mk(t_h2s, "h2s")
+        mk = lambda t: self._entry(nbytes / t / 1e9, "GB/s", f"full (reshape/transpose/contiguous chain): {t * 1e3:.0f} ms")
+        return mk(t_s2h), mk(t_h2s)
 
     def merge(self):
         torch, O = self.torch, self.O
@@ -281,8 +295,7 @@ class CpuLegs:
         blk = torch.randn((1, 32, 1024, 128), generator=g).to(torch.bfloat16)
         bl = torch.randn((1, 32, 1024, 1), generator=g)
         t = cpu_time(lambda: O.merge(acc, lse, blk.float(), bl))
-        return self._entry((acc.numel() * 10 + lse.numel() * 12) / t / 1e9, "GB/s",
-                           f"one config-3 chunk [1,32,1024,128]: sigmoid / logsigmoid merge of a bf16 block into fp32 (out, lse), {t * 1e3:.1f} ms (median of 5)")
+        return self._entry((acc.numel() * 10 + lse.numel() * 12) / t / 1e9, "GB/s", f"full (sigmoid/logsigmoid form): {t * 1e3:.1f} ms")
 
     def backward(self, n_diag, n_full):
         torch, O = self.torch, self.O
@@ -293,17 +306,71 @@ class CpuLegs:
         full = 2.5 * 4.0 * 16 * 2048 * 2048 * 128
         secs = n_diag * t_d + n_full * t_f
         return self._entry((n_full * full + n_diag * full / 2) / secs / 1e12, "TFLOP/s",
-                           f"config 5 backward: measured 1 diagonal ({t_d * 1e3:.0f} ms) + 1 full ({t_f * 1e3:.0f} ms) block pair [1,2048,16,128] "
-                           f"through torch CPU autograd of softmax(QK^T)V (forward recompute included, as in the reference), median of 3, "
-                           f"extrapolated to {n_diag} + {n_full} pairs = {secs:.1f} s; 5-GEMM FLOP count; bf16 up-cast to fp32")
+                           f"backward pairs [1,2048,16,128]: 1 d {t_d * 1e3:.0f} ms + 1 f {t_f * 1e3:.0f} ms measured, x {n_diag} d + {n_full} f = {secs:.1f} s")
 
 
 # ------------------------------------------------------------------------------------ rows
-def roof(bound, kernel, achieved, peak, unit, **extra):
-    r = {"bound": bound, "kernel": kernel, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-         "frac": round(achieved / peak, 4), "traffic": None}
-    r.update(extra)
-    return r
+# What each row of `rows` runs (the line itself carries a short `workload` only).
+ROW_NOTES = {
+    "config1_fp32_block_forward": "config 1: fp32 B=1 S=512 H=8 D=64 non-causal block forward, out + lse (flash_fwd32_kernel<64>)",
+    "config2_ring_rank2_of_4": "config 2: bf16 B=2 S=4096 (P=4 chunks of 1024) H=32 D=64 causal, rank 2: diagonal chunk 2, then chunks 1, 0, "
+                               "merged; value = one launch for the rank, step_tflops = one launch per ring step (3 launches)",
+    "config3_zigzag_ring": "config 3 tensors with zigzag sharding (rank r holds half-chunks r and 15-r): every rank runs 1 diagonal "
+                           "block [1024 x 1024], r blocks [1024 x 512] and 7-r blocks [512 x 1024]; same 549.76 GFLOP; value = one launch "
+                           "per rank, step_tflops = one launch per (rank, step)",
+    "config4_relayout_s2h": "config 4 re-layout: [P=8,B=1,s=2048,H=32,D=128] bf16 -> [8,1,16384,4,128], one tensor per launch, q / k / v in "
+                            "turn (nothing cache-resident), recorded calls replayed (ops.prepared); host cost of the call included",
+    "config4_relayout_h2s": "the inverse of config4_relayout_s2h",
+    "config4_ulysses_forward": "config 4: 3 re-layouts in, full causal attention per head group [8,1,16384,4,128], 1 re-layout out, output "
+                               "allocation included; views_tflops = the same result with head groups read and written in place (B = 1)",
+    "block_forward_fp8_kv": "causal block forward over the config-3 sequence, bf16 q [1,8192,32,128], K / V e4m3 + fp32 scale per (batch, "
+                            "head), one call; bf16_kv_tflops = the same call with bf16 K / V",
+    "merge_update_out_and_lse": "update_out_and_lse: merge of a bf16 block into the fp32 running (out, lse) of one config-3 rank "
+                                "[1,1024,32,128], 8 operand sets in turn, recorded calls replayed; host cost of the call included",
+    "config5_ring_forward": "config 5 forward: bf16 qkv [1,32768,3,16,128] (strided views) causal, ring of 16 chunks of 2048, 16 diagonal + "
+                            "120 full pairs; value = schedule all, rank_tflops / step_tflops = 16 / 136 launches",
+    "config5_ring_backward": "config 5 backward: dq/dk/dv by block-wise recompute with the global lse over the same 136 block pairs, one launch "
+                             "per kernel, delta pre-pass and output allocation included, gradients written in bf16 (spa_flash_bwd_out); "
+                             "5-GEMM FLOP count (the two kernels execute 7); step_tflops = one launch pair per block pair into fp32 "
+                             "accumulators (spa_flash_bwd), zero-fill and final casts included",
+}
+
+# name -> (short workload text, unit, roofline bound, kernel, peak, extra config keys)
+ROW_SPECS = {
+    "config1_fp32_block_forward": ("config 1: fp32 [1,512,8,64] block forward", "TFLOP/s", "mfma", "flash_fwd32<64>", MFMA_F32_PEAK_TFLOPS, ()),
+    "config2_ring_rank2_of_4": ("config 2: bf16 D=64, rank 2 of P=4, 1 launch", "TFLOP/s", "mfma", "flash_fwd16<bf16,64>", MFMA_BF16_PEAK_TFLOPS,
+                                ("step_tflops",)),
+    "config3_zigzag_ring": ("config 3, zigzag shards, 1 launch per rank", "TFLOP/s", "mfma", "flash_fwd16<bf16,128>", MFMA_BF16_PEAK_TFLOPS,
+                            ("step_tflops", "all_tflops")),
+    "config4_relayout_s2h": ("config 4 re-layout s2h, 268 MB per launch", "GB/s", "hbm", "relayout<16,s2h>", HBM_PEAK_GBPS, ()),
+    "config4_relayout_h2s": ("config 4 re-layout h2s, 268 MB per launch", "GB/s", "hbm", "relayout<16,h2s>", HBM_PEAK_GBPS, ()),
+    "config4_ulysses_forward": ("config 4: 3 re-layouts, attention, 1 re-layout", "TFLOP/s", "mfma", "relayout x4 + flash_fwd16<bf16,128>",
+                                MFMA_BF16_PEAK_TFLOPS, ("views_tflops",)),
+    "block_forward_fp8_kv": ("causal block forward [1,8192,32,128], e4m3 K/V", "TFLOP/s", "mfma", "flash_fwd16<bf16,128,e4m3 K/V>",
+                             MFMA_BF16_PEAK_TFLOPS, ("bf16_kv_tflops",)),
+    "merge_update_out_and_lse": ("merge of a bf16 block [1,1024,32,128] into fp32 (out, lse), 42.3 MB", "GB/s", "hbm", "merge<bf16>",
+                                 HBM_PEAK_GBPS, ()),
+    "config5_ring_forward": ("config 5 forward, P=16, 1 launch", "TFLOP/s", "mfma", "flash_fwd16<bf16,128>", MFMA_BF16_PEAK_TFLOPS,
+                             ("rank_tflops", "step_tflops")),
+    "config5_ring_backward": ("config 5 backward, 1 launch per kernel, 5-GEMM count", "TFLOP/s", "mfma", "flash_bwd_dq + flash_bwd_dkdv",
+                              MFMA_BF16_PEAK_TFLOPS, ("step_tflops",)),
+}
+
+
+def make_row(name, ms_per_step, value, **extra):
+    """One entry of `rows` (without cpu_baseline) from the table above."""
+    workload, unit, bound, kernel, peak, keys = ROW_SPECS[name]
+    if set(extra) != set(keys):
+        raise KeyError(f"{name}: expected extras {keys}, got {sorted(extra)}")
+    cfg = {"workload": workload}
+    cfg.update({k2: round(v2, 2) for k2, v2 in extra.items()})
+    return {"row": name, "value": round(value, 2), "unit": unit, "ms_per_step": round(ms_per_step, 4), "config": cfg,
+            "roofline": {"bound": bound, "kernel": kernel, "achieved": round(value, 2), "peak": peak, "unit": unit,
+                         "frac": round(value / peak, 4), "traffic": None}}
+
+
+def tfl(flops, m):
+    return flops / (m["ms_per_step"] * 1e-3) / 1e12
 
 
 def gpu_rows(torch, spa, ops, which, steps, warmup):
@@ -312,9 +379,8 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
     rows = {}
     light = dict(min_s=0.05, do_settle=False)
 
-    def finish(name, m, config, value, unit, roofline):
-        rows[name] = {"row": name, "value": round(value, 2), "unit": unit, "ms_per_step": round(m["ms_per_step"], 4),
-                      "timed_blocks": m["timed_blocks"], "config": config, "roofline": roofline}
+    def finish(name, m, value, **extra):
+        rows[name] = make_row(name, m["ms_per_step"], value, **extra)
 
     if "config1" in which:
         q, k, v = rand_tensors(torch, (1, 512, 8, 64), 0, 3, 1.0, torch.float32, dev)
@@ -322,9 +388,8 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
         lse = torch.empty((1, 8, 512), dtype=torch.float32, device=dev)
         fn = lambda: ops.flash_fwd(q, k, v, 0.125, False, layout="bshd", out=out, lse=lse)
         m = measure(torch, fn, 20, 5, **light)
-        tf = 4.0 * 8 * 512 * 512 * 64 / (m["ms_per_step"] * 1e-3) / 1e12
-        finish("config1_fp32_block_forward", m, {"workload": "config 1: fp32 B=1 S=512 H=8 D=64 non-causal block forward, out + lse"},
-               tf, "TFLOP/s", roof("mfma", "flash_fwd32_kernel<64>", tf, MFMA_F32_PEAK_TFLOPS, "TFLOP/s"))
+        tf = tfl(4.0 * 8 * 512 * 512 * 64, m)
+        finish("config1_fp32_block_forward", m, tf)
     if "config2" in which:
         Bn, Sn, Hn, Dn, Pn, r = 2, 4096, 32, 64, 4, 2
         q, k, v = rand_tensors(torch, (Bn, Sn, Hn, Dn), 1, 3, 1.0, torch.bfloat16, dev)
@@ -337,13 +402,22 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
             fn = lambda fuse=fuse: ops.ring_fwd(q, k, v, Pn, None, True, rank=r, out=out, lse=lse, workspace=ws, fuse=fuse)
             sched[fuse] = measure(torch, fn, 20, 5, **light)
         m = sched["rank"]
-        tf = flops / (m["ms_per_step"] * 1e-3) / 1e12
-        tf_step = flops / (sched["step"]["ms_per_step"] * 1e-3) / 1e12
-        finish("config2_ring_rank2_of_4", m,
-               {"workload": "config 2: bf16 B=2 S=4096 (P=4 chunks of 1024) H=32 D=64 causal, rank 2: diagonal chunk 2, then chunks 1, 0, merged",
-                "flops_per_step": flops, "one_launch_per_ring_step": {"ms_per_step": round(sched["step"]["ms_per_step"], 4), "tflops": round(tf_step, 2),
-                                                                        "launches_per_step": 3}},
-               tf, "TFLOP/s", roof("mfma", "flash_fwd16_kernel<bf16,64,2>", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", launches_per_step=1))
+        tf = tfl(flops, m)
+        finish("config2_ring_rank2_of_4", m, tf, step_tflops=tfl(flops, sched["step"]))
+    if "zigzag" in which and hasattr(spa.ring, "zigzag_order"):
+        q, k, v = rand_tensors(torch, (B, S, H, D), SEED, 3, INPUT_SCALE, torch.bfloat16, dev)
+        order = spa.ring.zigzag_order(S, P, dev)
+        q, k, v = [t.index_select(1, order).contiguous() for t in (q, k, v)]
+        total, _, _ = sweep_flops()
+        sched = {}
+        for fuse in ("step", "rank", "all"):
+            f = spa.ring.make_ring_forward_step(q, k, v, D ** -0.5, True, P, fuse=fuse, sharding="zigzag")
+            f()
+            sched[fuse] = measure(torch, f, 20, 5, **light)
+        m = sched["rank"]
+        tf = tfl(total, m)
+        finish("config3_zigzag_ring", m, tf, step_tflops=tfl(total, sched["step"]), all_tflops=tfl(total, sched["all"]))
+        del q, k, v
     if "config4" in which:
         Pn, Bn, sn, Hn, Dn = 8, 1, 2048, 32, 128
         q, k, v = rand_tensors(torch, (Pn, Bn, sn, Hn, Dn), 3, 3, 1.0, torch.bfloat16, dev)
@@ -367,14 +441,10 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
             i = turn[0] = (turn[0] + 1) % 3
             h2s_runs[i]()
 
-        for name, fn, kern in (("s2h", s2h, "relayout_kernel<16,s2h>"), ("h2s", h2s, "relayout_kernel<16,h2s>")):
+        for name, fn in (("s2h", s2h), ("h2s", h2s)):
             m = measure(torch, fn, 21, 6, **light)
             gb = nbytes / (m["ms_per_step"] * 1e-3) / 1e9
-            finish(f"config4_relayout_{name}", m,
-                   {"workload": f"config 4 re-layout {name}: [P=8,B=1,s=2048,H=32,D=128] bf16 <-> [8,1,16384,4,128], one tensor and one direction per "
-                                "launch, q / k / v in turn, recorded calls replayed (ops.prepared)",
-                    "bytes_per_launch": nbytes, "includes": "host cost of the call (event-timed back to back); kernel-only time is in profiles/"},
-                   gb, "GB/s", roof("hbm", kern, gb, HBM_PEAK_GBPS, "GB/s"))
+            finish(f"config4_relayout_{name}", m, gb)
         y = ys[0]
         del ys, backs
         scale = Dn ** -0.5
@@ -382,17 +452,12 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
         fn()
         m = measure(torch, fn, 5, 2, **light)
         flops = 4.0 * Bn * Hn * (Pn * sn) ** 2 * Dn / 2
-        tf = flops / (m["ms_per_step"] * 1e-3) / 1e12
+        tf = tfl(flops, m)
         # the same result with head groups read and written in place (B = 1: no re-layout pass at all)
         fv = lambda: spa.intel_ulysses_flash_attn_forward(None, q, k, v, scale, causal=True, relayout="views")
         fv()
         mv = measure(torch, fv, 5, 2, **light)
-        finish("config4_ulysses_forward", m,
-               {"workload": "config 4: q,k,v [P=8,B=1,s=2048,H=32,D=128] bf16 -> head-sharded [8,1,16384,4,128], full causal attention per head group, "
-                            "inverse re-layout of out (3 re-layouts in, attention, 1 out; output allocation included)", "flops_per_step": flops,
-                "same_result_through_strided_views": {"ms_per_step": round(mv["ms_per_step"], 4),
-                                                      "tflops": round(flops / (mv["ms_per_step"] * 1e-3) / 1e12, 2)}},
-               tf, "TFLOP/s", roof("mfma", "relayout_kernel x4 + flash_fwd16_kernel<bf16,128,2>", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
+        finish("config4_ulysses_forward", m, tf, views_tflops=tfl(flops, mv))
         del q, k, v, y, xs
     if "fp8kv" in which:
         # the config-3 sequence as one causal block call, K / V in e4m3 with per-head scales, against
@@ -408,12 +473,8 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
         f16 = lambda: ops.flash_fwd(q, k, v, None, True, out=out, lse=lse)
         m16 = measure(torch, f16, 20, 5, **light)
         m = measure(torch, f8, 20, 5, **light)
-        tf = flops / (m["ms_per_step"] * 1e-3) / 1e12
-        finish("block_forward_fp8_kv", m,
-               {"workload": "causal block forward over the config-3 sequence (bf16 q [1,8192,32,128], K / V e4m3 + fp32 scale per (batch, head)), one call",
-                "flops_per_step": flops, "same_call_with_bf16_kv": {"ms_per_step": round(m16["ms_per_step"], 4),
-                                                                     "tflops": round(flops / (m16["ms_per_step"] * 1e-3) / 1e12, 2)}},
-               tf, "TFLOP/s", roof("mfma", "flash_fwd16_kernel<bf16,128,2,e4m3 K/V>", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
+        tf = tfl(flops, m)
+        finish("block_forward_fp8_kv", m, tf, bf16_kv_tflops=tfl(flops, m16))
         del q, k, v, k8, v8
     if "merge" in which:
         Bn, sn, Hn, Dn = 1, 1024, 32, 128
@@ -435,11 +496,7 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
         m = measure(torch, fn, 24, 8, **light)
         nbytes = Bn * sn * Hn * Dn * 10 + Bn * Hn * sn * 12
         gb = nbytes / (m["ms_per_step"] * 1e-3) / 1e9
-        finish("merge_update_out_and_lse", m,
-               {"workload": "update_out_and_lse: merge of a bf16 block into the fp32 running (out, lse) of one config-3 rank [1,1024,32,128], "
-                            "8 operand sets in turn, recorded calls replayed (ops.prepared)",
-                "bytes_per_launch": nbytes, "includes": "host cost of the call (event-timed back to back); kernel-only time is in profiles/"},
-               gb, "GB/s", roof("hbm", "merge_kernel<bf16>", gb, HBM_PEAK_GBPS, "GB/s"))
+        finish("merge_update_out_and_lse", m, gb)
         del sets
     if "config5" in which:
         Bn, Sn, Hn, Dn, Pn = 1, 32768, 16, 128, 16
@@ -451,29 +508,23 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
         out, lse = fstep()
         m = measure(torch, fstep, 3, 1, **light)
         fwd_flops = 4.0 * Bn * Hn * Sn * Sn * Dn / 2
-        tf = fwd_flops / (m["ms_per_step"] * 1e-3) / 1e12
+        tf = tfl(fwd_flops, m)
         sched5 = {}
-        for fuse, launches in (("rank", Pn), ("step", Pn * (Pn + 1) // 2)):
+        for fuse in ("rank", "step"):
             f5 = spa.ring.make_ring_forward_step(q, k, v, scale, True, Pn, fuse=fuse)
             f5()
-            mm = measure(torch, f5, 3, 1, **light)
-            sched5[fuse] = {"ms_per_step": round(mm["ms_per_step"], 4), "tflops": round(fwd_flops / (mm["ms_per_step"] * 1e-3) / 1e12, 2),
-                            "launches_per_step": launches}
+            sched5[fuse] = tfl(fwd_flops, measure(torch, f5, 3, 1, **light))
             del f5
-        finish("config5_ring_forward", m,
-               {"workload": "config 5 forward: bf16 qkv [1,32768,3,16,128] (strided views) causal, ring of 16 chunks of 2048, 16 diagonal + 120 full pairs, schedule 'all'",
-                "flops_per_step": fwd_flops, "other_schedules": sched5},
-               tf, "TFLOP/s", roof("mfma", "flash_fwd16_kernel<bf16,128,2>", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s", launches_per_step=1))
+        finish("config5_ring_forward", m, tf, rank_tflops=sched5["rank"], step_tflops=sched5["step"])
         fn = lambda: spa.ring.ring_flash_attn_backward(dout, q, k, v, out, lse, scale, True, Pn, fuse="all")
         fn()
         m = measure(torch, fn, 3, 1, **light)
         bwd_flops = 2.5 * fwd_flops
-        tf = bwd_flops / (m["ms_per_step"] * 1e-3) / 1e12
-        finish("config5_ring_backward", m,
-               {"workload": "config 5 backward: dq/dk/dv by block-wise recompute with the global lse over the same 136 block pairs, one launch per kernel "
-                            "(delta pre-pass and output allocation included; the kernels write the gradients in bf16: spa_flash_bwd_out); 5-GEMM FLOP count (the two kernels execute 7)",
-                "flops_per_step": bwd_flops},
-               tf, "TFLOP/s", roof("mfma", "flash_bwd_dq_kernel + flash_bwd_dkdv_kernel", tf, MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"))
+        tf = tfl(bwd_flops, m)
+        fs = lambda: spa.ring.ring_flash_attn_backward(dout, q, k, v, out, lse, scale, True, Pn, fuse="step")
+        fs()
+        ms_ = measure(torch, fs, 2, 1, **light)
+        finish("config5_ring_backward", m, tf, step_tflops=tfl(bwd_flops, ms_))
         del qkv, dout, out, lse
     torch.cuda.empty_cache()
     return rows
@@ -485,19 +536,22 @@ def attach_cpu(rows, cpu):
         rows["config1_fp32_block_forward"]["cpu_baseline"] = cpu.config1()
     if "config2_ring_rank2_of_4" in rows:
         rows["config2_ring_rank2_of_4"]["cpu_baseline"] = cpu.config2()
+    if "config3_zigzag_ring" in rows:
+        # the same 36 block pairs' worth of work as config 3 (zigzag only reorders them)
+        rows["config3_zigzag_ring"]["cpu_baseline"] = cpu.ring_forward(B, H, S // P, D, P, P * (P - 1) // 2, SEED)
     if "config4_relayout_s2h" in rows:
         a, b = cpu.relayout()
         rows["config4_relayout_s2h"]["cpu_baseline"] = a
         rows["config4_relayout_h2s"]["cpu_baseline"] = b
-        rows["config4_ulysses_forward"]["cpu_baseline"] = cpu.ring_forward(
-            1, 4, 2048, 128, 8, 28, 3, "config 4 attention of one head group [1,4,16384,128] as 2048-row blocks (x 8 groups: same ratio); re-layouts not included")
+        # attention of one head group [1,4,16384,128] as 2048-row blocks (x 8 groups: same ratio); re-layouts not included
+        rows["config4_ulysses_forward"]["cpu_baseline"] = cpu.ring_forward(1, 4, 2048, 128, 8, 28, 3)
     if "block_forward_fp8_kv" in rows:
-        rows["block_forward_fp8_kv"]["cpu_baseline"] = cpu.ring_forward(
-            1, 32, 1024, 128, 8, 28, SEED, "the same attention with dequantised K / V as 1024-row blocks (the reference has no 8-bit path)")
+        # the same attention with dequantised K / V as 1024-row blocks (the reference has no 8-bit path)
+        rows["block_forward_fp8_kv"]["cpu_baseline"] = cpu.ring_forward(1, 32, 1024, 128, 8, 28, SEED)
     if "merge_update_out_and_lse" in rows:
         rows["merge_update_out_and_lse"]["cpu_baseline"] = cpu.merge()
     if "config5_ring_forward" in rows:
-        rows["config5_ring_forward"]["cpu_baseline"] = cpu.ring_forward(1, 16, 2048, 128, 16, 120, 4, "config 5 forward")
+        rows["config5_ring_forward"]["cpu_baseline"] = cpu.ring_forward(1, 16, 2048, 128, 16, 120, 4)
         rows["config5_ring_backward"]["cpu_baseline"] = cpu.backward(16, 120)
 
 
@@ -605,7 +659,63 @@ def pmc_summary(fetch_dir, write_dir):
 
 # ------------------------------------------------------------------------------------ main
 ROW_SETS = {"fp8kv": {"fp8kv"}, "relayout": {"config4"}, "ulysses": {"config4"}, "merge": {"merge"}, "backward": {"config5"},
-            "config1": {"config1"}, "config2": {"config2"}}
+            "config1": {"config1"}, "config2": {"config2"}, "zigzag": {"zigzag"}}
+ALL_ROWS = {"config1", "config2", "zigzag", "config4", "fp8kv", "merge", "config5"}
+LINE_LIMIT = 7500  # bytes of the printed line: readers that keep only the end of the output keep 8 KB
+
+
+def assemble_line(steps, warmup, head, m_head, other, rows, cpu_head, host, traffic, traffic_src):
+    """The JSON line from the measurements (a pure function: tests build it from made-up numbers).
+    Key order matters: `rows` come before `other_schedules`, `ring_step` and `protocol`."""
+    total_flops, n_pairs, _ = sweep_flops()
+    ms = m_head["ms_per_step"]
+    tflops = total_flops / (ms * 1e-3) / 1e12
+    launches = {"all": 1, "rank": P, "step": n_pairs}[head]
+    roofline = {
+        "bound": "mfma", "kernel": "flash_fwd16_kernel<bf16,128,2>", "achieved": round(tflops, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+        "unit": "TFLOP/s", "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": traffic, "traffic_source": traffic_src,
+        "avg_launch_us": round(ms * 1e3 / launches, 2), "flops_per_launch": total_flops / launches, "launches_per_step": launches,
+        "algorithmic_bytes_per_launch": algorithmic_bytes() / launches,
+    }
+    for name in ("rank", "step"):
+        if name in other:
+            roofline[name + "_tflops"] = other[name]["tflops"]
+            roofline[name + "_frac"] = round(other[name]["tflops"] / MFMA_BF16_PEAK_TFLOPS, 4)
+    line = {
+        "metric": "fwd attn TFLOP/s + % bf16 MFMA peak, ring-step causal S=8K H32 D128",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"config 3: simulated ring P=8, bf16 [1,8192,32,128] causal, 8 diagonal + 28 full block pairs, schedule '{head}'",
+            "flops_per_step": total_flops,
+            "block_pairs": n_pairs,
+        },
+        "pct_of_bf16_mfma_peak": round(100.0 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
+        "roofline": roofline,
+    }
+    if cpu_head is not None:
+        line["cpu_baseline"] = cpu_head
+    if host is not None:
+        line["host"] = host
+    if rows:
+        line["rows"] = list(rows.values())
+    line["other_schedules"] = other
+    if "step" in other:
+        line["ring_step"] = {"what": "one launch per (rank, ring step), merge in the last step's epilogue",
+                             "tflops": other["step"]["tflops"], "pct_of_bf16_mfma_peak": other["step"]["pct_of_bf16_mfma_peak"],
+                             "avg_launch_us": other["step"]["avg_launch_us"]}
+    line["protocol"] = {k2: m_head[k2] for k2 in ("settle_launches", "settle_ms", "settle_ended_by", "cold_ms_per_step", "timed_blocks",
+                                                  "block_ms_min", "block_ms_max", "timed_region_s") if k2 in m_head}
+    return line
 
 
 def main():
@@ -658,9 +768,7 @@ def main():
     # preallocated buffers, no allocation per step
     steps = {m: spa.ring.make_ring_forward_step(q, k, v, scale, True, P, fuse=m) for m in ("all", "rank", "step")}
     head = args.schedule if args.only_all else "all"
-    m_all = measure(torch, steps[head], args.steps, args.warmup)
-    ms = m_all["ms_per_step"]
-    tflops = total_flops / (ms * 1e-3) / 1e12
+    m_head = measure(torch, steps[head], args.steps, args.warmup)
 
     other = {}
     if not args.only_all:
@@ -670,7 +778,7 @@ def main():
             launches = P if name == "rank" else n_pairs
             other[name] = {"ms_per_step": round(t, 4), "tflops": round(total_flops / (t * 1e-3) / 1e12, 2),
                            "pct_of_bf16_mfma_peak": round(100.0 * total_flops / (t * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
-                           "launches_per_step": launches, "avg_launch_us": round(t * 1e3 / launches, 2), "timed_blocks": mm["timed_blocks"]}
+                           "launches_per_step": launches, "avg_launch_us": round(t * 1e3 / launches, 2)}
 
     if args.traffic_leg:
         src = torch.empty(COPY_BYTES, dtype=torch.uint8, device=dev)
@@ -682,68 +790,26 @@ def main():
     traffic = traffic_src = None
     if os.path.exists(TRAFFIC_JSON):
         try:
-            traffic = json.load(open(TRAFFIC_JSON)).get("hbm_bytes_per_launch")
-            traffic_src = ("profiles/flash_fwd_traffic.json: two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of this "
-                           "kernel, scaled by a 1 GiB copy; a recorded constant, not measured in this run")
-        except (ValueError, OSError):
+            traffic = round(json.load(open(TRAFFIC_JSON)).get("hbm_bytes_per_launch"))
+            traffic_src = "recorded: profiles/flash_fwd_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB copy)"
+        except (ValueError, OSError, TypeError):
             traffic = None
 
     rows = {}
     if not args.no_rows and not args.only_all:
         del steps
-        rows = gpu_rows(torch, spa, ops, {"config1", "config2", "config4", "fp8kv", "merge", "config5"}, args.steps, args.warmup)
+        rows = gpu_rows(torch, spa, ops, ALL_ROWS, args.steps, args.warmup)
 
-    launches = {"all": 1, "rank": P, "step": n_pairs}[head]
-    line = {
-        "metric": "fwd attn TFLOP/s + % bf16 MFMA peak, ring-step causal S=8K H32 D128",
-        "value": round(tflops, 2),
-        "unit": "TFLOP/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
-        "config": {
-            "workload": "config 3: simulated ring P=8 on one GPU, bf16 B=1 S=8192 (8 chunks of 1024) H=32 D=128 causal, "
-                        "8 diagonal + 28 full block pairs in ring order, seed 2 N(0,1)*0.5; "
-                        f"schedule '{head}'" + (" (one launch holds every rank's ring; ring steps merge in the online softmax; a one-GPU fusion)" if head == "all" else ""),
-            "flops_per_step": total_flops,
-            "block_pairs": n_pairs,
-        },
-        "pct_of_bf16_mfma_peak": round(100.0 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
-        "protocol": {k2: m_all[k2] for k2 in ("settle_launches", "settle_ms", "cold_ms_per_step", "timed_blocks", "block_ms_min",
-                                              "block_ms_max", "timed_region_s") if k2 in m_all},
-        "other_schedules": other,
-        "roofline": {
-            "bound": "mfma",
-            "kernel": "flash_fwd16_kernel<bf16,128,2>",
-            "achieved": round(tflops, 2),
-            "peak": MFMA_BF16_PEAK_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-            "traffic": traffic,
-            "traffic_source": traffic_src,
-            "avg_launch_us": round(ms * 1e3 / launches, 2),
-            "flops_per_launch": total_flops / launches,
-            "launches_per_step": launches,
-            "algorithmic_bytes_per_launch": algorithmic_bytes() / launches,
-        },
-    }
-    if "step" in other:
-        line["ring_step"] = {"what": "the per-ring-step schedule (one launch per (rank, step), merge in the epilogue): what a rank of a real ring runs",
-                             "tflops": other["step"]["tflops"], "pct_of_bf16_mfma_peak": other["step"]["pct_of_bf16_mfma_peak"],
-                             "avg_launch_us": other["step"]["avg_launch_us"]}
+    cpu_head = host = None
     if not args.no_cpu_baseline:
         cpu = CpuLegs(torch)
-        line["cpu_baseline"] = cpu.ring_forward(B, H, S // P, D, P, P * (P - 1) // 2, SEED, "config 3")
+        cpu_head = cpu.ring_forward(B, H, S // P, D, P, P * (P - 1) // 2, SEED)
         attach_cpu(rows, cpu)
-    if rows:
-        line["rows"] = list(rows.values())
-    print(json.dumps(line))
+        host = cpu.host
+    text = json.dumps(assemble_line(args.steps, args.warmup, head, m_head, other, rows, cpu_head, host, traffic, traffic_src))
+    if len(text) > LINE_LIMIT:
+        print(f"bench.py: the line is {len(text)} bytes, over {LINE_LIMIT}", file=sys.stderr)
+    print(text)
 
 
 if __name__ == "__main__":
