@@ -178,10 +178,19 @@ int spa_ring_fwd_fp8kv(const void* q, const void* k8, const void* v8,
  * exceed the buffer are rejected with SPA_EINVAL when the schedule needs the scratch.  All calls
  * on one device share that device's buffer: calls that overlap in time on one device (two
  * streams, two threads) race; serialise them.  Same kernels, same results as spa_ring_fwd.
- * This entry point has no counterpart in the reference.
+ * Cost: SPA_STATIC_SCRATCH_BYTES (32 MiB) of device memory on every device the library is loaded
+ * on, whether or not this entry point is ever called.
+ * Before a stream capture: the device address of the buffer is looked up (hipGetSymbolAddress) on
+ * the first use per device, and every kernel variant sets its dynamic-LDS attribute on its first
+ * launch per device; neither belongs into a capture.  Call spa_static_scratch_init() with the
+ * device current, and make one eager call with the shapes to be captured, before capturing.
+ * These entry points have no counterpart in the reference.
  */
 #define SPA_STATIC_SCRATCH_BYTES (32 << 20)
 int64_t spa_static_scratch_bytes(void);
+/* Looks up the buffer's address on the current device (idempotent, allocates nothing, launches
+ * nothing).  SPA_OK or SPA_ELAUNCH. */
+int spa_static_scratch_init(void);
 int spa_ring_fwd_static(const void* q, const void* k, const void* v, void* out, float* lse,
                         int B, int H, int S, int D, int P, int rank,
                         const int64_t q_strides[3], const int64_t k_strides[3],

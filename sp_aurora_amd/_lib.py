@@ -5,6 +5,7 @@ fallback path: a missing library raises, it never degrades to torch ops.
 """
 import ctypes
 import os
+import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsp_aurora_hip.so")
@@ -31,6 +32,7 @@ SIGNATURES = {
     "spa_ring_fwd_workspace_bytes": (ctypes.c_int64, [_i, _i, _i, _i, _i, _i]),
     "spa_ring_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _i, _vp]),
     "spa_static_scratch_bytes": (ctypes.c_int64, []),
+    "spa_static_scratch_init": (_i, []),
     "spa_ring_fwd_static": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _i, _vp]),
     "spa_tune": (_i, [_i, _i]),
     "spa_merge": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _s3, _s3, _i, _i, _vp]),
@@ -56,6 +58,10 @@ class SpaError(RuntimeError):
         self.code = code
 
 
+# entry points that return an int but launch nothing: they run as they are while recording
+_QUERIES = ("spa_abi_version", "spa_tune", "spa_device_info", "spa_static_scratch_init")
+
+
 class _Recorder:
     """Stands in for the library while ops.prepared() records a call sequence: every spa_* call is
     stored with its arguments converted to ctypes objects once, and reports success."""
@@ -66,7 +72,7 @@ class _Recorder:
 
     def __getattr__(self, name):
         fn = getattr(self._lib, name)
-        if name not in SIGNATURES or fn.restype is not _i or name in ("spa_abi_version", "spa_tune"):
+        if name not in SIGNATURES or fn.restype is not _i or name in _QUERIES:
             return fn  # queries run as they are
 
         def record(*args):
@@ -79,14 +85,16 @@ class _Recorder:
         return record
 
 
-_recorder = None
+# the recorder of ops.prepared() belongs to the thread that records: other threads keep calling the library
+_tls = threading.local()
 
 
 def load():
     """Load the shared library once and attach the prototypes.  Raises if it was not built."""
     global _lib
-    if _recorder is not None:
-        return _recorder
+    rec = getattr(_tls, "recorder", None)
+    if rec is not None:
+        return rec
     if _lib is not None:
         return _lib
     if not os.path.exists(LIB_PATH):
@@ -130,19 +138,17 @@ def strides2(vals):
 
 
 class recording:
-    """Context manager: inside it, load() hands out a recorder instead of the library."""
+    """Context manager: inside it, load() hands the calling thread a recorder instead of the library."""
 
     def __enter__(self):
-        global _recorder
-        if _recorder is not None:
+        if getattr(_tls, "recorder", None) is not None:
             raise RuntimeError("recording() does not nest")
         lib = load()
-        _recorder = _Recorder(lib)
-        return _recorder
+        _tls.recorder = _Recorder(lib)
+        return _tls.recorder
 
     def __exit__(self, *exc):
-        global _recorder
-        _recorder = None
+        _tls.recorder = None
         return False
 
 

@@ -42,11 +42,14 @@ def build(verbose: bool = True) -> str:
         hipcc = "hipcc"
     objdir = os.path.join(HERE, "_obj")
     os.makedirs(objdir, exist_ok=True)
-    objs = []
-    for src in SOURCES:
-        obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        _run([hipcc] + FLAGS + EXTRA.get(src, []) + ["-c", "-o", obj, os.path.join(CSRC, src)], verbose)
-        objs.append(obj)
+    objs = [os.path.join(objdir, src.replace(".hip", ".o")) for src in SOURCES]
+    # the translation units are independent: compile them side by side (the two attention files take most of the time)
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 1)) as pool:
+        jobs = [pool.submit(_run, [hipcc] + FLAGS + EXTRA.get(src, []) + ["-c", "-o", obj, os.path.join(CSRC, src)], verbose)
+                for src, obj in zip(SOURCES, objs)]
+        for j in jobs:
+            j.result()
     _run([hipcc, "--offload-arch=gfx950", "-fPIC", "-shared", "-o", LIB_PATH] + objs, verbose)
     return LIB_PATH
 

@@ -368,6 +368,11 @@ int spa_ring_fwd_fp8kv(const void* q, const void* k8, const void* v8, const floa
 
 int64_t spa_static_scratch_bytes(void) { return (int64_t)SPA_STATIC_SCRATCH_BYTES; }
 
+int spa_static_scratch_init(void) {
+  void* ws = nullptr;
+  return static_scratch(&ws);
+}
+
 int spa_ring_fwd_static(const void* q, const void* k, const void* v, void* out, float* lse, int B, int H, int S,
                         int D, int P, int rank, const int64_t q_strides[3], const int64_t k_strides[3],
                         const int64_t v_strides[3], const int64_t o_strides[3], float scale, int mask_mode,

@@ -47,23 +47,26 @@ def intel_flash_attn_backward(dout, q, k, v, out, softmax_lse, dq=None, dk=None,
     The reference's function of this name is an empty stub (sp_aurora/intel_flash_attn.py:129-157)
     and its ring backward re-runs autograd per block instead
     (sp_aurora/intel_ring_flash_attn.py:229-244); this one does the block-wise recompute
-    with the given lse.  Writes into dq/dk/dv when given (flash-attn convention) and returns them.
+    with the given lse (spa_flash_bwd_out: no fp32 accumulators to zero, read back and cast).
+    Writes into dq/dk/dv when given (flash-attn convention) and returns them.
     """
     _check_unsupported(dropout_p, window_size, alibi_slopes)
     delta = ops.bwd_delta(out, dout, layout="bhsd")
-    dq_acc = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
-    dk_acc = torch.zeros(k.shape, dtype=torch.float32, device=q.device)
-    dv_acc = torch.zeros(v.shape, dtype=torch.float32, device=q.device)
     lse = softmax_lse if softmax_lse.is_contiguous() else softmax_lse.contiguous()
-    ops.flash_bwd(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, softmax_scale, bool(causal), layout="bhsd")
-    res = []
-    for acc, dst, like in ((dq_acc, dq, q), (dk_acc, dk, k), (dv_acc, dv, v)):
-        if dst is None:
-            res.append(acc.to(like.dtype))
-        else:
-            dst.copy_(acc)
-            res.append(dst)
-    return tuple(res)
+    # one call computes the whole gradient of the block: the kernels write it in the inputs' type,
+    # straight into dq / dk / dv when those are given in a form the kernels can write
+    given = (dq, dk, dv)
+    direct = [g if g is not None and g.dtype == q.dtype and g.shape == like.shape and ops._rows_ok(g, g.element_size()) else None
+              for g, like in zip(given, (q, k, v))]
+    res = ops.flash_bwd_out(q, k, v, dout, lse, delta, softmax_scale, bool(causal), layout="bhsd",
+                            dq=direct[0], dk=direct[1], dv=direct[2])
+    out_grads = []
+    for got, dst, was_direct in zip(res, given, direct):
+        if dst is not None and was_direct is None:
+            dst.copy_(got)
+            got = dst
+        out_grads.append(got)
+    return tuple(out_grads)
 
 
 # the names the ring code imports (sp_aurora/intel_flash_attn.py:161-168)

@@ -385,6 +385,29 @@ def check_cu_seqlens(cu, total, max_seqlen, what):
         raise ValueError(f"{what}: longest sequence {int(lens.max())} exceeds max_seqlen {int(max_seqlen)}")
 
 
+# (address, version counter, length, device, total rows, max_seqlen) of cu_seqlens arrays that passed
+# check_cu_seqlens: a training loop hands the same array to every layer, and one look is enough
+_CU_CHECKED = {}
+
+
+def check_cu_seqlens_once(cu, total, max_seqlen, what):
+    """check_cu_seqlens, remembered per distinct array (same storage address, same version counter,
+    same sizes), so that only the first call with an array pays the blocking device-to-host read.
+    While the current stream is being captured nothing is read (a synchronous copy is illegal
+    there): the caller of a captured region vouches for its offsets.  Returns True when the array
+    is known to be good, False when the check was skipped."""
+    key = (cu.data_ptr(), cu._version, cu.numel(), str(cu.device), int(total), int(max_seqlen))
+    if key in _CU_CHECKED:
+        return True
+    if cu.is_cuda and torch.cuda.is_current_stream_capturing():
+        return False
+    check_cu_seqlens(cu, total, max_seqlen, what)
+    if len(_CU_CHECKED) >= 256:
+        _CU_CHECKED.clear()
+    _CU_CHECKED[key] = True
+    return True
+
+
 
 def _thd(t, what):
     """(rows, H, D) sizes and (head, row) element strides of a packed 3-D tensor."""
@@ -540,13 +563,17 @@ def flash_bwd_varlen(q, k, v, dout, lse, delta, dq_acc, dk_acc, dv_acc, cu_seqle
 
 
 def flash_bwd_varlen_out(q, k, v, dout, lse, delta, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-                         softmax_scale=None, causal=False, dq=None, dk=None, dv=None):
+                         softmax_scale=None, causal=False, dq=None, dk=None, dv=None, rows_covered=False):
     """Backward of flash_fwd_varlen in one call: returns (dq, dk, dv) in q's dtype, written by the
-    kernels (no fp32 accumulators).  cu_seqlens must cover every row of the packed tensors: rows of
-    no sequence are not written.  Calls spa_flash_bwd_varlen_out."""
-    dq = torch.empty(q.shape, dtype=q.dtype, device=q.device) if dq is None else dq
-    dk = torch.empty(k.shape, dtype=q.dtype, device=q.device) if dk is None else dk
-    dv = torch.empty(v.shape, dtype=q.dtype, device=q.device) if dv is None else dv
+    kernels (no fp32 accumulators).  The kernels write the rows of the sequences cu_seqlens names, up
+    to max_seqlen each: a row of no sequence is not touched.  Gradients allocated here therefore start
+    as zeros unless the caller vouches with rows_covered=True that the offsets end at the tensors' row
+    counts and no sequence exceeds max_seqlen (what check_cu_seqlens establishes); tensors passed in
+    as dq / dk / dv are the caller's to initialise.  Calls spa_flash_bwd_varlen_out."""
+    alloc = torch.empty if rows_covered else torch.zeros
+    dq = alloc(q.shape, dtype=q.dtype, device=q.device) if dq is None else dq
+    dk = alloc(k.shape, dtype=q.dtype, device=q.device) if dk is None else dk
+    dv = alloc(v.shape, dtype=q.dtype, device=q.device) if dv is None else dv
     _flash_bwd_varlen("spa_flash_bwd_varlen_out", q, k, v, dout, lse, delta, dq, dk, dv, q.dtype,
                       cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, causal)
     return dq, dk, dv

@@ -135,7 +135,7 @@ def intel_ulysses_flash_attn_forward(process_group, q, k, v, softmax_scale, drop
     if q.dim() == 4:
         return ops.flash_fwd(q, k, v, softmax_scale, causal, layout="bshd")
     P, B, s, H, D = q.shape
-    views_ok = B == 1 and H % P == 0 and all(t.is_contiguous() for t in (q, k, v)) and q.shape == k.shape == v.shape
+    views_ok = _views_ok(q, k, v)
     if relayout == "views" and not views_ok:
         raise ValueError("relayout='views' needs B = 1 and compact q, k, v of one shape")
     if relayout != "kernels" and views_ok:
@@ -152,6 +152,14 @@ def intel_ulysses_flash_attn_forward(process_group, q, k, v, softmax_scale, drop
                            softmax_scale, causal, layout="bshd")
     out = ops.relayout_h2s(o.view(P, B, P * s, h, D), P)
     return out, lse.view(P, B, h, P * s)
+
+
+def _views_ok(q, *others):
+    """Can head groups be read / written as strided views of these rank-stacked [P,B,s,H,D] tensors?
+    B = 1, heads divisible by the ranks, every tensor compact and of q's shape (a view is built
+    with q's sizes, so a tensor of another shape would be read wrongly)."""
+    P, B, s, H, D = q.shape
+    return B == 1 and H % P == 0 and all(t.shape == q.shape and t.is_contiguous() for t in (q,) + others)
 
 
 class UlyssesFlashAttnFunc(torch.autograd.Function):
@@ -180,13 +188,13 @@ class UlyssesFlashAttnFunc(torch.autograd.Function):
         else:
             P, B, s, H, D = q.shape
             h = H // P
-            if B == 1 and all(t.is_contiguous() for t in (q, k, v, out)):
+            if _views_ok(q, k, v, out) and dout.shape == q.shape:
                 # as in the forward: head groups are strided views of the stacked tensors, and the kernels
                 # write the gradients through such views of stacked tensors, so nothing is re-laid
                 grp = lambda t: t.as_strided((P, P * s, h, D), (h * D, H * D, D, 1), t.storage_offset())
                 dout = dout.contiguous()
                 delta = ops.bwd_delta(grp(out), grp(dout), layout="bshd")
-                grads = [torch.empty_like(q) for _ in range(3)]
+                grads = [torch.empty_like(t) for t in (q, k, v)]
                 ops.flash_bwd_out(grp(q), grp(k), grp(v), grp(dout), lse.view(P, h, P * s), delta, ctx.softmax_scale, ctx.causal,
                                   layout="bshd", dq=grp(grads[0]), dk=grp(grads[1]), dv=grp(grads[2]))
                 return tuple(grads) + (None,) * 8

@@ -254,3 +254,28 @@ def test_cu_seqlens_are_checked_on_the_host():
         spa.sp_aurora_varlen_func(q, q, q, torch.tensor([0, 5, 10], dtype=torch.int32), max_seqlen=5)
     with pytest.raises(ValueError, match="exceeds"):
         spa.sp_aurora_varlen_func(q, q, q, torch.tensor([0, 5, 12], dtype=torch.int32), max_seqlen=5)
+
+
+def test_recording_belongs_to_the_recording_thread():
+    """ops.prepared() swaps a recorder in for the calling thread only: another thread that calls into
+    the library meanwhile reaches the real library (here: a query that must run, not be recorded)."""
+    import threading
+    seen = {}
+    with _lib.recording() as rec:
+        assert _lib.load() is rec
+
+        def other():
+            lib = _lib.load()
+            seen["is_recorder"] = lib is rec
+            seen["version"] = lib.spa_abi_version()
+
+        t = threading.Thread(target=other)
+        t.start()
+        t.join()
+        # queries that launch nothing run as they are, also on the recording thread
+        assert rec.spa_static_scratch_bytes() == 32 << 20
+        buf = ctypes.create_string_buffer(8)
+        assert rec.spa_device_info(buf, 0) == -1  # ran (and refused the zero-sized buffer) instead of being recorded
+        assert rec.calls == []
+    assert seen == {"is_recorder": False, "version": 1}
+    assert not isinstance(_lib.load(), _lib._Recorder)

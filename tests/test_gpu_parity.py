@@ -555,6 +555,15 @@ def test_backward_packed_and_operator_entry():
     dq, dk, dv = spa._flash_attn_backward(t(dout), q, k, v, o, l, causal=True)
     for got, w, name in zip((dq, dk, dv), want, "qkv"):
         check_grad(got.transpose(1, 2), w, torch.bfloat16, "operator d" + name)
+    # gradients written into tensors the caller passes: as they are when the kernels can write them
+    # (here dq, and dk as one half of a packed buffer), through a copy when not (dv is fp32)
+    gq = torch.full_like(q, 7.0)
+    gkv = torch.full((B, H, S, 2, D), 7.0, dtype=q.dtype, device=DEV)
+    gv = torch.full(v.shape, 7.0, dtype=torch.float32, device=DEV)
+    r = spa._flash_attn_backward(t(dout), q, k, v, o, l, dq=gq, dk=gkv[:, :, :, 0], dv=gv, causal=True)
+    assert r[0] is gq and r[2] is gv and r[1].data_ptr() == gkv.data_ptr()
+    assert torch.equal(gq, dq) and torch.equal(gkv[:, :, :, 0], dk) and torch.equal(gv, dv.float())
+    assert (gkv[:, :, :, 1] == 7.0).all()
 
 
 def test_delta_kernel():

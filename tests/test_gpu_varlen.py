@@ -175,3 +175,42 @@ def test_varlen_lse_helpers_round_trip():
     padded = spa.unflatten_varlen_lse(lse.t().unsqueeze(-1), cu, 64)     # [nseq, H, max]
     assert padded.shape == (3, H, 64)
     assert torch.equal(spa.flatten_varlen_lse(padded, cu), lse)
+
+
+def test_varlen_offsets_are_read_on_the_host_once_per_array():
+    """The first call with a cu_seqlens array validates it (a blocking device-to-host read); later calls
+    with the same array, with max_seqlen given, must not synchronise with the device at all - and a changed
+    array is looked at again."""
+    lengths, H, D = [30, 64, 7], 2, 64
+    T = sum(lengths)
+    q, k, v = (rand((T, H, D), 440 + i, torch.bfloat16).to(DEV) for i in range(3))
+    cu = cu_of(lengths).to(DEV)
+    first = spa.sp_aurora_varlen_func(q, k, v, cu, cu, max_seqlen=64, causal=True)
+    torch.cuda.synchronize()
+    torch.cuda.set_sync_debug_mode("error")
+    try:
+        again = spa.sp_aurora_varlen_func(q, k, v, cu, cu, max_seqlen=64, causal=True)
+        unchecked = spa.sp_aurora_varlen_func(q, k, v, cu.clone(), None, max_seqlen=64, causal=True, check_offsets=False)
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
+    assert torch.equal(first, again) and torch.equal(first, unchecked)
+    cu[-1] = T - 1  # in place: same address, new version counter
+    with pytest.raises(ValueError):
+        spa.sp_aurora_varlen_func(q, k, v, cu, cu, max_seqlen=64, causal=True)
+
+
+def test_varlen_backward_leaves_zeros_in_rows_of_no_sequence():
+    """Direct callers of ops.flash_bwd_varlen_out may pass offsets that end before the tensors do: the
+    gradients allocated by the wrapper are zero there (the kernels do not touch such rows)."""
+    lengths, H, D, dtype = [40, 24], 2, 64, torch.bfloat16
+    used, T = sum(lengths), sum(lengths) + 19
+    q, k, v, dout = (rand((T, H, D), 450 + i, dtype).to(DEV) for i in range(4))
+    cu = cu_of(lengths).to(DEV)
+    out, lse = ops.flash_fwd_varlen(q, k, v, cu, cu, 40, 40, None, True, out=torch.zeros_like(q),
+                                    lse=torch.zeros((H, T), dtype=torch.float32, device=DEV))
+    delta = ops.bwd_delta(out.unsqueeze(0), dout.unsqueeze(0), layout="bshd")[0]
+    junk = torch.full((64 << 20,), 1e30, dtype=torch.float32, device=DEV)  # what a recycled allocation may hold
+    del junk
+    dq, dk, dv = ops.flash_bwd_varlen_out(q, k, v, dout, lse, delta, cu, cu, 40, 40, None, True)
+    for g in (dq, dk, dv):
+        assert not g[used:].any() and g[:used].float().abs().max() > 0
