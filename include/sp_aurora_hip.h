@@ -144,8 +144,17 @@ int spa_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* 
  * It may be NULL only when no launch needs it: 16-bit types in the fused modes, or a schedule in
  * which no rank visits more than one block (P = 1; causal rank 0).  fp32 inputs with more than
  * one block per rank always need it (SPA_EINVAL otherwise).
+ * Zigzag shards: `fuse | SPA_RING_ZIGZAG` declares that the rows of q, k, v (and of out, lse) are in
+ * zigzag-sharded order — with the sequence cut into 2P half-chunks, chunk r of the tensors holds
+ * half-chunks r and 2P-1-r — the sharding the reference's test names and does not ship
+ * (zigzag_sp_aurora_varlen_func, test/flash_attention/test_intel_ring_flash_attn_varlen.py:25,205-215).
+ * Every rank of a causal ring then has the same work: step 0 is causal attention on the rank's own
+ * chunk; at step t >= 1 (chunk c = (r - t) mod P) all local queries see the first half of the
+ * chunk when c < r, and the second half of the local queries sees the whole chunk when c > r; all P
+ * steps run for every rank.  Needs S divisible by 2P; without a mask the flag changes nothing.
  */
 enum { SPA_RING_PER_STEP = 0, SPA_RING_PER_RANK = 1, SPA_RING_ALL_RANKS = 2 };
+#define SPA_RING_ZIGZAG 16
 int64_t spa_ring_fwd_workspace_bytes(int B, int H, int S, int D, int P, int dtype);
 int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
                  int B, int H, int S, int D, int P, int rank,

@@ -17,7 +17,8 @@ forms (uniform keys, one visible key, constant V), library routines
 invariants the reference's own tests assert (ring == full attention,
 test/test_ring_attention_full_accuracy.py:122-171; packed == unpacked,
 test/test_ring_attention_comprehensive.py:205-218; inverse o forward re-layout is
-the identity).  No function is left "parity unpinned".
+the identity; a zigzag-sharded ring == full causal attention after un-permuting the rows).
+No function is left "parity unpinned".
 
 Layouts: the block operator uses the reference's operator layout [B, H, S, D]
 (sp_aurora/intel_flash_attn.py:56); the ring and Ulysses drivers use the public
@@ -183,6 +184,59 @@ def ring_forward(q, k, v, P, softmax_scale=None, causal=False, compute_dtype=CD,
     qs, ks, vs = q.chunk(P, dim=1), list(k.chunk(P, dim=1)), list(v.chunk(P, dim=1))
     outs, lses = zip(*[ring_forward_rank(qs[r], ks, vs, r, softmax_scale, causal, compute_dtype, out_dtype)
                        for r in range(P)])
+    return torch.cat(outs, dim=1), torch.cat(lses, dim=2)
+
+
+def zigzag_order(S, P):
+    """Row order of a zigzag-sharded sequence: with the S rows cut into 2P half-chunks, rank r holds
+    half-chunk r followed by half-chunk 2P-1-r, and the ranks' shards are stacked in rank order.
+    Returns idx (int64 [S]) with sharded = natural.index_select(1, idx).  The sharding the
+    reference's test names (zigzag_sp_aurora_varlen_func,
+    test/flash_attention/test_intel_ring_flash_attn_varlen.py:25,205-215) without shipping it:
+    every rank of a causal ring then has the same amount of work."""
+    if S % (2 * P):
+        raise ValueError(f"zigzag sharding needs 2 * P = {2 * P} to divide the sequence length {S}")
+    hc = S // (2 * P)
+    idx = []
+    for r in range(P):
+        idx += list(range(r * hc, (r + 1) * hc)) + list(range((2 * P - 1 - r) * hc, (2 * P - r) * hc))
+    return torch.tensor(idx, dtype=torch.int64)
+
+
+def ring_forward_zigzag_rank(q_local, k_chunks, v_chunks, rank, softmax_scale=None, compute_dtype=CD, out_dtype=None):
+    """Causal ring forward of rank `rank` on zigzag shards: the step loop of
+    intel_ring_flash_attn_forward (sp_aurora/intel_ring_flash_attn.py:72-148) with the block of each
+    step cut to what a zigzag shard can see.  The rank holds half-chunks (rank, 2P-1-rank); at step t
+    it has the shard of rank c = (rank - t) mod P, half-chunks (c, 2P-1-c):
+      t == 0       its own shard: plain causal attention on the local rows (the local order is the global one)
+      c <  rank    every local query sees the first half of the shard (half-chunk c), none of the second
+      c >  rank    only the second half of the local queries sees anything, and it sees the whole shard
+    every step is merged with update_out_and_lse (for c > rank into the second half of the rows only)."""
+    P = len(k_chunks)
+    out_dtype = out_dtype or q_local.dtype
+    hs = q_local.shape[1] // 2
+    q = q_local.transpose(1, 2)
+    out, lse = attn_block(q, k_chunks[rank].transpose(1, 2), v_chunks[rank].transpose(1, 2), softmax_scale, True, compute_dtype)
+    lse = lse.unsqueeze(-1)
+    for step in range(1, P):
+        c = (rank - step) % P
+        kc, vc = k_chunks[c].transpose(1, 2), v_chunks[c].transpose(1, 2)
+        if c < rank:
+            b_out, b_lse = attn_block(q, kc[:, :, :hs], vc[:, :, :hs], softmax_scale, False, compute_dtype)
+            out, lse = merge(out, lse, b_out, b_lse.unsqueeze(-1))
+        else:
+            b_out, b_lse = attn_block(q[:, :, hs:], kc, vc, softmax_scale, False, compute_dtype)
+            o2, l2 = merge(out[:, :, hs:], lse[:, :, hs:], b_out, b_lse.unsqueeze(-1))
+            out = torch.cat([out[:, :, :hs], o2], dim=2)
+            lse = torch.cat([lse[:, :, :hs], l2], dim=2)
+    return out.transpose(1, 2).to(out_dtype), lse.squeeze(-1)
+
+
+def ring_forward_zigzag(q, k, v, P, softmax_scale=None, compute_dtype=CD, out_dtype=None):
+    """All P ranks of a causal zigzag ring; q,k,v [B,S,H,D] in zigzag-sharded row order (zigzag_order);
+    out and lse come back in the same order."""
+    qs, ks, vs = q.chunk(P, dim=1), list(k.chunk(P, dim=1)), list(v.chunk(P, dim=1))
+    outs, lses = zip(*[ring_forward_zigzag_rank(qs[r], ks, vs, r, softmax_scale, compute_dtype, out_dtype) for r in range(P)])
     return torch.cat(outs, dim=1), torch.cat(lses, dim=2)
 
 

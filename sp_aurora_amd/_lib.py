@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libsp_aurora_hip.so")
 SPA_F32, SPA_BF16, SPA_F16 = 0, 1, 2
 SPA_MASK_NONE, SPA_MASK_CAUSAL = 0, 1
 SPA_RING_PER_STEP, SPA_RING_PER_RANK, SPA_RING_ALL_RANKS = 0, 1, 2
+SPA_RING_ZIGZAG = 16  # or-ed into `fuse`: the rows are in zigzag-sharded order
 
 _I64x3 = ctypes.c_int64 * 3
 _vp = ctypes.c_void_p

@@ -123,7 +123,13 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const float vsc = KV8 ? p.v_scale[bh] : 1.f;
   const int qt = p.nqt - 1 - (int)blockIdx.y;
   const int rank = p.rank0 + p.nranks - 1 - (int)blockIdx.z;
-  const int q0 = qt * C::BMW;
+  // Zigzag shards: the tiles of the two halves of the chunk are laid out one half after the other (a tile
+  // never holds rows of both), the second (heavier) half first in dispatch order.
+  const bool zz = p.zigzag != 0;
+  const int zz_hs = p.Sq >> 1;                                    // rows per half-chunk
+  const int zz_nqh = p.zz_half ? p.nqt : p.nqt >> 1;              // tiles per half
+  const bool zhalf = zz && (p.zz_half || qt >= zz_nqh);           // this workgroup's rows lie in the second half
+  const int q0 = zz ? (zhalf ? zz_hs : 0) + (qt - (zhalf && !p.zz_half ? zz_nqh : 0)) * C::BMW : qt * C::BMW;
   if (p.cu_q) {
     const int q_lo = p.cu_q[b], k_lo = p.cu_k[b];
     p.Sq = p.cu_q[b + 1] - q_lo;
@@ -147,6 +153,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       return;
     }
   }
+  const int q_lim = zz && !zhalf ? zz_hs : p.Sq;  // one past the last row this workgroup may own
   const int qw0 = q0 + (SHARE ? grp * FWD_BM : 0) + w * 32;
   const int64_t qoff = (int64_t)rank * p.Sq;  // first row of this rank's query chunk
 
@@ -155,7 +162,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const KVT* vp = (const KVT*)p.v + b * p.vs.b + h * p.vs.h;
 
   const int qrow = qw0 + ln;
-  const int qrow_c = qrow < p.Sq ? qrow : p.Sq - 1;
+  const int qrow_c = qrow < q_lim ? qrow : q_lim - 1;
 
   frag qf[D / 16];
   const unsigned qsign = p.negq ? 0x80008000u : 0u;  // negative softmax scale: -q with |scale|
@@ -175,19 +182,73 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   constexpr int BN = C::BN, NT = C::NT;
   constexpr int TILE = SHARE ? BN : BN * NG;  // keys between two sub-tiles of one group
   constexpr int KSTEP = SHARE ? 1 : NG;
-  const int nsteps = p.causal ? (rank + 1 < p.P ? rank + 1 : p.P) : p.P;
+  // A zigzag ring has P steps for the second half of a chunk's rows and steps 0..r for the first half;
+  // steps 1..r use the first half of their chunk's keys (zz_last_half: the last such step, -1 without zigzag).
+  const int nsteps = p.causal ? (zhalf ? p.P : rank + 1 < p.P ? rank + 1 : p.P) : p.P;
   const int t_end = p.t_count < 0 || p.t_begin + p.t_count > nsteps ? nsteps : p.t_begin + p.t_count;
   const bool diag = p.causal && p.t_begin == 0;
   const int kv_end = q0 + C::BMW < p.Sk ? q0 + C::BMW : p.Sk;  // keys of the diagonal chunk in use
   const int n_diag = diag ? (kv_end + TILE - 1) / TILE : 0;
   const int npc = (p.Sk + TILE - 1) / TILE;                    // sub-tiles per full chunk
+  const int zz_last_half = zz ? rank : -1;
+  const int klen_h = zz ? zz_hs : p.Sk;                        // keys of a half step
+  const int npc_h = (klen_h + TILE - 1) / TILE;                // sub-tiles of a half step
   const int t_full0 = p.t_begin + (diag ? 1 : 0);              // first unmasked step
-  const int n = n_diag + (t_end - t_full0 > 0 ? (t_end - t_full0) * npc : 0);
+  const int t_half_end = t_end < zz_last_half + 1 ? t_end : zz_last_half + 1;  // unmasked steps before this one are half steps
+  const int n_hsteps = t_half_end > t_full0 ? t_half_end - t_full0 : 0;
+  const int n_fsteps = t_end - t_full0 - n_hsteps > 0 ? t_end - t_full0 - n_hsteps : 0;
+  const int n = n_diag + n_hsteps * npc_h + n_fsteps * npc;
+  if constexpr (FINALN) {
+    if (n == 0) {
+      // The launch of a zigzag rank's last step, first half of the rows: no block here (their last block was
+      // step `rank`), so the workgroup only applies update_out_and_lse (sp_aurora/utils.py:103-104) to the
+      // slots of steps 0 .. rank, in that order, and writes the rows' final (out, lse).
+      typedef Mma16<T> MM;
+      constexpr float LOG2E = 1.4426950408889634f;
+      const int nslot = rank + 1 < p.npart ? rank + 1 : p.npart;
+      const RingSlots slots(p.B, p.H, p.Sq, D);
+      const int64_t slot_rs = (int64_t)p.H * D;  // a slot is contiguous [B, Sq, H, D]
+      const int64_t slot_bh = (int64_t)b * p.Sq * slot_rs + h * D;
+      const int64_t qoff0 = (int64_t)rank * p.Sq;
+      T* const out0 = (T*)p.out + b * p.os.b + h * p.os.h + qoff0 * p.os.s;
+      float* const lse0 = p.lse + ((int64_t)b * p.H + h) * p.lse_bh + qoff0;
+      for (int idx = tid; idx < C::BMW * (D / 8); idx += FWD_THREADS * NG) {
+        const int grow = q0 + idx / (D / 8), ch = idx % (D / 8);
+        if (grow >= q_lim) break;
+        float x[8], lb = -INFINITY, wsum = 0.f;
+#pragma unroll
+        for (int k2 = 0; k2 < 8; ++k2) x[k2] = 0.f;
+        for (int j = 0; j < nslot; ++j) {
+          const u32x4 raw = *(const u32x4*)(slots.template out<T>(p.part, j) + slot_bh + (int64_t)grow * slot_rs + ch * 8);
+          const float lj = (slots.lse(p.part, p.P, j) + ((int64_t)b * p.H + h) * p.Sq)[grow];
+          const float mx = fmaxf(lb, lj);  // slot 0, the diagonal block, is finite in every row
+          const float wa = fast_exp2((lb - mx) * LOG2E), wb = fast_exp2((lj - mx) * LOG2E);
+          wsum = wsum * wa + wb;
+          lb = mx;
+#pragma unroll
+          for (int k2 = 0; k2 < 4; ++k2) {
+            float lo, hi;
+            MM::unpack2(raw[k2], lo, hi);
+            x[2 * k2] = x[2 * k2] * wa + lo * wb;
+            x[2 * k2 + 1] = x[2 * k2 + 1] * wa + hi * wb;
+          }
+        }
+        const float inv = 1.f / wsum;
+        u32x4 st;
+#pragma unroll
+        for (int k2 = 0; k2 < 4; ++k2) st[k2] = MM::pack2(x[2 * k2] * inv, x[2 * k2 + 1] * inv);
+        *(u32x4*)(out0 + (int64_t)grow * p.os.s + ch * 8) = st;
+        if (ch == 0) lse0[grow] = lb + fast_log2(wsum) * 0.6931471805599453f;
+      }
+      return;
+    }
+  }
 
   struct Sub {
     int krel;   // first key of the sub-tile, relative to its chunk
     int krow;   // the same as a row of the K/V tensors
     int kend;   // one past the chunk's last row
+    int klen;   // keys of the chunk this step may use (half a chunk in some steps of a zigzag ring)
     bool masked;
   };
   // The loop walks the sub-tiles in order with three cursors (softmax at i, V loads at i+1,
@@ -202,7 +263,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     if (c.i == n_diag) {
       c.j = 0;
       c.t = t_full0;
-    } else if (c.i > n_diag && c.j == npc) {
+    } else if (c.i > n_diag && c.j == (c.t <= zz_last_half ? npc_h : npc)) {
       c.j = 0;
       ++c.t;
     }
@@ -210,6 +271,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     ch = ch < 0 ? ch + p.P : ch;
     ch = ch < 0 ? 0 : ch;  // only past the end of the schedule, where nothing is used
     c.sb.masked = c.i < n_diag;
+    c.sb.klen = c.i >= n_diag && c.t <= zz_last_half ? klen_h : p.Sk;
     c.sb.krel = (c.j * KSTEP + (SHARE ? 0 : grp)) * BN;
     c.sb.krow = ch * p.Sk + c.sb.krel;
     c.sb.kend = ch * p.Sk + p.Sk;
@@ -390,9 +452,9 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   auto softmax_phase = [&](const Sub& sb, frag (&pfr)[NT][2]) {
     const int key0 = sb.krel;
     const bool causal_here = sb.masked;
-    const bool need_mask = (causal_here && key0 + BN - 1 > qw0) || (key0 + BN > p.Sk);
+    const bool need_mask = (causal_here && key0 + BN - 1 > qw0) || (key0 + BN > sb.klen);
     if (need_mask) {
-      const int lim = causal_here ? (qrow < p.Sk - 1 ? qrow : p.Sk - 1) : p.Sk - 1;  // last visible key
+      const int lim = causal_here ? (qrow < sb.klen - 1 ? qrow : sb.klen - 1) : sb.klen - 1;  // last visible key
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -441,7 +503,10 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     // 2^8 in the exp2 domain; until then P <= 256, harmless in fp32 sums and bf16 operands.
     if (__builtin_amdgcn_ballot_w64((mx - m_run) * c > 8.f) != 0) {
       const float m_new = fmaxf(m_run, mx);
-      const float alpha = fast_exp2((m_run - m_new) * c);
+      // (a lane whose row has seen no key yet, here or before, while another row of the wave asks for the
+      // rescale: -inf - -inf; nothing of that row needs scaling.  Rows of a wave differ in this only when
+      // the tile's first row is not a multiple of the sub-tile size: the second half of a zigzag shard.)
+      const float alpha = m_new == -INFINITY ? 1.f : fast_exp2((m_run - m_new) * c);
       m_run = m_new;
       l_run *= alpha;
 #pragma unroll
@@ -493,6 +558,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     int ch = rank - cs.t;
     ch = ch < 0 ? ch + p.P : ch;
     cs.sb.masked = n_diag > 0;
+    cs.sb.klen = n_diag == 0 && cs.t <= zz_last_half ? klen_h : p.Sk;
     cs.sb.krel = (SHARE ? 0 : grp) * BN;
     cs.sb.krow = ch * p.Sk + cs.sb.krel;
     cs.sb.kend = ch * p.Sk + p.Sk;
@@ -623,7 +689,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     // lanes of a row side by side.  No LDS round trip, no barrier.
     const float l_tot = halves_sum(l_run);
     const float inv = vsc / l_tot;
-    if (hh == 0 && qrow < p.Sq) lse_bh[qrow] = (m_run * c + fast_log2(l_tot)) * 0.6931471805599453f;
+    if (hh == 0 && qrow < q_lim) lse_bh[qrow] = (m_run * c + fast_log2(l_tot)) * 0.6931471805599453f;
     T* const orow = out_bh + qrow_c * out_rs;
 #pragma unroll
     for (int db = 0; db < D / 32; ++db)
@@ -642,7 +708,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
           st[k] = r[0];      // lanes 0-31: own dims 0-3 of the even group; lanes 32-63: partner's dims 0-3 of the odd group
           st[2 + k] = r[1];  // lanes 0-31: partner's dims 4-7 of the even group; lanes 32-63: own dims 4-7 of the odd group
         }
-        if (qrow < p.Sq) *(u32x4*)(orow + db * 32 + 8 * (2 * gp + hh)) = st;
+        if (qrow < q_lim) *(u32x4*)(orow + db * 32 + 8 * (2 * gp + hh)) = st;
       }
     return;
   } else {
@@ -682,7 +748,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
 #pragma unroll
           for (int it = 0; it < NIT; ++it) {
             const int grow = q0 + crow[it];
-            if (grow < p.Sq) {
+            if (grow < q_lim) {
               raw[jj][it] = *(const u32x4*)(so + (int64_t)grow * slot_rs + cch[it] * 8);
               rl[jj][it] = sl[grow];
             }
@@ -792,7 +858,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
       const int grow = q0 + crow[it];
-      if (grow >= p.Sq) continue;
+      if (grow >= q_lim) continue;
       u32x4 st;
       st[0] = M::pack2(x[it][0], x[it][1]);
       st[1] = M::pack2(x[it][2], x[it][3]);
@@ -1027,6 +1093,14 @@ hipError_t launch(int threads, int smem, const FwdParams& p, hipStream_t stream)
   return hipGetLastError();
 }
 
+// Query tiles of `bm` rows per (batch, head, rank): zigzag shards are tiled half by half (no tile holds
+// rows of both halves); a launch for the second half only (zz_half) has that half's tiles.
+int fwd_tiles(const FwdParams& p, int bm) {
+  if (!p.zigzag) return (p.Sq + bm - 1) / bm;
+  const int per_half = (p.Sq / 2 + bm - 1) / bm;
+  return p.zz_half ? per_half : 2 * per_half;
+}
+
 // Two wave groups once there are at least two 64-key sub-tiles to split; 256-row workgroups with
 // shared K/V buffers once that still leaves every CU at least two workgroups.  spa_tune() can
 // force either choice (experiments and tests).
@@ -1040,7 +1114,7 @@ hipError_t launch16(FwdParams p, hipStream_t stream) {
     return launch<flash_fwd16_kernel<T, D, 1, false, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
   }
   if (two && D >= 64) {
-    const int nqt2 = (p.Sq + 2 * FWD_BM - 1) / (2 * FWD_BM);
+    const int nqt2 = fwd_tiles(p, 2 * FWD_BM);
     const int64_t wgs = (int64_t)p.B * p.H * nqt2 * p.nranks;
     const bool share = force_share ? force_share == 2 : wgs >= 2 * (int64_t)spa_device_cus();
     if (share) {
@@ -1063,7 +1137,7 @@ hipError_t launch16_kv8(FwdParams p, hipStream_t stream) {
     return launch<flash_fwd16_kernel<T, D, 1, false, true, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
   }
   if (two) {
-    const int nqt2 = (p.Sq + 2 * FWD_BM - 1) / (2 * FWD_BM);
+    const int nqt2 = fwd_tiles(p, 2 * FWD_BM);
     const int64_t wgs = (int64_t)p.B * p.H * nqt2 * p.nranks;
     const bool share = force_share ? force_share == 2 : wgs >= 2 * (int64_t)spa_device_cus();
     if (share) {
@@ -1079,7 +1153,8 @@ hipError_t launch16_kv8(FwdParams p, hipStream_t stream) {
 
 // Returns hipSuccess, or hipErrorInvalidValue for an unsupported (dtype, D).
 hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream) {
-  p.nqt = (p.Sq + FWD_BM - 1) / FWD_BM;
+  if (p.zigzag && (dtype == 0 || !p.causal || (p.Sq & 1) || p.cu_q)) return hipErrorInvalidValue;  // 16-bit causal rings only
+  p.nqt = fwd_tiles(p, FWD_BM);
   if (p.epi == SPA_EPI_PART) {
     // A ring step that is not the rank's last: the kernel writes the block as it would write any
     // result, and out / lse are pointed at the step's slot here.  The kernel adds the rank's row

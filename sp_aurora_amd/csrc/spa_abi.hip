@@ -235,7 +235,11 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   if (rank < -1 || rank >= P) return fail(SPA_EINVAL, "%s: rank %d outside [-1, %d)", what, rank, P);
   if (!dtype_ok(dtype)) return fail(SPA_EINVAL, "%s: bad dtype %d", what, dtype);
   if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "%s: bad mask_mode %d", what, mask_mode);
+  const bool zig_req = (fuse & SPA_RING_ZIGZAG) != 0;
+  fuse &= ~SPA_RING_ZIGZAG;
   if (fuse < SPA_RING_PER_STEP || fuse > SPA_RING_ALL_RANKS) return fail(SPA_EINVAL, "%s: bad fuse mode %d", what, fuse);
+  if (zig_req && S % (2 * P) != 0)
+    return fail(SPA_EINVAL, "%s: zigzag sharding needs 2 * ring size = %d to divide the sequence length %d", what, 2 * P, S);
   if (!scale_ok(scale)) return fail(SPA_EINVAL, "%s: softmax scale must be finite", what);
   if (D != 32 && D != 64 && D != 128) return fail(SPA_EUNSUPPORTED, "%s: head dim %d not in {32,64,128}", what, D);
   const bool kv8 = k_scale || v_scale;
@@ -253,7 +257,9 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   const bool causal = mask_mode == SPA_MASK_CAUSAL;
   const int s = S / P;
   if (dtype == SPA_F32) fuse = SPA_RING_PER_STEP;  // the fp32 kernel handles one block pair per launch
-  const bool multi = P > 1 && (!causal || rank != 0);  // does some rank visit more than one block?
+  // zigzag shards only change a causal ring (without a mask the order of the rows does not matter)
+  const bool zig = zig_req && causal && P > 1;
+  const bool multi = P > 1 && (!causal || rank != 0 || zig);  // does some rank visit more than one block?
   if (fuse == SPA_RING_PER_STEP && multi && !workspace)
     return fail(SPA_EINVAL, "%s: workspace required when steps are separate launches", what);
   if (fuse == SPA_RING_PER_STEP && multi && ws_bytes >= 0 && spa_ring_fwd_workspace_bytes(B, H, S, D, P, dtype) > ws_bytes)
@@ -287,6 +293,8 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   p.epi = SPA_EPI_PLAIN;
   p.cu_q = nullptr; p.cu_k = nullptr;
   p.k_scale = k_scale; p.v_scale = v_scale;
+  p.zigzag = zig && dtype != SPA_F32;
+  p.zz_half = 0;
 
   if (fuse == SPA_RING_ALL_RANKS) {  // one launch: every requested rank, every step
     p.rank0 = r_lo; p.nranks = r_hi - r_lo; p.t_begin = 0; p.t_count = -1;
@@ -300,7 +308,8 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
       if (e != hipSuccess) return launch_result(e, what);
       continue;
     }
-    const int nsteps = causal ? r + 1 : P;
+    const int nsteps = causal && !zig ? r + 1 : P;  // a zigzag rank has work in every step
+    const int hs = s / 2;
     for (int t = 0; t < nsteps; ++t) {
       hipError_t e;
       if (dtype != SPA_F32) {
@@ -309,7 +318,33 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
         p.epi = nsteps == 1 ? SPA_EPI_PLAIN : t + 1 == nsteps ? SPA_EPI_FINALN : SPA_EPI_PART;
         p.part_slot = t;
         p.npart = nsteps - 1;
+        // zigzag, a step past the rank's own number: only the second half of the rows has a block.  The launch
+        // covers that half's tiles, except the last step's: there the first half's workgroups merge their slots.
+        p.zz_half = zig && t > r && t + 1 < nsteps;
         e = spa_launch_flash_fwd(p, D, dtype, st);
+      } else if (zig) {
+        // fp32, zigzag: plain block launches on explicit sub-blocks, merged by the stand-alone kernels
+        // (step 0: the rank's own chunk, causal; chunk c < r: all rows x first half of the keys; c > r:
+        // second half of the rows x all keys, merged into those rows only)
+        const int c = ((r - t) % P + P) % P;
+        const bool lower = t > r;  // c > r
+        const int rows = lower ? hs : s, keys = (t >= 1 && !lower) ? hs : s, row0 = lower ? hs : 0;
+        FwdParams pb = p;
+        pb.zigzag = 0;
+        pb.P = 1; pb.rank0 = 0; pb.nranks = 1; pb.t_begin = 0; pb.t_count = -1;
+        pb.Sq = rows; pb.Sk = keys;
+        pb.q = (const char*)q + ((int64_t)r * s + row0) * p.qs.s * esz;
+        pb.k = (const char*)k + (int64_t)c * s * p.ks.s * esz;
+        pb.v = (const char*)v + (int64_t)c * s * p.vs.s * esz;
+        pb.causal = t == 0;
+        pb.epi = SPA_EPI_PLAIN;
+        pb.out = blk_out; pb.os = as; pb.lse = blk_lse; pb.lse_bh = rows;
+        e = spa_launch_flash_fwd(pb, D, dtype, st);
+        float* lser = lse + (int64_t)r * s;
+        if (e == hipSuccess)
+          e = spa_launch_merge(acc + (int64_t)row0 * as.s, lser + row0, blk_out, blk_lse, B, H, rows, D, as, as, SPA_F32, t == 0, S, st);
+        if (e == hipSuccess && t + 1 == nsteps)
+          e = spa_launch_finalize((char*)out + (int64_t)r * s * p.os.s * esz, acc, B, H, s, D, p.os, as, SPA_F32, st);
       } else {
         // fp32: one plain block pair per launch on explicit chunk pointers, merged by the stand-alone kernels
         const int c = ((r - t) % P + P) % P;

@@ -50,6 +50,14 @@ struct FwdParams {
   // V = v8 * v_scale[b*H + h], fp32, one per (batch or sequence, head); strides of k, v in bytes
   const float* k_scale;
   const float* v_scale;
+  // zigzag sharding of a causal ring (16-bit kernels; 0: contiguous chunks): the chunk of rank r holds
+  // half-chunks r and 2P-1-r of the sequence, Sq/2 rows each.  Step 0 is plain causal attention on the
+  // rank's own chunk; at step t >= 1 (chunk c = (r - t) mod P) every local query sees the first half of
+  // the chunk when c < r, and only the second half of the queries sees anything, the whole chunk, when
+  // c > r.  Query tiles never straddle the two halves.  zz_half = 1: the launch covers the tiles of
+  // the second half only (a step with c > r that is not the rank's last).
+  int zigzag = 0;
+  int zz_half = 0;
 };
 
 // Layout of the ring-step slots of one rank in the caller's workspace (16-bit inputs, ring of P):

@@ -176,12 +176,14 @@ RING_FUSE = {"step": _lib.SPA_RING_PER_STEP, "rank": _lib.SPA_RING_PER_RANK, "al
 
 
 def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layout="bshd", out=None, lse=None,
-             workspace=None, fuse="rank", static_scratch=False, k_scale=None, v_scale=None):
+             workspace=None, fuse="rank", static_scratch=False, k_scale=None, v_scale=None, sharding="contiguous"):
     """Simulated ring forward of one rank (or all, rank=-1) over the full-sequence q,k,v: one C call
     that enqueues the kernels in ring order.  Calls spa_ring_fwd.  `fuse`: "step" = one launch per
     (q chunk, kv chunk) pair, "rank" = one launch per rank walking its chunks, "all" = one launch.
     Returns (out like q, lse fp32 [B,H,S]); with rank >= 0 only that rank's rows are written.
     k, v may be torch.float8_e4m3fn with k_scale, v_scale fp32 [B,H] (spa_ring_fwd_fp8kv).
+    sharding="zigzag": the rows of q, k, v are in zigzag-sharded order (chunk r of the tensors holds
+    half-chunks r and 2P-1-r of the sequence); out and lse come back in the same order.
     static_scratch=True calls spa_ring_fwd_static instead: no workspace tensor, the library's built-in
     32 MiB buffer holds a rank's earlier block results between step launches (for callers that must not allocate;
     calls that overlap on one device race)."""
@@ -211,6 +213,8 @@ def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layo
         lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
     if fuse not in RING_FUSE:
         raise ValueError(f"fuse must be one of {sorted(RING_FUSE)}, got {fuse!r}")
+    if sharding not in ("contiguous", "zigzag"):
+        raise ValueError(f"sharding must be 'contiguous' or 'zigzag', got {sharding!r}")
     if static_scratch and workspace is not None:
         raise ValueError("static_scratch=True takes no workspace")
     if workspace is None and not static_scratch and (fuse == "step" or q.dtype == torch.float32):
@@ -219,7 +223,7 @@ def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layo
     tail = (B, H, S, D, int(ring_size), int(rank),
             _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
             float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE,
-            _dtype_code(q), RING_FUSE[fuse], _stream())
+            _dtype_code(q), RING_FUSE[fuse] | (_lib.SPA_RING_ZIGZAG if sharding == "zigzag" else 0), _stream())
     with _on(q.device):
         if fp8:
             ksc, vsc = _fp8_scales(k, v, k_scale, v_scale, B, H)

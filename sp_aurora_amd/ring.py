@@ -14,6 +14,11 @@ Additive, keyword-only extensions of the reference signatures:
     ring_size=P   split the given sequence into P contiguous shards and run every rank
                   (ring_size=1 is the reference's single-process path: one block over the
                   whole sequence, sp_aurora/intel_ring_flash_attn.py:415-435).
+    sharding="zigzag"   the rows of the given tensors are in zigzag-sharded order (zigzag_order):
+                  shard r holds half-chunks r and 2P-1-r of the sequence, so that every rank of a
+                  causal ring has the same work; the sharding the reference's test names without
+                  shipping it (test/flash_attention/test_intel_ring_flash_attn_varlen.py:25,205-215).
+                  Results (and gradients) come back in the same row order.
 """
 import torch
 import torch.distributed as dist
@@ -22,7 +27,7 @@ from . import ops
 from .flash_attn import _check_unsupported
 
 __all__ = [
-    "ring_flash_attn_forward_rank", "ring_flash_attn_forward", "ring_flash_attn_backward", "make_ring_forward_step",
+    "zigzag_order", "ring_flash_attn_forward_rank", "ring_flash_attn_forward", "ring_flash_attn_backward", "make_ring_forward_step",
     "RingFlashAttnFunc", "IntelRingFlashAttnFunc",
     "ring_flash_attn_func", "ring_flash_attn_kvpacked_func", "ring_flash_attn_qkvpacked_func",
     "intel_ring_flash_attn_func", "intel_ring_flash_attn_kvpacked_func", "intel_ring_flash_attn_qkvpacked_func",
@@ -35,6 +40,26 @@ def _no_multi_gpu(group):
         raise NotImplementedError(
             "this build runs the ring on one GPU (ring_size=P simulates the P ranks); "
             "process groups / multi-GPU rings are not part of it")
+
+
+def zigzag_order(S, ring_size, device=None):
+    """Row order of zigzag shards: idx (int64 [S]) with sharded = natural.index_select(1, idx).  The S rows
+    are cut into 2P half-chunks; shard r is half-chunk r followed by half-chunk 2P-1-r."""
+    P = int(ring_size)
+    if P < 1 or S % (2 * P):
+        raise ValueError(f"zigzag sharding needs 2 * ring_size = {2 * P} to divide the sequence length {S}")
+    hc = S // (2 * P)
+    halves = torch.arange(2 * P, device=device).view(2, P)
+    order = torch.stack([halves[0], halves[1].flip(0)], dim=1).reshape(-1)  # r, 2P-1-r for r = 0 .. P-1
+    return (order[:, None] * hc + torch.arange(hc, device=device)[None, :]).reshape(-1)
+
+
+def _check_sharding(sharding, S, P):
+    if sharding not in ("contiguous", "zigzag"):
+        raise ValueError(f"sharding must be 'contiguous' or 'zigzag', got {sharding!r}")
+    if sharding == "zigzag" and S % (2 * P):
+        raise ValueError(f"zigzag sharding needs 2 * ring_size = {2 * P} to divide the sequence length {S}")
+    return sharding == "zigzag"
 
 
 class _RingWorkspace:
@@ -83,22 +108,24 @@ def ring_flash_attn_forward_rank(q_local, k_chunks, v_chunks, rank, softmax_scal
 
 
 def ring_flash_attn_forward(q, k, v, softmax_scale=None, causal=False, ring_size=1, out=None, lse=None,
-                            workspace=None, fuse="rank"):
+                            workspace=None, fuse="rank", sharding="contiguous"):
     """All ranks of a simulated ring over contiguous shards of q,k,v [B,S,H,D]: one call into the
     C ring driver, which enqueues the block-pair kernels in ring order and merges each step in the
     kernel epilogue.  Returns out [B,S,H,D] (q dtype) and lse fp32 [B,H,S]; `out`, `lse`,
-    `workspace` (ops.ring_fwd_workspace) may be passed in to run without allocating."""
+    `workspace` (ops.ring_fwd_workspace) may be passed in to run without allocating.
+    sharding="zigzag": the rows are in zigzag-sharded order (see the module docstring)."""
     B, S, H, D = q.shape
     P = int(ring_size)
     if P < 1 or S % P or (P > 1 and k.shape[1] != S):
         raise ValueError(f"ring_size={P} must divide the sequence length {S} (and k/v must match q)")
+    _check_sharding(sharding, S, P)
     if P == 1:
         return ops.flash_fwd(q, k, v, softmax_scale, causal, layout="bshd", out=out, lse=lse)
     return ops.ring_fwd(q, k, v, P, softmax_scale, causal, rank=-1, layout="bshd", out=out, lse=lse,
-                        workspace=workspace, fuse=fuse)
+                        workspace=workspace, fuse=fuse, sharding=sharding)
 
 
-def make_ring_forward_step(q, k, v, softmax_scale=None, causal=False, ring_size=1, fuse="rank"):
+def make_ring_forward_step(q, k, v, softmax_scale=None, causal=False, ring_size=1, fuse="rank", sharding="contiguous"):
     """Preallocates every buffer ring_flash_attn_forward needs and returns a zero-argument
     callable that runs the whole ring forward into them and returns (out, lse)."""
     B, S, H, D = q.shape
@@ -108,13 +135,24 @@ def make_ring_forward_step(q, k, v, softmax_scale=None, causal=False, ring_size=
     ws = ops.ring_fwd_workspace(q, P) if P > 1 else None
 
     def step():
-        return ring_flash_attn_forward(q, k, v, softmax_scale, causal, P, out=out, lse=lse, workspace=ws, fuse=fuse)
+        return ring_flash_attn_forward(q, k, v, softmax_scale, causal, P, out=out, lse=lse, workspace=ws, fuse=fuse,
+                                       sharding=sharding)
 
     return step
 
 
+def _zigzag_pairs(P):
+    """The block pairs of a causal zigzag ring, in the ring's order: (rank, chunk, query rows, key rows,
+    masked) with rows as 'all', 'first' or 'second' half of the shard."""
+    for r in range(P):
+        yield r, r, "all", "all", True
+        for t in range(1, P):
+            c = (r - t) % P
+            yield (r, c, "all", "first", False) if c < r else (r, c, "second", "all", False)
+
+
 def ring_flash_attn_backward(dout, q, k, v, out, softmax_lse, softmax_scale=None, causal=False, ring_size=1,
-                             fuse="all"):
+                             fuse="all", sharding="contiguous"):
     """dq, dk, dv of ring attention by block-wise recompute with the global lse.
 
     The schedule is the reference's (sp_aurora/intel_ring_flash_attn.py:192-271): per visited
@@ -128,13 +166,35 @@ def ring_flash_attn_backward(dout, q, k, v, out, softmax_lse, softmax_scale=None
     walks the same pairs inside one launch of each kernel (the blocks of a simulated ring tile
     the causal / full score matrix exactly, and with a shared global lse their sum is the
     backward of attention over the whole sequence), accumulators in registers.
+
+    sharding="zigzag" (rows in zigzag-sharded order, causal): fuse="step" launches the zigzag ring's
+    block pairs (own shard masked; all rows x first half of an earlier rank's shard; second half of
+    the rows x a later rank's whole shard); fuse="all" brings the rows into natural order with one
+    gather per tensor, runs the one-launch backward there and scatters the gradients back.
     """
     if fuse not in ("step", "all"):
         raise ValueError(f"fuse must be 'step' or 'all', got {fuse!r}")
     B, S, H, D = q.shape
     P = int(ring_size)
+    zig = _check_sharding(sharding, S, P) and causal and P > 1
     lse = softmax_lse if softmax_lse.is_contiguous() else softmax_lse.contiguous()
+    if zig and fuse == "all":
+        idx = zigzag_order(S, P, q.device)
+        inv = torch.argsort(idx)
+        nat = lambda t: t.index_select(1, inv)
+        grads = ring_flash_attn_backward(nat(dout), nat(q), nat(k), nat(v), nat(out), lse.index_select(2, inv), softmax_scale,
+                                         True, P, fuse="all")
+        return tuple(g.index_select(1, idx) for g in grads)
     delta = ops.bwd_delta(out, dout, layout="bshd")
+    if zig:
+        dq, dk, dv = (torch.zeros((B, S, H, D), dtype=torch.float32, device=q.device) for _ in range(3))
+        s, hs = S // P, S // (2 * P)
+        rows = lambda r, part: slice(r * s + (hs if part == "second" else 0), r * s + (hs if part == "first" else s))
+        for r, c, qpart, kpart, masked in _zigzag_pairs(P):
+            qs, ks = rows(r, qpart), rows(c, kpart)
+            ops.flash_bwd(q[:, qs], k[:, ks], v[:, ks], dout[:, qs], lse[:, :, qs].contiguous(), delta[:, :, qs].contiguous(),
+                          dq[:, qs], dk[:, ks], dv[:, ks], softmax_scale, masked, layout="bshd")
+        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype)
     if P == 1 or fuse == "all":
         # one launch of each kernel computes the whole gradient: written in q's dtype, no fp32 accumulators
         return ops.flash_bwd_out(q, k, v, dout, lse, delta, softmax_scale, causal, layout="bshd")
@@ -161,16 +221,17 @@ class RingFlashAttnFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, dropout_p, softmax_scale, causal, window_size, alibi_slopes, deterministic,
-                return_softmax, group, ring_size=1):
+                return_softmax, group, ring_size=1, sharding="contiguous"):
         if softmax_scale is None:
             softmax_scale = q.shape[-1] ** (-0.5)
         _check_unsupported(dropout_p, window_size, alibi_slopes)
         _no_multi_gpu(group)
-        out, softmax_lse = ring_flash_attn_forward(q, k, v, softmax_scale, causal, ring_size)
+        out, softmax_lse = ring_flash_attn_forward(q, k, v, softmax_scale, causal, ring_size, sharding=sharding)
         ctx.save_for_backward(q, k, v, out, softmax_lse)
         ctx.softmax_scale = softmax_scale
         ctx.causal = causal
         ctx.ring_size = ring_size
+        ctx.sharding = sharding
         ctx.mark_non_differentiable(softmax_lse)
         return out if not return_softmax else (out, softmax_lse, None)
 
@@ -178,8 +239,8 @@ class RingFlashAttnFunc(torch.autograd.Function):
     def backward(ctx, dout, *args):
         q, k, v, out, softmax_lse = ctx.saved_tensors
         dq, dk, dv = ring_flash_attn_backward(dout, q, k, v, out, softmax_lse, ctx.softmax_scale, ctx.causal,
-                                              ctx.ring_size)
-        return dq, dk, dv, None, None, None, None, None, None, None, None, None
+                                              ctx.ring_size, sharding=ctx.sharding)
+        return dq, dk, dv, None, None, None, None, None, None, None, None, None, None
 
 
 IntelRingFlashAttnFunc = RingFlashAttnFunc
@@ -187,28 +248,28 @@ IntelRingFlashAttnFunc = RingFlashAttnFunc
 
 def ring_flash_attn_qkvpacked_func(qkv, dropout_p=0.0, softmax_scale=None, causal=False, window_size=(-1, -1),
                                    alibi_slopes=None, deterministic=False, return_attn_probs=False, group=None,
-                                   *, ring_size=1):
+                                   *, ring_size=1, sharding="contiguous"):
     """qkv [B,S,3,H,D]; the strided views qkv[:, :, i] go to the kernels as they are
     (sp_aurora/intel_ring_flash_attn.py:344-368)."""
     return RingFlashAttnFunc.apply(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], dropout_p, softmax_scale, causal,
-                                   window_size, alibi_slopes, deterministic, return_attn_probs, group, ring_size)
+                                   window_size, alibi_slopes, deterministic, return_attn_probs, group, ring_size, sharding)
 
 
 def ring_flash_attn_kvpacked_func(q, kv, dropout_p=0.0, softmax_scale=None, causal=False, window_size=(-1, -1),
                                   alibi_slopes=None, deterministic=False, return_attn_probs=False, group=None,
-                                  *, ring_size=1):
+                                  *, ring_size=1, sharding="contiguous"):
     """q [B,S,H,D], kv [B,S,2,H,D] (sp_aurora/intel_ring_flash_attn.py:371-396)."""
     return RingFlashAttnFunc.apply(q, kv[:, :, 0], kv[:, :, 1], dropout_p, softmax_scale, causal, window_size,
-                                   alibi_slopes, deterministic, return_attn_probs, group, ring_size)
+                                   alibi_slopes, deterministic, return_attn_probs, group, ring_size, sharding)
 
 
 def ring_flash_attn_func(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, window_size=(-1, -1),
                          alibi_slopes=None, deterministic=False, return_attn_probs=False, group=None,
-                         *, ring_size=1):
+                         *, ring_size=1, sharding="contiguous"):
     """q,k,v [B,S,H,D] -> out [B,S,H,D], or (out, lse fp32 [B,H,S], None) with return_attn_probs
     (sp_aurora/intel_ring_flash_attn.py:399-449)."""
     return RingFlashAttnFunc.apply(q, k, v, dropout_p, softmax_scale, causal, window_size, alibi_slopes,
-                                   deterministic, return_attn_probs, group, ring_size)
+                                   deterministic, return_attn_probs, group, ring_size, sharding)
 
 
 # names the reference package exports (sp_aurora/__init__.py:59-63) and its own

@@ -139,7 +139,7 @@ def test_public_signatures_match_the_reference():
                      (spa.ring_flash_attn_qkvpacked_func, ["qkv"])):
         sig = inspect.signature(fn)
         names = list(sig.parameters)
-        assert names == head + base + ["ring_size"]
+        assert names == head + base + ["ring_size", "sharding"]
         assert sig.parameters["ring_size"].kind is inspect.Parameter.KEYWORD_ONLY
         assert sig.parameters["dropout_p"].default == 0.0
         assert sig.parameters["causal"].default is False

@@ -70,6 +70,7 @@ def spot_check_rows(out_h, lse_h, q_h, k_h, v_h, scale, causal, what, n_rows=24,
 
 def assert_out(got, want, what):
     got, want = got.float(), want.float()
+    assert torch.isfinite(got).all(), f"{what}: non-finite values"
     bad = (got - want).abs() > OUT_ATOL + OUT_RTOL * want.abs()
     assert not bad.any(), f"{what}: {int(bad.sum())} out of tolerance, max abs err {(got - want).abs().max().item():.3e}"
 

@@ -30,6 +30,7 @@ def check_out(got, want, dtype, what="out"):
     want = want.to(torch.float64)
     assert got.shape == want.shape, (what, got.shape, want.shape)
     tol = OUT_TOL[dtype]
+    assert torch.isfinite(got).all(), f"{what}: {int((~torch.isfinite(got)).sum())} non-finite values"
     bad = (got - want).abs() > tol["atol"] + tol["rtol"] * want.abs()
     assert not bad.any(), f"{what}: {int(bad.sum())} elements out of tolerance, max abs err {(got - want).abs().max():.3e}"
 

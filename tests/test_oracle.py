@@ -183,6 +183,39 @@ def test_ring_schedule_visits_chunks_in_ring_order():
         assert torch.allclose(out, torch.full_like(out, (1 + 2 + 3 + 4) / 4))
 
 
+@pytest.mark.parametrize("P", [1, 2, 3, 4])
+def test_zigzag_ring_equals_full_causal_attention_after_unpermuting(P):
+    """The zigzag schedule against the closed form: shard the rows (rank r gets half-chunks r and
+    2P-1-r), run the ring, undo the permutation, compare with full causal attention in natural order.
+    A wrong half, a wrong comparison (c < rank) or a merge into the wrong rows fails it."""
+    S = 8 * P
+    q, k, v = rand_qkv((2, S, 3, 8), 31, F64)
+    idx = O.zigzag_order(S, P)
+    assert sorted(idx.tolist()) == list(range(S))
+    hc = S // (2 * P)
+    for r in range(P):  # rank r's shard = half-chunk r, then half-chunk 2P-1-r
+        assert idx[2 * hc * r:2 * hc * (r + 1)].tolist() == list(range(r * hc, (r + 1) * hc)) + list(range((2 * P - 1 - r) * hc, (2 * P - r) * hc))
+    f_out, f_lse = O.full_attention(q, k, v, None, True)
+    z_out, z_lse = O.ring_forward_zigzag(q[:, idx], k[:, idx], v[:, idx], P, None)
+    inv = torch.argsort(idx)
+    assert torch.allclose(z_out[:, inv], f_out, atol=1e-12)
+    assert torch.allclose(z_lse[:, :, inv], f_lse, atol=1e-12)
+
+
+def test_zigzag_ring_balances_the_work_of_the_ranks():
+    """Counting with tagged values: keys are zero (every visible key weighs the same), so exp(lse) of a
+    row is the number of keys it sees; per rank these sum to the same total, P * s * s / 2 + s / 2."""
+    P, s = 4, 4
+    S = P * s
+    q = torch.zeros(1, S, 1, 2, dtype=F64)
+    _, lse = O.ring_forward_zigzag(q, q, q, P, 1.0)
+    seen = torch.exp(lse[0, 0]).view(P, s).sum(1)
+    assert torch.allclose(seen, torch.full((P,), P * s * s / 2 + s / 2, dtype=F64))
+    # and a row at natural position n sees n + 1 keys
+    idx = O.zigzag_order(S, P)
+    assert torch.allclose(torch.exp(lse[0, 0]), (idx + 1).to(F64))
+
+
 def test_packed_equals_unpacked():
     """test/test_ring_attention_comprehensive.py:205-218."""
     qkv = rand((1, 8, 3, 2, 4), 31, F64)
