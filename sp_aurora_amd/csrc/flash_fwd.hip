@@ -91,7 +91,8 @@ __device__ __forceinline__ int v_swizzle(int row) {
 // the barrier at which the direct loads of the 16-bit form are waited for.)
 // FINALN: the variant for a rank's last ring step (epilogue SPA_EPI_FINALN); the others write a
 // block result as it is (SPA_EPI_PLAIN / SPA_EPI_PART).
-template <typename T, int D, int NG, bool SHARE, bool KV8 = false, bool FINALN = false>
+// ZZ: the variant for zigzag shards (FwdParams::zigzag); the others carry none of its bookkeeping.
+template <typename T, int D, int NG, bool SHARE, bool KV8 = false, bool FINALN = false, bool ZZ = false>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams pk) {
   static_assert(!(FINALN && SHARE), "the merging epilogue goes with 128-row workgroups");
   typedef typename std::conditional<KV8, unsigned char, T>::type KVT;  // element type of K / V in memory
@@ -125,7 +126,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const int rank = p.rank0 + p.nranks - 1 - (int)blockIdx.z;
   // Zigzag shards: the tiles of the two halves of the chunk are laid out one half after the other (a tile
   // never holds rows of both), the second (heavier) half first in dispatch order.
-  const bool zz = p.zigzag != 0;
+  constexpr bool zz = ZZ;
   const int zz_hs = p.Sq >> 1;                                    // rows per half-chunk
   const int zz_nqh = p.zz_half ? p.nqt : p.nqt >> 1;              // tiles per half
   const bool zhalf = zz && (p.zz_half || qt >= zz_nqh);           // this workgroup's rows lie in the second half
@@ -198,7 +199,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const int n_hsteps = t_half_end > t_full0 ? t_half_end - t_full0 : 0;
   const int n_fsteps = t_end - t_full0 - n_hsteps > 0 ? t_end - t_full0 - n_hsteps : 0;
   const int n = n_diag + n_hsteps * npc_h + n_fsteps * npc;
-  if constexpr (FINALN) {
+  if constexpr (FINALN && ZZ) {
     if (n == 0) {
       // The launch of a zigzag rank's last step, first half of the rows: no block here (their last block was
       // step `rank`), so the workgroup only applies update_out_and_lse (sp_aurora/utils.py:103-104) to the
@@ -506,7 +507,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       // (a lane whose row has seen no key yet, here or before, while another row of the wave asks for the
       // rescale: -inf - -inf; nothing of that row needs scaling.  Rows of a wave differ in this only when
       // the tile's first row is not a multiple of the sub-tile size: the second half of a zigzag shard.)
-      const float alpha = m_new == -INFINITY ? 1.f : fast_exp2((m_run - m_new) * c);
+      const float alpha = ZZ && m_new == -INFINITY ? 1.f : fast_exp2((m_run - m_new) * c);
       m_run = m_new;
       l_run *= alpha;
 #pragma unroll
@@ -1104,14 +1105,14 @@ int fwd_tiles(const FwdParams& p, int bm) {
 // Two wave groups once there are at least two 64-key sub-tiles to split; 256-row workgroups with
 // shared K/V buffers once that still leaves every CU at least two workgroups.  spa_tune() can
 // force either choice (experiments and tests).
-template <typename T, int D>
+template <typename T, int D, bool ZZ>
 hipError_t launch16(FwdParams p, hipStream_t stream) {
   const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
   const int force_share = spa_knob(SPA_KNOB_FWD_SHARE);
   const bool two = force ? force == 2 : p.Sk > fwd_bn<D>();
   if (p.epi == SPA_EPI_FINALN) {
-    if (two) return launch<flash_fwd16_kernel<T, D, 2, false, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
-    return launch<flash_fwd16_kernel<T, D, 1, false, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+    if (two) return launch<flash_fwd16_kernel<T, D, 2, false, false, true, ZZ>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+    return launch<flash_fwd16_kernel<T, D, 1, false, false, true, ZZ>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
   }
   if (two && D >= 64) {
     const int nqt2 = fwd_tiles(p, 2 * FWD_BM);
@@ -1119,22 +1120,22 @@ hipError_t launch16(FwdParams p, hipStream_t stream) {
     const bool share = force_share ? force_share == 2 : wgs >= 2 * (int64_t)spa_device_cus();
     if (share) {
       p.nqt = nqt2;
-      return launch<flash_fwd16_kernel<T, D, 2, (D >= 64)>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, (D >= 64)>::SMEM, p, stream);
+      return launch<flash_fwd16_kernel<T, D, 2, (D >= 64), false, false, ZZ>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, (D >= 64)>::SMEM, p, stream);
     }
   }
-  if (two) return launch<flash_fwd16_kernel<T, D, 2, false>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
-  return launch<flash_fwd16_kernel<T, D, 1, false>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+  if (two) return launch<flash_fwd16_kernel<T, D, 2, false, false, false, ZZ>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+  return launch<flash_fwd16_kernel<T, D, 1, false, false, false, ZZ>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
 }
 
 // e4m3 K/V: the register-staged variants, chosen like the 16-bit ones.
-template <typename T, int D>
+template <typename T, int D, bool ZZ>
 hipError_t launch16_kv8(FwdParams p, hipStream_t stream) {
   const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
   const int force_share = spa_knob(SPA_KNOB_FWD_SHARE);
   const bool two = force ? force == 2 : p.Sk > fwd_bn<D>();
   if (p.epi == SPA_EPI_FINALN) {
-    if (two) return launch<flash_fwd16_kernel<T, D, 2, false, true, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
-    return launch<flash_fwd16_kernel<T, D, 1, false, true, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+    if (two) return launch<flash_fwd16_kernel<T, D, 2, false, true, true, ZZ>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+    return launch<flash_fwd16_kernel<T, D, 1, false, true, true, ZZ>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
   }
   if (two) {
     const int nqt2 = fwd_tiles(p, 2 * FWD_BM);
@@ -1142,14 +1143,49 @@ hipError_t launch16_kv8(FwdParams p, hipStream_t stream) {
     const bool share = force_share ? force_share == 2 : wgs >= 2 * (int64_t)spa_device_cus();
     if (share) {
       p.nqt = nqt2;
-      return launch<flash_fwd16_kernel<T, D, 2, true, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, true>::SMEM, p, stream);
+      return launch<flash_fwd16_kernel<T, D, 2, true, true, false, ZZ>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, true>::SMEM, p, stream);
     }
   }
-  if (two) return launch<flash_fwd16_kernel<T, D, 2, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
-  return launch<flash_fwd16_kernel<T, D, 1, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+  if (two) return launch<flash_fwd16_kernel<T, D, 2, false, true, false, ZZ>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+  return launch<flash_fwd16_kernel<T, D, 1, false, true, false, ZZ>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+}
+
+// (dtype, D) -> kernel family; the zigzag variants are instantiated beside the plain ones
+template <bool ZZ>
+hipError_t launch16_any(const FwdParams& p, int D, int dtype, hipStream_t stream) {
+  if (p.k_scale) {  // K / V are e4m3 bytes, q / out of type `dtype`
+    if (!p.v_scale) return hipErrorInvalidValue;
+    if (dtype == 1) {
+      if (D == 128) return launch16_kv8<__bf16, 128, ZZ>(p, stream);
+      if (D == 64) return launch16_kv8<__bf16, 64, ZZ>(p, stream);
+    } else if (dtype == 2) {
+      if (D == 128) return launch16_kv8<_Float16, 128, ZZ>(p, stream);
+      if (D == 64) return launch16_kv8<_Float16, 64, ZZ>(p, stream);
+    }
+    return hipErrorInvalidValue;
+  }
+  if (dtype == 1) {
+    if (D == 128) return launch16<__bf16, 128, ZZ>(p, stream);
+    if (D == 64) return launch16<__bf16, 64, ZZ>(p, stream);
+    if (D == 32) return launch16<__bf16, 32, ZZ>(p, stream);
+  } else if (dtype == 2) {
+    if (D == 128) return launch16<_Float16, 128, ZZ>(p, stream);
+    if (D == 64) return launch16<_Float16, 64, ZZ>(p, stream);
+    if (D == 32) return launch16<_Float16, 32, ZZ>(p, stream);
+  }
+  return hipErrorInvalidValue;
 }
 
 }  // namespace
+
+// This file makes two objects: compiled with SPA_FWD_ZIGZAG_UNIT it holds the zigzag variants of the 16-bit
+// kernel and nothing else, without it everything else (so that the two halves compile side by side).
+#ifdef SPA_FWD_ZIGZAG_UNIT
+hipError_t spa_launch_fwd16_zigzag(const FwdParams& p, int D, int dtype, hipStream_t stream) {
+  return launch16_any<true>(p, D, dtype, stream);
+}
+#else
+hipError_t spa_launch_fwd16_zigzag(const FwdParams& p, int D, int dtype, hipStream_t stream);
 
 // Returns hipSuccess, or hipErrorInvalidValue for an unsupported (dtype, D).
 hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream) {
@@ -1167,26 +1203,8 @@ hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t strea
     p.out = (char*)slots.out<char>(p.part, p.part_slot) - row0 * p.os.s * 2;
     p.lse = slots.lse(p.part, p.P, p.part_slot) - row0;
   }
-  if (p.k_scale) {  // K / V are e4m3 bytes, q / out of type `dtype`
-    if (!p.v_scale) return hipErrorInvalidValue;
-    if (dtype == 1) {
-      if (D == 128) return launch16_kv8<__bf16, 128>(p, stream);
-      if (D == 64) return launch16_kv8<__bf16, 64>(p, stream);
-    } else if (dtype == 2) {
-      if (D == 128) return launch16_kv8<_Float16, 128>(p, stream);
-      if (D == 64) return launch16_kv8<_Float16, 64>(p, stream);
-    }
-    return hipErrorInvalidValue;
-  }
-  if (dtype == 1) {
-    if (D == 128) return launch16<__bf16, 128>(p, stream);
-    if (D == 64) return launch16<__bf16, 64>(p, stream);
-    if (D == 32) return launch16<__bf16, 32>(p, stream);
-  } else if (dtype == 2) {
-    if (D == 128) return launch16<_Float16, 128>(p, stream);
-    if (D == 64) return launch16<_Float16, 64>(p, stream);
-    if (D == 32) return launch16<_Float16, 32>(p, stream);
-  } else if (dtype == 0) {
+  if (dtype == 1 || dtype == 2) return p.zigzag ? spa_launch_fwd16_zigzag(p, D, dtype, stream) : launch16_any<false>(p, D, dtype, stream);
+  if (dtype == 0) {
     if (p.epi != SPA_EPI_PLAIN) return hipErrorInvalidValue;  // fp32 ring steps merge with the separate kernel
     if (D == 128) return launch<flash_fwd32_kernel<128>>(FWD_THREADS, Fwd32Cfg<128>::SMEM, p, stream);
     if (D == 64) return launch<flash_fwd32_kernel<64>>(FWD_THREADS, Fwd32Cfg<64>::SMEM, p, stream);
@@ -1194,3 +1212,4 @@ hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t strea
   }
   return hipErrorInvalidValue;
 }
+#endif  // SPA_FWD_ZIGZAG_UNIT

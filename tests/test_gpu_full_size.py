@@ -138,6 +138,29 @@ def test_config3_ring_sweep_all_ranks():
     assert (o_ones.float() - 1).abs().max().item() <= 2 ** -7
 
 
+def test_config3_zigzag_shards_give_the_same_attention():
+    """The config-3 tensors with their rows in zigzag order (rank r holds half-chunks r and 15-r): the three
+    schedules against the contiguous ring on the rows in natural order (itself checked above), eight heads
+    against the on-device fp32 evaluation, float64 rows of one head."""
+    B, S, H, D, P = 1, 8192, 32, 128, 8
+    scale = D ** -0.5
+    q, k, v = config_qkv((B, S, H, D), 2, 0.5)
+    idx = spa.ring.zigzag_order(S, P, DEV)
+    qz, kz, vz = (t.index_select(1, idx) for t in (q, k, v))
+    o_nat, l_nat = spa.ring.ring_flash_attn_forward(q, k, v, scale, True, P, fuse="all")
+    res = {f: spa.ring.ring_flash_attn_forward(qz, kz, vz, scale, True, P, fuse=f, sharding="zigzag") for f in ("step", "rank", "all")}
+    for f, (o, l) in res.items():
+        assert_out(o, o_nat.index_select(1, idx), f"zigzag {f} vs contiguous ring")
+        assert_lse(l, l_nat.index_select(2, idx), f"zigzag {f} vs contiguous ring")
+    inv = torch.argsort(idx)
+    o_all, l_all = res["all"][0].index_select(1, inv), res["all"][1].index_select(2, inv)
+    for h in (1, 5, 10, 14, 19, 23, 28, 30):
+        want_o, want_l = ref_head(q[0, :, h], k[0, :, h], v[0, :, h], scale, True)
+        assert_out(o_all[0, :, h], want_o, f"zigzag all h{h}")
+        assert_lse(l_all[0, h], want_l, f"zigzag all h{h}")
+    spot_check_rows(o_all[0, :, 20], l_all[0, 20], q[0, :, 20], k[0, :, 20], v[0, :, 20], scale, True, "cfg3 zigzag fp64", n_rows=12)
+
+
 # ------------------------------------------------------------------ config 4
 def test_config4_ulysses_relayout_and_attention():
     """bf16 [P=8, B=1, s=2048, H=32, D=128] -> [8, 1, 16384, 4, 128], causal attention, and back."""
@@ -201,6 +224,29 @@ def test_config5_qkvpacked_long_context_forward_backward():
             assert not bad.any(), f"{name} h{h}: {int(bad.sum())} out of tolerance, max err {(got - ref).abs().max().item():.3e} (scale {ref.abs().max().item():.3e})"
         del qh, kh, vh, want_o, want_l
         torch.cuda.empty_cache()
+
+
+def test_config5_zigzag_shards_forward_and_backward():
+    """Config 5's tensors in zigzag order, P = 16: forward (one launch per rank) and both backward forms against
+    the contiguous ring's results on the rows in natural order (checked against fp32 / float64 above)."""
+    B, S, H, D, P = 1, 32768, 16, 128, 16
+    scale = D ** -0.5
+    qkv = randn((B, S, 3, H, D), 4, torch.bfloat16)
+    dout = randn((B, S, H, D), 5, torch.bfloat16)
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+    idx = spa.ring.zigzag_order(S, P, DEV)
+    o_nat, l_nat = spa.ring.ring_flash_attn_forward(q, k, v, scale, True, P, fuse="all")
+    g_nat = spa.ring.ring_flash_attn_backward(dout, q, k, v, o_nat, l_nat, scale, True, P, fuse="all")
+    qz, kz, vz, dz = (t.index_select(1, idx) for t in (q, k, v, dout))
+    oz, lz = spa.ring.ring_flash_attn_forward(qz, kz, vz, scale, True, P, fuse="rank", sharding="zigzag")
+    assert_out(oz, o_nat.index_select(1, idx), "zigzag rank vs contiguous ring")
+    assert_lse(lz, l_nat.index_select(2, idx), "zigzag rank vs contiguous ring")
+    for fuse in ("step", "all"):
+        gz = spa.ring.ring_flash_attn_backward(dz, qz, kz, vz, oz, lz, scale, True, P, fuse=fuse, sharding="zigzag")
+        for name, got, ref in zip(("dq", "dk", "dv"), gz, g_nat):
+            ref = ref.index_select(1, idx).float()
+            bad = (got.float() - ref).abs() > 3e-2 * ref.abs().max() + 3e-2 * ref.abs()
+            assert torch.isfinite(got).all() and not bad.any(), f"zigzag {fuse} {name}: {int(bad.sum())} out of tolerance"
 
 
 # ------------------------------------------------------------------ beyond the configs: a long sequence

@@ -1,5 +1,5 @@
 """A bounded, fixed-seed sweep of random shapes through every entry of the HIP path against the
-float64 oracle: block forward, ring forward in its three schedules, e4m3 K/V (block and ring),
+float64 oracle: block forward, ring forward in its three schedules (contiguous and zigzag shards), e4m3 K/V (block and ring),
 packed variable-length batches, and the three backward forms.  Shapes are drawn from lists that
 straddle the kernels' tile sizes (1, 63..65, 127..130, 255..257, ragged tails) and the
 workgroup-form overrides are drawn as well, so that every kernel variant sees awkward sizes.
@@ -49,7 +49,7 @@ def _case(rng):
     D, H, B = rng.choice([32, 64, 128]), rng.choice([1, 2, 3]), rng.choice([1, 2])
     causal = rng.random() < 0.5
     kind = rng.choice(["block", "block", "ring", "ring_bwd", "fp8", "fp8", "fp8_ring", "varlen", "block_bwd", "block_bwd",
-                       "varlen_bwd", "varlen_bwd"])
+                       "varlen_bwd", "varlen_bwd", "zigzag", "zigzag"])
     share, groups = rng.choice([0, 0, 1, 2, 2]), rng.choice([0, 0, 1, 2])
     _lib.tune("fwd_share", share)
     _lib.tune("fwd_groups", groups)
@@ -75,6 +75,16 @@ def _case(rng):
         o, l = spa.ring.ring_flash_attn_forward(q.to(DEV), k.to(DEV), v.to(DEV), None, causal, P, fuse=fuse)
         _close("out", o, want_o, atol, rtol, info)
         _close("lse", l, want_l, LSE_ATOL, 0, info)
+    elif kind == "zigzag":
+        P, hc, fuse = rng.choice([2, 3, 4, 5]), rng.choice([8, 32, 50, 64, 96, 100, 128, 130]), rng.choice(["step", "rank", "all"])
+        info = (kind, dtype, B, H, P, hc, D, fuse, share, groups)
+        q, k, v = (mk(B, 2 * P * hc, H, D) for _ in range(3))
+        idx = O.zigzag_order(2 * P * hc, P)
+        want_o, want_l = O.full_attention(q, k, v, None, True)
+        o, l = spa.ring.ring_flash_attn_forward(q[:, idx].to(DEV), k[:, idx].to(DEV), v[:, idx].to(DEV), None, True, P, fuse=fuse,
+                                                sharding="zigzag")
+        _close("out", o, want_o[:, idx], atol, rtol, info)
+        _close("lse", l, want_l[:, :, idx], LSE_ATOL, 0, info)
     elif kind == "ring_bwd":
         S = rng.choice([2, 33, 64, 100, 128, 200, 257, 384])
         P = rng.choice([1, 1, 2, 4]) if S % 4 == 0 else 1
