@@ -123,7 +123,6 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const float ksc = KV8 ? p.k_scale[bh] : 1.f;
   const float vsc = KV8 ? p.v_scale[bh] : 1.f;
   const int qt = p.nqt - 1 - (int)blockIdx.y;
-  const int rank = p.rank0 + p.nranks - 1 - (int)blockIdx.z;
   // Zigzag shards: the tiles of the two halves of the chunk are laid out one half after the other (a tile
   // never holds rows of both), the second (heavier) half first in dispatch order.
   constexpr bool zz = ZZ;
@@ -131,6 +130,9 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const int zz_nqh = p.zz_half ? p.nqt : p.nqt >> 1;              // tiles per half
   const bool zhalf = zz && (p.zz_half || qt >= zz_nqh);           // this workgroup's rows lie in the second half
   const int q0 = zz ? (zhalf ? zz_hs : 0) + (qt - (zhalf && !p.zz_half ? zz_nqh : 0)) * C::BMW : qt * C::BMW;
+  // Ranks heaviest first: the last rank with contiguous chunks.  With zigzag shards the second half of a shard's
+  // rows is heavier the lower the rank and the first half the higher, and every grid plane z holds the same work.
+  const int rank = zz && zhalf ? p.rank0 + (int)blockIdx.z : p.rank0 + p.nranks - 1 - (int)blockIdx.z;
   if (p.cu_q) {
     const int q_lo = p.cu_q[b], k_lo = p.cu_k[b];
     p.Sq = p.cu_q[b + 1] - q_lo;
@@ -683,24 +685,36 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   T* const out_bh = (T*)p.out + b * p.os.b + h * p.os.h + qoff * p.os.s;
   const int64_t out_rs = p.os.s;
   float* const lse_bh = p.lse + ((int64_t)b * p.H + h) * p.lse_bh + qoff;
-  if constexpr (SHARE) {
-    // A wave's rows are complete and nothing is merged: straight from the registers.  A lane holds
-    // 4 consecutive head dims per register group and its partner 32 lanes on the next 4; one
-    // v_permlane32_swap per dword pairs them up so that every lane stores 16-byte pieces, the two
-    // lanes of a row side by side.  No LDS round trip, no barrier.
-    const float l_tot = halves_sum(l_run);
-    const float inv = vsc / l_tot;
-    if (hh == 0 && qrow < q_lim) lse_bh[qrow] = (m_run * c + fast_log2(l_tot)) * 0.6931471805599453f;
+  // Rows leave straight from the registers wherever nothing is merged into them (every variant but a rank's
+  // last ring step).  A lane holds 4 consecutive head dims per register group and its partner 32 lanes on the
+  // next 4; one v_permlane32_swap per dword pairs them up so that every lane stores 16-byte pieces, the two
+  // lanes of a row side by side.  `other`: the same rows' partial sums of the other wave group, staged in LDS
+  // in the accumulator's own layout (128 rows of D + 4 floats), or null.
+  auto store_rows = [&](float a_own, auto with_other, const float* other, float a_other, float lse_val) {
+    constexpr bool OTHER = decltype(with_other)::value;
+    if (hh == 0 && qrow < q_lim) lse_bh[qrow] = lse_val;
     T* const orow = out_bh + qrow_c * out_rs;
 #pragma unroll
     for (int db = 0; db < D / 32; ++db)
 #pragma unroll
       for (int gp = 0; gp < 2; ++gp) {
-        unsigned x[2], y[2];  // this lane's 4 dims of the even and of the odd group, as two packed pairs each
+        float e[8];  // this lane's 4 dims of the even and of the odd register group
+#pragma unroll
+        for (int i = 0; i < 8; ++i) e[i] = o[db][8 * gp + i] * a_own;
+        if constexpr (OTHER) {
+          const f32x4 p0 = *(const f32x4*)(other + db * 32 + 8 * (2 * gp) + 4 * hh);
+          const f32x4 p1 = *(const f32x4*)(other + db * 32 + 8 * (2 * gp + 1) + 4 * hh);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            e[i] = __builtin_fmaf(p0[i], a_other, e[i]);
+            e[4 + i] = __builtin_fmaf(p1[i], a_other, e[4 + i]);
+          }
+        }
+        unsigned x[2], y[2];  // as two packed pairs each
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
-          x[k] = M::pack2(o[db][8 * gp + 2 * k] * inv, o[db][8 * gp + 2 * k + 1] * inv);
-          y[k] = M::pack2(o[db][8 * gp + 4 + 2 * k] * inv, o[db][8 * gp + 4 + 2 * k + 1] * inv);
+          x[k] = M::pack2(e[2 * k], e[2 * k + 1]);
+          y[k] = M::pack2(e[4 + 2 * k], e[4 + 2 * k + 1]);
         }
         u32x4 st;
 #pragma unroll
@@ -711,6 +725,47 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         }
         if (qrow < q_lim) *(u32x4*)(orow + db * 32 + 8 * (2 * gp + hh)) = st;
       }
+  };
+  if constexpr (SHARE || (NG == 1 && !FINALN)) {
+    // a wave's rows are complete: no LDS round trip, no barrier
+    const float l_tot = halves_sum(l_run);
+    store_rows(vsc / l_tot, std::false_type{}, nullptr, 0.f, (m_run * c + fast_log2(l_tot)) * 0.6931471805599453f);
+    return;
+  } else if constexpr (!FINALN) {
+    // Two groups hold partial sums of the same rows.  Group 1 stages its unscaled partial O (fp32, its own
+    // register layout) and (m, l) in LDS, free now, and leaves; group 0 weighs both by exp2((m - m_all) c) / l_all
+    // and stores the rows from its registers.  One barrier, one staged tile.
+    constexpr int TP = D + 4;  // floats per staged row
+    float* const tile = (float*)smem;
+    float* const ml = tile + FWD_BM * TP;  // [128](m, l) of group 1
+    const int rloc = w * 32 + ln;
+    const float l_own = halves_sum(l_run);
+    if (grp == 1) {
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f32x4 st;
+          st[0] = o[db][4 * g + 0];
+          st[1] = o[db][4 * g + 1];
+          st[2] = o[db][4 * g + 2];
+          st[3] = o[db][4 * g + 3];
+          *(f32x4*)(tile + rloc * TP + db * 32 + 8 * g + 4 * hh) = st;
+        }
+      if (hh == 0) {
+        ml[rloc * 2] = m_run;
+        ml[rloc * 2 + 1] = l_own;
+      }
+    }
+    __syncthreads();
+    if (grp == 1) return;
+    const float m2 = ml[rloc * 2], l2 = ml[rloc * 2 + 1];
+    const float m_all = fmaxf(m_run, m2);  // finite: some group has seen key 0 of the first chunk
+    const float a1 = fast_exp2((m_run - m_all) * c);
+    const float a2 = fast_exp2((m2 - m_all) * c);
+    const float l_all = l_own * a1 + l2 * a2;
+    const float sc = vsc / l_all;
+    store_rows(a1 * sc, std::true_type{}, tile + rloc * TP, a2 * sc, (m_all * c + fast_log2(l_all)) * 0.6931471805599453f);
     return;
   } else {
     constexpr int TP = D + 4;  // floats per staged row
