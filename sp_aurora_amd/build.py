@@ -10,15 +10,18 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libsp_aurora_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-# (source, object, extra flags).  flash_fwd.hip makes two objects: the zigzag variants of the 16-bit forward kernel
-# are a translation unit of their own, so that the two halves of the longest compile run side by side.
+# (source, object, extra flags).  flash_fwd.hip makes three objects: the zigzag variants of the 16-bit forward kernel
+# and the variants for tensors of 2 GiB and more per (batch, head) are translation units of their own, so that the
+# parts of the longest compile run side by side; flash_bwd.hip likewise makes two.
 # The forward kernels' softmax phase gains 1-3 % from the scheduler that maximises instruction-level
 # parallelism; the backward kernels lose 2 % with it.
 _FWD = ["-mllvm", "-amdgpu-sched-strategy=max-ilp"]
 UNITS = [
     ("flash_fwd.hip", "flash_fwd.o", _FWD),
     ("flash_fwd.hip", "flash_fwd_zigzag.o", _FWD + ["-DSPA_FWD_ZIGZAG_UNIT"]),
+    ("flash_fwd.hip", "flash_fwd_big.o", _FWD + ["-DSPA_FWD_BIG_UNIT"]),
     ("flash_bwd.hip", "flash_bwd.o", []),
+    ("flash_bwd.hip", "flash_bwd_big.o", ["-DSPA_BWD_BIG_UNIT"]),
     ("spa_abi.hip", "spa_abi.o", []),
     ("merge.hip", "merge.o", []),
     ("relayout.hip", "relayout.o", []),

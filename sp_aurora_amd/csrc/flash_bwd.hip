@@ -84,14 +84,20 @@ struct TileReads {
 
 // Global side of the direct loads: thread tid owns 16-byte slot tid of every round of 256 slots;
 // round j covers rows j * RPD + tid / CPR.  Slot (row, pos) receives chunk pos ^ swizzle(row).
-template <typename T, int D, int THREADS = BWD_THREADS>
+// BIG: the tensor's rows of one (batch, head) may span 2 GiB or more; the descriptor is re-based per tile
+// (buffer_window) instead of covering the whole tensor.
+template <typename T, int D, int THREADS = BWD_THREADS, bool BIG = false>
 struct TileLoader {
   u32x4 rsrc;
   unsigned lane_off;  // bytes
   unsigned row_b;     // bytes per tensor row
+  const T* base_;             // BIG only
+  unsigned long long total_;  // BIG only: bytes from base_ to the end of the last row
   __device__ __forceinline__ void init(const T* base, int64_t row_stride, int rows, int tid) {
     typedef BwdCfg<D, THREADS> C;
-    rsrc = buffer_descriptor(base, (unsigned)((((int64_t)rows - 1) * row_stride + D) * (int64_t)sizeof(T)));
+    total_ = (unsigned long long)((((int64_t)rows - 1) * row_stride + D) * (int64_t)sizeof(T));
+    base_ = base;
+    rsrc = buffer_descriptor(base, BIG ? 0u : (unsigned)total_);  // (BIG: an empty range, for tiles that are not wanted)
     const int drow = tid / C::CPR, dpos = tid % C::CPR;
     lane_off = (unsigned)((drow * row_stride + ((dpos ^ tile_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(T));
     row_b = (unsigned)(row_stride * (int64_t)sizeof(T));
@@ -99,6 +105,13 @@ struct TileLoader {
   // round q of the tile whose first tensor row is row0 (on = false: store zeros) into LDS at lds_wave
   __device__ __forceinline__ void load(int q, bool on, int row0, unsigned lds_wave) const {
     typedef BwdCfg<D, THREADS> C;
+    if constexpr (BIG) {
+      unsigned rel = OFF_NONE;
+      u32x4 rs = rsrc;
+      if (on) rs = buffer_window(base_, total_, (unsigned long long)(unsigned)row0 * row_b, rel);
+      load_to_lds_b128(rs, lane_off + rel + (unsigned)(q * C::RPD) * row_b, lds_wave + q * (THREADS * 16));
+      return;
+    }
     const unsigned u = on ? (unsigned)(row0 + q * C::RPD) * row_b : OFF_NONE;
     load_to_lds_b128(rsrc, lane_off + u, lds_wave + q * (THREADS * 16));
   }
@@ -215,7 +228,7 @@ __device__ __forceinline__ void zero_grad_row(E* rowp, int hh) {
     }
 }
 
-template <typename T, int D, int NW>
+template <typename T, int D, int NW, bool BIG = false>
 __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParams pk) {
   BwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
   typedef BwdCfg<D, NW * 64> C;
@@ -271,7 +284,7 @@ __global__ void __launch_bounds__(NW * 64, 1) flash_bwd_dq_kernel(const BwdParam
   const int kv_end = p.causal ? (q0 + NW * 32 < p.Sk ? q0 + NW * 32 : p.Sk) : p.Sk;
   const int nt = (kv_end + BWD_ROWS - 1) / BWD_ROWS;  // key tiles this workgroup visits
 
-  TileLoader<T, D, NW * 64> kld, vld;
+  TileLoader<T, D, NW * 64, BIG> kld, vld;
   kld.init(kp, p.ks.s, p.Sk, tid);
   vld.init(vp, p.vs.s, p.Sk, tid);
   TileReads<D> rd;
@@ -490,7 +503,7 @@ struct DkvCfg {
 
 // ASM = false: the D = 128 kernel with every MFMA left to the compiler (its uniform accumulator
 // form, its own hazard handling): slower, kept as the test twin of the hand-issued form.
-template <typename T, int D, bool ASM = true>
+template <typename T, int D, bool ASM = true, bool BIG = false>
 __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const BwdParams pk) {
   BwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
   typedef BwdCfg<D> C;
@@ -544,7 +557,7 @@ __global__ void __launch_bounds__(BWD_THREADS, 1) flash_bwd_dkdv_kernel(const Bw
   const int it0 = p.causal ? k0 / BWD_ROWS : 0;
   const int nt = (p.Sq + BWD_ROWS - 1) / BWD_ROWS;  // query tiles it0 .. nt-1 are visited
 
-  TileLoader<T, D> qld, dold;
+  TileLoader<T, D, BWD_THREADS, BIG> qld, dold;
   qld.init(qp, p.qs.s, p.Sq, tid);
   dold.init(dop, p.dos.s, p.Sq, tid);
   // per-row statistics: waves 0, 2 fetch the tile's 64 lse values, waves 1, 3 its 64 delta values
@@ -1145,12 +1158,39 @@ hipError_t launch_both(const BwdParams& p, hipStream_t stream) {
   return launch<flash_bwd_dkdv_kernel<T, D>>(DkvCfg<D>::SMEM, kblocks, p, stream);
 }
 
+// A tensor of 2 GiB or more per (batch, head): the re-based variants, 128-row dq workgroups.
+template <typename T, int D>
+hipError_t launch_both_big(const BwdParams& p, hipStream_t stream) {
+  const hipError_t e = launch<flash_bwd_dq_kernel<T, D, 4, true>>(DqCfg<D, 4>::SMEM, (unsigned)((int64_t)p.B * p.H * p.nqt), p, stream);
+  if (e != hipSuccess) return e;
+  return launch<flash_bwd_dkdv_kernel<T, D, true, true>>(DkvCfg<D>::SMEM, (unsigned)((int64_t)p.B * p.H * p.nkt), p, stream);
+}
+
 }  // namespace
+
+// This file makes two objects: compiled with SPA_BWD_BIG_UNIT it holds the re-based variants of the 16-bit kernels
+// and nothing else, without it everything else (so that the two parts compile side by side).
+#ifdef SPA_BWD_BIG_UNIT
+hipError_t spa_launch_bwd16_big(const BwdParams& p, int D, int dtype, hipStream_t stream) {
+  if (dtype == 1) {
+    if (D == 128) return launch_both_big<__bf16, 128>(p, stream);
+    if (D == 64) return launch_both_big<__bf16, 64>(p, stream);
+    if (D == 32) return launch_both_big<__bf16, 32>(p, stream);
+  } else if (dtype == 2) {
+    if (D == 128) return launch_both_big<_Float16, 128>(p, stream);
+    if (D == 64) return launch_both_big<_Float16, 64>(p, stream);
+    if (D == 32) return launch_both_big<_Float16, 32>(p, stream);
+  }
+  return hipErrorInvalidValue;
+}
+#else
+hipError_t spa_launch_bwd16_big(const BwdParams& p, int D, int dtype, hipStream_t stream);
 
 // Returns hipSuccess, or hipErrorInvalidValue for an unsupported (dtype, D).
 hipError_t spa_launch_flash_bwd(BwdParams p, int D, int dtype, hipStream_t stream) {
   p.nqt = (p.Sq + 127) / 128;
   p.nkt = (p.Sk + 127) / 128;
+  if (p.big && dtype != 0) return spa_launch_bwd16_big(p, D, dtype, stream);
   if (dtype == 1) {
     if (D == 128) return launch_both<__bf16, 128>(p, stream);
     if (D == 64) return launch_both<__bf16, 64>(p, stream);
@@ -1173,3 +1213,4 @@ hipError_t spa_launch_flash_bwd(BwdParams p, int D, int dtype, hipStream_t strea
   }
   return hipErrorInvalidValue;
 }
+#endif  // SPA_BWD_BIG_UNIT

@@ -92,7 +92,9 @@ __device__ __forceinline__ int v_swizzle(int row) {
 // FINALN: the variant for a rank's last ring step (epilogue SPA_EPI_FINALN); the others write a
 // block result as it is (SPA_EPI_PLAIN / SPA_EPI_PART).
 // ZZ: the variant for zigzag shards (FwdParams::zigzag); the others carry none of its bookkeeping.
-template <typename T, int D, int NG, bool SHARE, bool KV8 = false, bool FINALN = false, bool ZZ = false>
+// BIG: the variant for K / V whose rows of one (batch, head) span 2 GiB or more: the buffer descriptors are
+// re-based per sub-tile (a few scalar instructions per tile that the others do without).
+template <typename T, int D, int NG, bool SHARE, bool KV8 = false, bool FINALN = false, bool ZZ = false, bool BIG = false>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams pk) {
   static_assert(!(FINALN && SHARE), "the merging epilogue goes with 128-row workgroups");
   typedef typename std::conditional<KV8, unsigned char, T>::type KVT;  // element type of K / V in memory
@@ -297,8 +299,11 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const unsigned krow_b = (unsigned)(p.ks.s * (int64_t)sizeof(KVT));  // bytes per K row
   const unsigned vrow_b = (unsigned)(p.vs.s * (int64_t)sizeof(KVT));
   const int64_t rows_all = (int64_t)p.P * p.Sk;
-  const u32x4 krsrc = buffer_descriptor(kp, (unsigned)(((rows_all - 1) * p.ks.s + D) * (int64_t)sizeof(KVT)));
-  const u32x4 vrsrc = buffer_descriptor(vp, (unsigned)(((rows_all - 1) * p.vs.s + D) * (int64_t)sizeof(KVT)));
+  const unsigned long long kbytes = (unsigned long long)(((rows_all - 1) * p.ks.s + D) * (int64_t)sizeof(KVT));
+  const unsigned long long vbytes = (unsigned long long)(((rows_all - 1) * p.vs.s + D) * (int64_t)sizeof(KVT));
+  static_assert(!(BIG && KV8), "the re-based variants are built for 16-bit K / V");
+  const u32x4 krsrc = buffer_descriptor(kp, BIG ? 0u : (unsigned)kbytes);  // (BIG: an empty range, for loads that are not wanted)
+  const u32x4 vrsrc = buffer_descriptor(vp, BIG ? 0u : (unsigned)vbytes);
   // LDS byte addresses of this group's buffers and of this wave's 1 KB share of a round
   const unsigned lds_group = (unsigned)(uintptr_t)(lds_u8*)smem + (SHARE ? 0 : grp * C::GROUP);
   const unsigned lds_wave = lds_group + (SHARE ? wave : w) * 1024;
@@ -314,6 +319,14 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   u32x2 stage[KV8 ? NLOADS : 1];
   auto load_one = [&](int q, bool kon, int k_row, unsigned kb, bool von, int v_row, unsigned vb) {
     if (q < C::NDMA) {
+      if constexpr (BIG) {
+        // the sub-tile's first row as a 64-bit byte offset -> window descriptor + offset inside it
+        unsigned rel = OFF_NONE;
+        u32x4 rs = krsrc;
+        if (kon) rs = buffer_window(kp, kbytes, (unsigned long long)(unsigned)k_row * krow_b, rel);
+        load_to_lds_b128(rs, kdoff + rel + (unsigned)(q * C::RPD) * krow_b, lds_wave + kb + q * (C::DTHREADS * 16));
+        return;
+      }
       const unsigned u = kon ? (unsigned)(k_row + q * C::RPD) * krow_b : OFF_NONE;
       if constexpr (KV8)
         stage[q] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(krs, kdoff + u, 0, 0));
@@ -321,6 +334,13 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         load_to_lds_b128(krsrc, kdoff + u, lds_wave + kb + q * (C::DTHREADS * 16));
     } else {
       const int r = q - C::NDMA;
+      if constexpr (BIG) {
+        unsigned rel = OFF_NONE;
+        u32x4 rs = vrsrc;
+        if (von) rs = buffer_window(vp, vbytes, (unsigned long long)(unsigned)v_row * vrow_b, rel);
+        load_to_lds_b128(rs, vdoff + rel + (unsigned)(r * C::RPD) * vrow_b, lds_wave + vb + r * (C::DTHREADS * 16));
+        return;
+      }
       const unsigned u = von ? (unsigned)(v_row + r * C::RPD) * vrow_b : OFF_NONE;
       if constexpr (KV8)
         stage[q] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(vrs, vdoff + u, 0, 0));
@@ -1205,6 +1225,15 @@ hipError_t launch16_kv8(FwdParams p, hipStream_t stream) {
   return launch<flash_fwd16_kernel<T, D, 1, false, true, false, ZZ>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
 }
 
+// K / V spanning 2 GiB or more per (batch, head): the re-based variants, 128-row workgroups with two wave groups
+// (such a tensor has more than enough rows for them).
+template <typename T, int D>
+hipError_t launch16_big(const FwdParams& p, hipStream_t stream) {
+  if (p.epi == SPA_EPI_FINALN)
+    return launch<flash_fwd16_kernel<T, D, 2, false, false, true, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+  return launch<flash_fwd16_kernel<T, D, 2, false, false, false, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+}
+
 // (dtype, D) -> kernel family; the zigzag variants are instantiated beside the plain ones
 template <bool ZZ>
 hipError_t launch16_any(const FwdParams& p, int D, int dtype, hipStream_t stream) {
@@ -1233,14 +1262,30 @@ hipError_t launch16_any(const FwdParams& p, int D, int dtype, hipStream_t stream
 
 }  // namespace
 
-// This file makes two objects: compiled with SPA_FWD_ZIGZAG_UNIT it holds the zigzag variants of the 16-bit
-// kernel and nothing else, without it everything else (so that the two halves compile side by side).
-#ifdef SPA_FWD_ZIGZAG_UNIT
+// This file makes three objects: compiled with SPA_FWD_ZIGZAG_UNIT it holds the zigzag variants of the 16-bit
+// kernel and nothing else, with SPA_FWD_BIG_UNIT the re-based variants, without either everything else (so that
+// the parts compile side by side).
+#if defined(SPA_FWD_ZIGZAG_UNIT)
 hipError_t spa_launch_fwd16_zigzag(const FwdParams& p, int D, int dtype, hipStream_t stream) {
   return launch16_any<true>(p, D, dtype, stream);
 }
+#elif defined(SPA_FWD_BIG_UNIT)
+hipError_t spa_launch_fwd16_big(const FwdParams& p, int D, int dtype, hipStream_t stream) {
+  if (p.k_scale || p.zigzag) return hipErrorInvalidValue;  // no re-based e4m3 or zigzag variants
+  if (dtype == 1) {
+    if (D == 128) return launch16_big<__bf16, 128>(p, stream);
+    if (D == 64) return launch16_big<__bf16, 64>(p, stream);
+    if (D == 32) return launch16_big<__bf16, 32>(p, stream);
+  } else if (dtype == 2) {
+    if (D == 128) return launch16_big<_Float16, 128>(p, stream);
+    if (D == 64) return launch16_big<_Float16, 64>(p, stream);
+    if (D == 32) return launch16_big<_Float16, 32>(p, stream);
+  }
+  return hipErrorInvalidValue;
+}
 #else
 hipError_t spa_launch_fwd16_zigzag(const FwdParams& p, int D, int dtype, hipStream_t stream);
+hipError_t spa_launch_fwd16_big(const FwdParams& p, int D, int dtype, hipStream_t stream);
 
 // Returns hipSuccess, or hipErrorInvalidValue for an unsupported (dtype, D).
 hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream) {
@@ -1258,7 +1303,9 @@ hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t strea
     p.out = (char*)slots.out<char>(p.part, p.part_slot) - row0 * p.os.s * 2;
     p.lse = slots.lse(p.part, p.P, p.part_slot) - row0;
   }
-  if (dtype == 1 || dtype == 2) return p.zigzag ? spa_launch_fwd16_zigzag(p, D, dtype, stream) : launch16_any<false>(p, D, dtype, stream);
+  if (dtype == 1 || dtype == 2)
+    return p.big ? spa_launch_fwd16_big(p, D, dtype, stream)
+                 : p.zigzag ? spa_launch_fwd16_zigzag(p, D, dtype, stream) : launch16_any<false>(p, D, dtype, stream);
   if (dtype == 0) {
     if (p.epi != SPA_EPI_PLAIN) return hipErrorInvalidValue;  // fp32 ring steps merge with the separate kernel
     if (D == 128) return launch<flash_fwd32_kernel<128>>(FWD_THREADS, Fwd32Cfg<128>::SMEM, p, stream);
@@ -1267,4 +1314,4 @@ hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t strea
   }
   return hipErrorInvalidValue;
 }
-#endif  // SPA_FWD_ZIGZAG_UNIT
+#endif  // SPA_FWD_ZIGZAG_UNIT / SPA_FWD_BIG_UNIT

@@ -63,9 +63,19 @@ bool dims_ok(int B, int H, int S, int D) { return B > 0 && H > 0 && S > 0 && D >
 
 bool pow2_8_512(int D) { return D >= 8 && D <= 512 && (D & (D - 1)) == 0; }
 
-// The 16-bit forward kernel addresses K and V of one (batch, head) through 32-bit buffer offsets.
+// The 16-bit kernels address the streamed tensors of one (batch, head) through buffer descriptors with 32-bit
+// per-lane offsets: below 2 GiB one descriptor covers the tensor (span_ok); beyond, the variants that re-base
+// the descriptor per tile take over, which need a tile of 128 rows to stay below 1 GiB (span_rebasable).
 bool span_ok(int64_t rows, int64_t row_stride, int D, int esz) {
   return ((rows - 1) * row_stride + D) * esz < 0x7fffffffLL;
+}
+bool span_rebasable(int64_t row_stride, int esz) { return row_stride * esz * 128 < 0x40000000LL; }
+// Can K / V that span 2 GiB or more be run?  fp32: yes (those kernels address with 64-bit pointers); e4m3: no
+// (no re-based variants); 16-bit: when both row strides allow re-basing.  Returns null or what is in the way.
+const char* big_kv_obstacle(bool kv8, int dtype, int64_t k_row_stride, int64_t v_row_stride, int esz) {
+  if (kv8) return "not supported for e4m3 K/V";
+  if (dtype == SPA_F32) return nullptr;
+  return span_rebasable(k_row_stride, esz) && span_rebasable(v_row_stride, esz) ? nullptr : "and 128 rows of them 1 GiB or more";
 }
 
 // Any finite softmax scale, as in the reference.  Zero is carried as 1e-30: every finite score then
@@ -135,9 +145,12 @@ int flash_fwd(const char* what, const void* q, const void* k, const void* v, con
   if (!aligned16(q, q_strides, esz) || !kv_aligned || !aligned16(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0)
     return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned (8-byte for e4m3 K/V)", what);
   if ((int64_t)B * H > 0x7fffffffLL || (Sq + 127) / 128 > 65535) return fail(SPA_EINVAL, "%s: grid too large", what);
-  if (!span_ok(Sk, k_strides[2], D, kesz) || !span_ok(Sk, v_strides[2], D, kesz))
-    return fail(SPA_EUNSUPPORTED, "%s: K/V of one (batch, head) span more than 2 GiB", what);
+  const bool big = !span_ok(Sk, k_strides[2], D, kesz) || !span_ok(Sk, v_strides[2], D, kesz);
+  if (big && big_kv_obstacle(kv8, dtype, k_strides[2], v_strides[2], esz))
+    return fail(SPA_EUNSUPPORTED, "%s: K/V of one (batch, head) span 2 GiB or more (%s)", what,
+                big_kv_obstacle(kv8, dtype, k_strides[2], v_strides[2], esz));
   FwdParams p;
+  p.big = big && dtype != SPA_F32;
   p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
   p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
   p.qs = S3(q_strides); p.ks = S3(k_strides); p.vs = S3(v_strides); p.os = S3(o_strides);
@@ -252,13 +265,17 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   if (!aligned16(q, q_strides, esz) || !kv_aligned ||
       !aligned16(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0 || ((uintptr_t)workspace & 15) != 0)
     return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned (8-byte for e4m3 K/V)", what);
-  if (!span_ok(S, k_strides[2], D, kesz) || !span_ok(S, v_strides[2], D, kesz))
-    return fail(SPA_EUNSUPPORTED, "%s: K/V of one (batch, head) span more than 2 GiB", what);
+  const bool big = !span_ok(S, k_strides[2], D, kesz) || !span_ok(S, v_strides[2], D, kesz);
+  if (big && big_kv_obstacle(kv8, dtype, k_strides[2], v_strides[2], esz))
+    return fail(SPA_EUNSUPPORTED, "%s: K/V of one (batch, head) span 2 GiB or more (%s)", what,
+                big_kv_obstacle(kv8, dtype, k_strides[2], v_strides[2], esz));
   const bool causal = mask_mode == SPA_MASK_CAUSAL;
   const int s = S / P;
   if (dtype == SPA_F32) fuse = SPA_RING_PER_STEP;  // the fp32 kernel handles one block pair per launch
   // zigzag shards only change a causal ring (without a mask the order of the rows does not matter)
   const bool zig = zig_req && causal && P > 1;
+  if (zig && big && dtype != SPA_F32)
+    return fail(SPA_EUNSUPPORTED, "%s: zigzag shards are not built for K/V of 2 GiB or more per (batch, head)", what);
   const bool multi = P > 1 && (!causal || rank != 0 || zig);  // does some rank visit more than one block?
   if (fuse == SPA_RING_PER_STEP && multi && !workspace)
     return fail(SPA_EINVAL, "%s: workspace required when steps are separate launches", what);
@@ -295,6 +312,7 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   p.k_scale = k_scale; p.v_scale = v_scale;
   p.zigzag = zig && dtype != SPA_F32;
   p.zz_half = 0;
+  p.big = big && dtype != SPA_F32;
 
   if (fuse == SPA_RING_ALL_RANKS) {  // one launch: every requested rank, every step
     p.rank0 = r_lo; p.nranks = r_hi - r_lo; p.t_begin = 0; p.t_count = -1;
@@ -498,15 +516,18 @@ int flash_bwd(const char* what, const void* q, const void* k, const void* v, con
       !aligned16(dout, do_strides, esz) || !aligned16(dq, dq_strides, gsz) || !aligned16(dk, dk_strides, gsz) ||
       !aligned16(dv, dv_strides, gsz))
     return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned", what);
-  if (!span_ok(Sq, q_strides[2], D, esz) || !span_ok(Sk, k_strides[2], D, esz) || !span_ok(Sk, v_strides[2], D, esz) ||
-      !span_ok(Sq, do_strides[2], D, esz))
-    return fail(SPA_EUNSUPPORTED, "%s: a tensor of one (batch, head) spans more than 2 GiB", what);
+  const bool big = !span_ok(Sq, q_strides[2], D, esz) || !span_ok(Sk, k_strides[2], D, esz) || !span_ok(Sk, v_strides[2], D, esz) ||
+                   !span_ok(Sq, do_strides[2], D, esz);
+  if (big && dtype != SPA_F32 && !(span_rebasable(q_strides[2], esz) && span_rebasable(k_strides[2], esz) &&
+                                   span_rebasable(v_strides[2], esz) && span_rebasable(do_strides[2], esz)))
+    return fail(SPA_EUNSUPPORTED, "%s: a tensor of one (batch, head) spans 2 GiB or more and 128 rows of it 1 GiB or more", what);
   if ((int64_t)B * H * ((Sq + 127) / 128) > 0x7fffffffLL || (int64_t)B * H * ((Sk + 127) / 128) > 0x7fffffffLL)
     return fail(SPA_EINVAL, "%s: grid too large", what);
   BwdParams p;
   p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta;
   p.dq = (float*)dq; p.dk = (float*)dk; p.dv = (float*)dv;
   p.grads_in_t = grads_in_t;
+  p.big = big && dtype != SPA_F32;
   p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
   p.qs = S3(q_strides); p.ks = S3(k_strides); p.vs = S3(v_strides); p.dos = S3(do_strides);
   p.dqs = S3(dq_strides); p.dks = S3(dk_strides); p.dvs = S3(dv_strides);
@@ -589,9 +610,12 @@ int flash_fwd_varlen(const char* what, const void* q, const void* k, const void*
                               : aligned16v(k, k_strides, esz) && aligned16v(v, v_strides, esz);
   if (!aligned16v(q, q_strides, esz) || !kv_aligned || !aligned16v(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0)
     return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned (8-byte for e4m3 K/V)", what);
-  if (!span_ok(max_sk, k_strides[1], D, kesz) || !span_ok(max_sk, v_strides[1], D, kesz))
-    return fail(SPA_EUNSUPPORTED, "%s: K/V of one (sequence, head) span more than 2 GiB", what);
+  const bool big = !span_ok(max_sk, k_strides[1], D, kesz) || !span_ok(max_sk, v_strides[1], D, kesz);
+  if (big && big_kv_obstacle(kv8, dtype, k_strides[1], v_strides[1], esz))
+    return fail(SPA_EUNSUPPORTED, "%s: K/V of one (sequence, head) span 2 GiB or more (%s)", what,
+                big_kv_obstacle(kv8, dtype, k_strides[1], v_strides[1], esz));
   FwdParams p;
+  p.big = big && dtype != SPA_F32;
   p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
   p.B = nseq; p.H = H; p.Sq = max_sq; p.Sk = max_sk;
   p.qs = S2(q_strides); p.ks = S2(k_strides); p.vs = S2(v_strides); p.os = S2(o_strides);
@@ -627,10 +651,13 @@ int flash_bwd_varlen(const char* what, const void* q, const void* k, const void*
       !aligned16v(dout, do_strides, esz) || !aligned16v(dq, dq_strides, gsz) || !aligned16v(dk, dk_strides, gsz) ||
       !aligned16v(dv, dv_strides, gsz) || (((uintptr_t)lse | (uintptr_t)delta) & 3) != 0)
     return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned", what);
-  if (!span_ok(max_sq, q_strides[1], D, esz) || !span_ok(max_sk, k_strides[1], D, esz) ||
-      !span_ok(max_sk, v_strides[1], D, esz) || !span_ok(max_sq, do_strides[1], D, esz))
-    return fail(SPA_EUNSUPPORTED, "%s: a tensor of one (sequence, head) spans more than 2 GiB", what);
+  const bool big = !span_ok(max_sq, q_strides[1], D, esz) || !span_ok(max_sk, k_strides[1], D, esz) ||
+                   !span_ok(max_sk, v_strides[1], D, esz) || !span_ok(max_sq, do_strides[1], D, esz);
+  if (big && dtype != SPA_F32 && !(span_rebasable(q_strides[1], esz) && span_rebasable(k_strides[1], esz) &&
+                                   span_rebasable(v_strides[1], esz) && span_rebasable(do_strides[1], esz)))
+    return fail(SPA_EUNSUPPORTED, "%s: a tensor of one (sequence, head) spans 2 GiB or more and 128 rows of it 1 GiB or more", what);
   BwdParams p;
+  p.big = big && dtype != SPA_F32;
   p.q = q; p.k = k; p.v = v; p.dout = dout; p.lse = lse; p.delta = delta;
   p.dq = (float*)dq; p.dk = (float*)dk; p.dv = (float*)dv;
   p.grads_in_t = grads_in_t;

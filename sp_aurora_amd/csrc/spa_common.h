@@ -58,6 +58,9 @@ struct FwdParams {
   // the second half only (a step with c > r that is not the rank's last).
   int zigzag = 0;
   int zz_half = 0;
+  // K / V rows of one (batch, head) span 2 GiB or more: the launcher takes the kernel variants that re-base their
+  // buffer descriptors per tile (16-bit kernels; the fp32 kernels address with 64-bit pointers anyway)
+  int big = 0;
 };
 
 // Layout of the ring-step slots of one rank in the caller's workspace (16-bit inputs, ring of P):
@@ -105,6 +108,8 @@ struct BwdParams {
   // 0: dq/dk/dv are fp32 accumulators, added to; 1: they are tensors of q's element type (strides in
   // those elements) and are WRITTEN: the whole gradient comes from this one launch
   int grads_in_t;
+  // some tensor's rows of one (batch, head) span 2 GiB or more (see FwdParams::big)
+  int big = 0;
 };
 
 // 16-bit element traits: MFMA 32x32x16 with 8 elements per lane per operand.
@@ -221,6 +226,19 @@ static __device__ __forceinline__ u32x4 buffer_descriptor(const void* base, unsi
   r[3] = 0x00020000u;
   return r;
 }
+// For tensors whose rows of one (batch, head) span 2 GiB or more, beyond what a 32-bit per-lane offset with its
+// sign bit spare can address: a descriptor over the part of the tensor that starts at the 1 GiB boundary below
+// byte offset `off` (wave-uniform) and `rel`, the offset inside that window (< 1 GiB; the lanes add less than
+// 1 GiB to it).  The hardware range check still ends at the tensor's last byte when that lies within 4 GiB of the
+// window's start, and beyond that every offset a lane can form is inside the tensor.
+static __device__ __forceinline__ u32x4 buffer_window(const void* base, unsigned long long total, unsigned long long off,
+                                                      unsigned& rel) {
+  const unsigned long long w = off & ~0x3fffffffULL;
+  rel = __builtin_amdgcn_readfirstlane((unsigned)(off - w));
+  const unsigned long long left = total > w ? total - w : 0ULL;
+  return buffer_descriptor((const char*)base + w, left > 0xffffffffULL ? 0xffffffffu : (unsigned)left);
+}
+
 // Transposing LDS read: in a block of 16 lanes, lane 4 e + c supplies the address of 8 bytes
 // (4 elements) of row e, and lane x receives element x (of the 16 the row's four pieces hold)
 // of rows 0..3.

@@ -279,3 +279,27 @@ def test_recording_belongs_to_the_recording_thread():
         assert rec.calls == []
     assert seen == {"is_recorder": False, "version": 1}
     assert not isinstance(_lib.load(), _lib._Recorder)
+
+
+@pytest.mark.skipif(__import__("torch").cuda.is_available(), reason="passes pointers that must never reach a device")
+def test_tensors_of_2_gib_and_more_per_head_pass_the_argument_checks():
+    """K / V (and in the backward q / dout) of one (batch, head) may span 2 GiB and more: H = 64, D = 128, S = 262144
+    in the public [B,S,H,D] layout is 4 GiB per head.  Without a device every check passes and the launch itself
+    reports the missing device (-4); what stays refused says why (-2)."""
+    lib = _lib.load()
+    p = ctypes.c_void_p(4096)
+    H, D, S = 64, 128, 262144
+    st = _s3(S * H * D, D, H * D)
+    assert lib.spa_flash_fwd(p, p, p, p, p, 1, H, S, S, D, st, st, st, st, 1.0, 1, 1, None) == -4
+    assert b"device" in lib.spa_last_error()
+    assert lib.spa_ring_fwd(p, p, p, p, p, p, 1, H, S, D, 16, -1, st, st, st, st, 1.0, 1, 1, 1, None) == -4
+    assert lib.spa_flash_bwd_out(*([p] * 9 + [1, H, S, S, D] + [st] * 7), 1.0, 1, 1, None) == -4
+    # e4m3 K/V (1 byte per element: 8 heads more), zigzag shards, and rows so far apart that 128 of them exceed 1 GiB
+    st8 = _s3(2 * S * H * D, D, 2 * H * D)
+    assert lib.spa_flash_fwd_fp8kv(p, p, p, p, p, p, p, 1, 2 * H, S, S, D, st, st8, st8, st, 1.0, 1, 1, None) == -2
+    assert b"e4m3" in lib.spa_last_error()
+    assert lib.spa_ring_fwd(p, p, p, p, p, p, 1, H, S, D, 16, -1, st, st, st, st, 1.0, 1, 1, 1 | 16, None) == -2
+    assert b"zigzag" in lib.spa_last_error()
+    far = _s3(0, D, 8 << 20)
+    assert lib.spa_flash_fwd(p, p, p, p, p, 1, 1, 1024, 1024, D, st, far, far, st, 1.0, 0, 1, None) == -2
+    assert b"1 GiB" in lib.spa_last_error()

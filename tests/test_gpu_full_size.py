@@ -284,3 +284,36 @@ def test_long_sequence_131072_forward_backward_spot_checks():
         for name, got, want in (("dv", dv, want_dv), ("dk", dk, want_dk)):
             err = (got[0, j, h].cpu().double() - want).abs().max().item()
             assert err <= 3e-2 * max(want.abs().max().item(), 1e-2), f"{name} row {j}: err {err:.3e} scale {want.abs().max().item():.3e}"
+
+
+# ------------------------------------------------------------------ beyond 2 GiB per (batch, head)
+def test_rows_of_one_head_spanning_more_than_2_gib():
+    """bf16 [B=1, S=8448, H=1024, D=128] viewed as H=4 heads of a tensor whose rows are 256 KiB apart: the rows of one
+    head span 2.06 GiB, past what one buffer descriptor with 32-bit offsets covers, so the variants that re-base their
+    descriptors per tile run (forward, ring forward in its three schedules, backward).  The same four heads packed
+    into compact tensors go through the ordinary variants: same mathematics, results within the bf16 tolerances,
+    and float64 rows of one head pin both."""
+    S, Hs, H, D, P = 8448, 1024, 4, 128, 4
+    scale = D ** -0.5
+    gen = torch.Generator(device=DEV).manual_seed(60)  # 1.1 G elements per tensor: drawn on the device
+    big = [torch.randn((1, S, Hs, D), generator=gen, device=DEV, dtype=torch.bfloat16) for _ in range(4)]
+    wide = [t[:, :, ::341] for t in big]  # heads 0, 341, 682, 1023 as strided views (head stride 341 D), no copy
+    assert all(w.shape == (1, S, H, D) and w.stride(1) * 2 * (S - 1) > 2 ** 31 for w in wide)
+    q, k, v, dout = wide
+    qc, kc, vc, dc = (w.contiguous() for w in wide)
+    o_ref, l_ref = ops.flash_fwd(qc, kc, vc, scale, True)
+    o, l = ops.flash_fwd(q, k, v, scale, True)
+    assert_out(o, o_ref, "block forward, rows 256 KiB apart")
+    assert_lse(l, l_ref, "block forward, rows 256 KiB apart")
+    spot_check_rows(o[0, :, 3], l[0, 3], qc[0, :, 3], kc[0, :, 3], vc[0, :, 3], scale, True, "2 GiB span fp64", n_rows=10)
+    for fuse in ("step", "rank", "all"):
+        o2, l2 = ops.ring_fwd(q, k, v, P, scale, True, fuse=fuse)
+        assert_out(o2, o_ref, f"ring {fuse}, rows 256 KiB apart")
+        assert_lse(l2, l_ref, f"ring {fuse}, rows 256 KiB apart")
+    delta = ops.bwd_delta(o_ref, dc)
+    g_ref = ops.flash_bwd_out(qc, kc, vc, dc, l_ref, delta, scale, True)
+    g = ops.flash_bwd_out(q, k, v, dout, l_ref, delta, scale, True)
+    for name, got, ref in zip(("dq", "dk", "dv"), g, g_ref):
+        ref = ref.float()
+        bad = (got.float() - ref).abs() > 3e-2 * ref.abs().max() + 3e-2 * ref.abs()
+        assert torch.isfinite(got).all() and not bad.any(), f"{name}: {int(bad.sum())} out of tolerance"
