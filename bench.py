@@ -63,6 +63,7 @@ sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 MFMA_F32_PEAK_TFLOPS = 157.3
+MFMA_FP8_BF16_MIX_PEAK_TFLOPS = 3333.3  # half the FLOPs at the fp8 rate (5000), half at the bf16 rate (2500)
 HBM_PEAK_GBPS = 8000.0
 
 B, S, H, D, P = 1, 8192, 32, 128, 8
@@ -323,8 +324,10 @@ ROW_NOTES = {
     "config4_relayout_h2s": "the inverse of config4_relayout_s2h",
     "config4_ulysses_forward": "config 4: 3 re-layouts in, full causal attention per head group [8,1,16384,4,128], 1 re-layout out, output "
                                "allocation included; views_tflops = the same result with head groups read and written in place (B = 1)",
-    "block_forward_fp8_kv": "causal block forward over the config-3 sequence, bf16 q [1,8192,32,128], K / V e4m3 + fp32 scale per (batch, "
-                            "head), one call; bf16_kv_tflops = the same call with bf16 K / V",
+    "block_forward_fp8": "causal block forward over the config-3 sequence [1,8192,32,128] as one call, q, K, V all e4m3 + fp32 scale per "
+                         "(batch, head), out bf16: scores on the 8-bit matrix instruction (spa_flash_fwd_fp8qkv), P V on the 16-bit one; "
+                         "peak = the mix of the two rates for equal FLOPs, 2 / (1/5000 + 1/2500); kv_only_tflops = bf16 q with e4m3 K / V "
+                         "(spa_flash_fwd_fp8kv, both contractions 16-bit), bf16_tflops = the same call with bf16 q, K, V",
     "merge_update_out_and_lse": "update_out_and_lse: merge of a bf16 block into the fp32 running (out, lse) of one config-3 rank "
                                 "[1,1024,32,128], 8 operand sets in turn, recorded calls replayed; host cost of the call included",
     "config5_ring_forward": "config 5 forward: bf16 qkv [1,32768,3,16,128] (strided views) causal, ring of 16 chunks of 2048, 16 diagonal + "
@@ -346,8 +349,8 @@ ROW_SPECS = {
     "config4_relayout_h2s": ("config 4 re-layout h2s, 268 MB per launch", "GB/s", "hbm", "relayout<16,h2s>", HBM_PEAK_GBPS, ()),
     "config4_ulysses_forward": ("config 4: 3 re-layouts, attention, 1 re-layout", "TFLOP/s", "mfma", "relayout x4 + flash_fwd16<bf16,128>",
                                 MFMA_BF16_PEAK_TFLOPS, ("views_tflops",)),
-    "block_forward_fp8_kv": ("causal block forward [1,8192,32,128], e4m3 K/V", "TFLOP/s", "mfma", "flash_fwd16<bf16,128,e4m3 K/V>",
-                             MFMA_BF16_PEAK_TFLOPS, ("bf16_kv_tflops",)),
+    "block_forward_fp8": ("causal block forward [1,8192,32,128], e4m3 q/K/V, 8-bit scores", "TFLOP/s", "mfma", "flash_fwd16<bf16,128,e4m3 q/K/V>",
+                          MFMA_FP8_BF16_MIX_PEAK_TFLOPS, ("kv_only_tflops", "bf16_tflops")),
     "merge_update_out_and_lse": ("merge of a bf16 block [1,1024,32,128] into fp32 (out, lse), 42.3 MB", "GB/s", "hbm", "merge<bf16>",
                                  HBM_PEAK_GBPS, ()),
     "config5_ring_forward": ("config 5 forward, P=16, 1 launch", "TFLOP/s", "mfma", "flash_fwd16<bf16,128>", MFMA_BF16_PEAK_TFLOPS,
@@ -464,18 +467,21 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
         # the same call with bf16 K / V (same kernel family, direct-to-LDS tiles)
         Bn, Sn, Hn, Dn = 1, 8192, 32, 128
         q, k, v = rand_tensors(torch, (Bn, Sn, Hn, Dn), SEED, 3, INPUT_SCALE, torch.bfloat16, dev)
+        q8, qsc = ops.quantize_fp8_per_head(q)
         k8, ksc = ops.quantize_fp8_per_head(k)
         v8, vsc = ops.quantize_fp8_per_head(v)
         out = torch.empty_like(q)
         lse = torch.empty((Bn, Hn, Sn), dtype=torch.float32, device=dev)
         flops = 4.0 * Bn * Hn * Sn * Sn * Dn / 2
-        f8 = lambda: ops.flash_fwd(q, k8, v8, None, True, out=out, lse=lse, k_scale=ksc, v_scale=vsc)
+        f8 = lambda: ops.flash_fwd(q8, k8, v8, None, True, out=out, lse=lse, q_scale=qsc, k_scale=ksc, v_scale=vsc)
+        f8kv = lambda: ops.flash_fwd(q, k8, v8, None, True, out=out, lse=lse, k_scale=ksc, v_scale=vsc)
         f16 = lambda: ops.flash_fwd(q, k, v, None, True, out=out, lse=lse)
         m16 = measure(torch, f16, 20, 5, **light)
+        mkv = measure(torch, f8kv, 20, 5, **light)
         m = measure(torch, f8, 20, 5, **light)
         tf = tfl(flops, m)
-        finish("block_forward_fp8_kv", m, tf, bf16_kv_tflops=tfl(flops, m16))
-        del q, k, v, k8, v8
+        finish("block_forward_fp8", m, tf, kv_only_tflops=tfl(flops, mkv), bf16_tflops=tfl(flops, m16))
+        del q, k, v, q8, k8, v8
     if "merge" in which:
         Bn, sn, Hn, Dn = 1, 1024, 32, 128
         g = torch.Generator().manual_seed(3)
@@ -545,9 +551,9 @@ def attach_cpu(rows, cpu):
         rows["config4_relayout_h2s"]["cpu_baseline"] = b
         # attention of one head group [1,4,16384,128] as 2048-row blocks (x 8 groups: same ratio); re-layouts not included
         rows["config4_ulysses_forward"]["cpu_baseline"] = cpu.ring_forward(1, 4, 2048, 128, 8, 28, 3)
-    if "block_forward_fp8_kv" in rows:
-        # the same attention with dequantised K / V as 1024-row blocks (the reference has no 8-bit path)
-        rows["block_forward_fp8_kv"]["cpu_baseline"] = cpu.ring_forward(1, 32, 1024, 128, 8, 28, SEED)
+    if "block_forward_fp8" in rows:
+        # the same attention with dequantised q / K / V as 1024-row blocks (the reference has no 8-bit path)
+        rows["block_forward_fp8"]["cpu_baseline"] = cpu.ring_forward(1, 32, 1024, 128, 8, 28, SEED)
     if "merge_update_out_and_lse" in rows:
         rows["merge_update_out_and_lse"]["cpu_baseline"] = cpu.merge()
     if "config5_ring_forward" in rows:

@@ -102,6 +102,23 @@ int spa_flash_fwd_fp8kv(const void* q, const void* k8, const void* v8,
                         float scale, int mask_mode, int dtype, void* stream);
 
 /*
+ * spa_flash_fwd_fp8kv with q held as e4m3 as well: Q = q8 * q_scale[b*H + h] (fp32 contiguous [B,H], positive),
+ * q8 [B,H,Sq,D] by strides in bytes, rows of q8 and k8 16-byte aligned, rows of v8 8-byte aligned; out (and the
+ * softmax) in `dtype` (SPA_BF16 or SPA_F16); D = 128.  The scores q8 . k8 are formed on the 8-bit matrix
+ * instruction (twice the rate of the 16-bit one; a product of two e4m3 values is exact in fp32, and the
+ * accumulation is fp32), q_scale * k_scale is folded into the softmax scale; V is widened to `dtype` and P V is the
+ * same 16-bit contraction as in spa_flash_fwd_fp8kv.  The result is that of spa_flash_fwd on the dequantised
+ * tensors up to fp32 rounding.  Same call sites as spa_flash_fwd_fp8kv; the reference has no 8-bit path.
+ */
+int spa_flash_fwd_fp8qkv(const void* q8, const void* k8, const void* v8,
+                         const float* q_scale, const float* k_scale, const float* v_scale,
+                         void* out, float* lse,
+                         int B, int H, int Sq, int Sk, int D,
+                         const int64_t q_strides[3], const int64_t k_strides[3],
+                         const int64_t v_strides[3], const int64_t o_strides[3],
+                         float scale, int mask_mode, int dtype, void* stream);
+
+/*
  * Merge of one block result into the running (out_acc, lse_acc):
  *   lse' = logaddexp(lse, lse_b);  out' = out - sigmoid(lse_b - lse) * (out - out_b)
  * Replaces update_out_and_lse / _update_out_and_lse (sp_aurora/utils.py:47-147).

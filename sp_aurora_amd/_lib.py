@@ -28,6 +28,7 @@ SIGNATURES = {
     "spa_device_info": (_i, [ctypes.c_char_p, _i]),
     "spa_flash_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _vp]),
     "spa_flash_fwd_fp8kv": (_i, [_vp] * 7 + [_i] * 5 + [_s3] * 4 + [_f, _i, _i, _vp]),
+    "spa_flash_fwd_fp8qkv": (_i, [_vp] * 8 + [_i] * 5 + [_s3] * 4 + [_f, _i, _i, _vp]),
     "spa_flash_fwd_varlen_fp8kv": (_i, [_vp] * 9 + [_i] * 7 + [_s3] * 4 + [_f, _i, _i, _vp]),
     "spa_ring_fwd_fp8kv": (_i, [_vp] * 8 + [_i] * 6 + [_s3] * 4 + [_f, _i, _i, _i, _vp]),
     "spa_ring_fwd_workspace_bytes": (ctypes.c_int64, [_i, _i, _i, _i, _i, _i]),

@@ -94,10 +94,18 @@ __device__ __forceinline__ int v_swizzle(int row) {
 // ZZ: the variant for zigzag shards (FwdParams::zigzag); the others carry none of its bookkeeping.
 // BIG: the variant for K / V whose rows of one (batch, head) span 2 GiB or more: the buffer descriptors are
 // re-based per sub-tile (a few scalar instructions per tile that the others do without).
-template <typename T, int D, int NG, bool SHARE, bool KV8 = false, bool FINALN = false, bool ZZ = false, bool BIG = false>
+// QK8 (with KV8, D = 128): q is e4m3 as well (Q = q8 * q_scale[b,h]) and S^T = K Q^T runs on the 8-bit matrix
+// instruction (v_mfma_f32_32x32x64_f8f6f4, twice the rate of the 16-bit one; products of two e4m3 values are exact
+// in fp32): K tiles stay bytes in LDS (direct loads again, half the size), Q fragments are 32 bytes per lane and
+// 64-deep step; V is widened to T as with KV8 and P V stays a 16-bit contraction.
+template <typename T, int D, int NG, bool SHARE, bool KV8 = false, bool FINALN = false, bool ZZ = false, bool BIG = false,
+          bool QK8 = false>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams pk) {
   static_assert(!(FINALN && SHARE), "the merging epilogue goes with 128-row workgroups");
+  static_assert(!QK8 || (KV8 && D == 128 && !FINALN && !ZZ && !BIG), "8-bit scores: e4m3 q, k, v, head dim 128, plain block calls");
   typedef typename std::conditional<KV8, unsigned char, T>::type KVT;  // element type of K / V in memory
+  typedef typename std::conditional<QK8, unsigned char, T>::type QT;   // element type of q in memory
+  constexpr bool KSTAGE = KV8 && !QK8;  // K tiles go through registers (widened on the way); V tiles do whenever KV8
   typedef Fwd16Cfg<D, NG, SHARE> C;
   FwdParams p = pk;  // a variable-length batch rewrites the sizes and bases for its sequence below
   typedef Mma16<T> M;
@@ -122,7 +130,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const int h = bh % p.H;
   int b = bh / p.H;
   // dequantisation scales of this (batch or sequence, head): K = k8 * ksc, V = v8 * vsc
-  const float ksc = KV8 ? p.k_scale[bh] : 1.f;
+  const float ksc = KV8 ? p.k_scale[bh] * (QK8 ? p.q_scale[bh] : 1.f) : 1.f;  // (with e4m3 q its scale rides along)
   const float vsc = KV8 ? p.v_scale[bh] : 1.f;
   const int qt = p.nqt - 1 - (int)blockIdx.y;
   // Zigzag shards: the tiles of the two halves of the chunk are laid out one half after the other (a tile
@@ -139,7 +147,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     const int q_lo = p.cu_q[b], k_lo = p.cu_k[b];
     p.Sq = p.cu_q[b + 1] - q_lo;
     p.Sk = p.cu_k[b + 1] - k_lo;
-    p.q = (const T*)p.q + (int64_t)q_lo * p.qs.s;
+    p.q = (const QT*)p.q + (int64_t)q_lo * p.qs.s;
     p.k = (const KVT*)p.k + (int64_t)k_lo * p.ks.s;
     p.v = (const KVT*)p.v + (int64_t)k_lo * p.vs.s;
     p.out = (T*)p.out + (int64_t)q_lo * p.os.s;
@@ -162,20 +170,34 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const int qw0 = q0 + (SHARE ? grp * FWD_BM : 0) + w * 32;
   const int64_t qoff = (int64_t)rank * p.Sq;  // first row of this rank's query chunk
 
-  const T* qp = (const T*)p.q + b * p.qs.b + h * p.qs.h + qoff * p.qs.s;
+  const QT* qp = (const QT*)p.q + b * p.qs.b + h * p.qs.h + qoff * p.qs.s;
   const KVT* kp = (const KVT*)p.k + b * p.ks.b + h * p.ks.h;
   const KVT* vp = (const KVT*)p.v + b * p.vs.b + h * p.vs.h;
 
   const int qrow = qw0 + ln;
   const int qrow_c = qrow < q_lim ? qrow : q_lim - 1;
 
-  frag qf[D / 16];
-  const unsigned qsign = p.negq ? 0x80008000u : 0u;  // negative softmax scale: -q with |scale|
+  frag qf[QK8 ? 1 : D / 16];
+  i32x8 qf8[QK8 ? D / 64 : 1];  // QK8: 32 bytes per lane and 64-deep contraction step (bytes 32 hh .. 32 hh + 31 of the step)
+  const unsigned qsign = p.negq ? (QK8 ? 0x80808080u : 0x80008000u) : 0u;  // negative softmax scale: -q with |scale|
+  if constexpr (QK8) {
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) {
-    u32x4 x = *(const u32x4*)(qp + (int64_t)qrow_c * p.qs.s + ks * 16 + hh * 8);
-    x[0] ^= qsign; x[1] ^= qsign; x[2] ^= qsign; x[3] ^= qsign;
-    qf[ks] = as_frag<frag>(x);
+    for (int kk = 0; kk < D / 64; ++kk) {
+      const u32x4 x0 = *(const u32x4*)(qp + (int64_t)qrow_c * p.qs.s + kk * 64 + hh * 32);
+      const u32x4 x1 = *(const u32x4*)(qp + (int64_t)qrow_c * p.qs.s + kk * 64 + hh * 32 + 16);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        qf8[kk][i] = (int)(x0[i] ^ qsign);
+        qf8[kk][4 + i] = (int)(x1[i] ^ qsign);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      u32x4 x = *(const u32x4*)(qp + (int64_t)qrow_c * p.qs.s + ks * 16 + hh * 8);
+      x[0] ^= qsign; x[1] ^= qsign; x[2] ^= qsign; x[3] ^= qsign;
+      qf[ks] = as_frag<frag>(x);
+    }
   }
 
   // ---- the schedule of this workgroup ----
@@ -294,7 +316,15 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // any tensor and stores zeros into a buffer nobody reads.
   constexpr unsigned OFF_NONE = 0x80000000u;
   const int drow = tg / C::CPR, dpos = tg % C::CPR;
-  const unsigned kdoff = (unsigned)((drow * p.ks.s + ((dpos ^ k_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(KVT));
+  // QK8: a K row is D bytes = D / 16 slots; rows 2 r, 2 r + 1 share a permutation (16 consecutive rows at one
+  // slot index then hit 16 different bank groups); NK direct loads per thread fill a sub-tile
+  constexpr int CPR8 = D / 16, ROWB8 = D;
+  constexpr int NK = QK8 ? (C::BN * ROWB8) / (C::DTHREADS * 16) : C::NDMA;
+  constexpr int RPD_K = QK8 ? C::DTHREADS / CPR8 : C::RPD;
+  static_assert(NK >= 1, "a K sub-tile must give every thread a load");
+  auto k8_swizzle = [](int row) { return (row >> 1) & (CPR8 - 1); };
+  const unsigned kdoff = QK8 ? (unsigned)((tg / CPR8) * p.ks.s + (((tg % CPR8) ^ k8_swizzle(tg / CPR8)) * 16))
+                             : (unsigned)((drow * p.ks.s + ((dpos ^ k_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(KVT));
   const unsigned vdoff = (unsigned)((drow * p.vs.s + ((dpos ^ v_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(KVT));
   const unsigned krow_b = (unsigned)(p.ks.s * (int64_t)sizeof(KVT));  // bytes per K row
   const unsigned vrow_b = (unsigned)(p.vs.s * (int64_t)sizeof(KVT));
@@ -310,7 +340,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   auto k_lds = [&](int i) { return (unsigned)((i & 1) * C::TILEB); };                  // relative to lds_group
   auto v_lds = [&](int i) { return (unsigned)(2 * C::TILEB + (i & 1) * C::TILEB); };
   // load number q of the pair (K sub-tile with first row k_row into buffer kb, V sub-tile v_row into vb)
-  constexpr int NLOADS = 2 * C::NDMA;
+  constexpr int NLOADS = NK + C::NDMA;
   // the same two descriptors as compiler-visible resources, for loads into registers
   const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, (int)krsrc[2], 0x00020000);
   const __amdgpu_buffer_rsrc_t vrs = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, (int)vrsrc[2], 0x00020000);
@@ -318,7 +348,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // the next VALU phase, which widens them and writes the 16-byte LDS slot (store_staged).
   u32x2 stage[KV8 ? NLOADS : 1];
   auto load_one = [&](int q, bool kon, int k_row, unsigned kb, bool von, int v_row, unsigned vb) {
-    if (q < C::NDMA) {
+    if (q < NK) {
       if constexpr (BIG) {
         // the sub-tile's first row as a 64-bit byte offset -> window descriptor + offset inside it
         unsigned rel = OFF_NONE;
@@ -327,13 +357,13 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         load_to_lds_b128(rs, kdoff + rel + (unsigned)(q * C::RPD) * krow_b, lds_wave + kb + q * (C::DTHREADS * 16));
         return;
       }
-      const unsigned u = kon ? (unsigned)(k_row + q * C::RPD) * krow_b : OFF_NONE;
-      if constexpr (KV8)
+      const unsigned u = kon ? (unsigned)(k_row + q * RPD_K) * krow_b : OFF_NONE;
+      if constexpr (KSTAGE)
         stage[q] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(krs, kdoff + u, 0, 0));
       else
         load_to_lds_b128(krsrc, kdoff + u, lds_wave + kb + q * (C::DTHREADS * 16));
     } else {
-      const int r = q - C::NDMA;
+      const int r = q - NK;
       if constexpr (BIG) {
         unsigned rel = OFF_NONE;
         u32x4 rs = vrsrc;
@@ -369,8 +399,8 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     if constexpr (KV8) {
       const unsigned slot = lds_group + (unsigned)tg * 16;
 #pragma unroll
-      for (int q = 0; q < NLOADS; ++q) {
-        const unsigned a = slot + (q < C::NDMA ? kb + q * (C::DTHREADS * 16) : vb + (q - C::NDMA) * (C::DTHREADS * 16));
+      for (int q = KSTAGE ? 0 : NK; q < NLOADS; ++q) {
+        const unsigned a = slot + (q < NK ? kb + q * (C::DTHREADS * 16) : vb + (q - NK) * (C::DTHREADS * 16));
         *(__attribute__((address_space(3))) u32x4*)(lds_u8*)(uintptr_t)a = widen(stage[q]);
       }
     }
@@ -382,9 +412,17 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // V (A operand of O^T += V^T P^T): the transposing read hands lane (dim, hh) four consecutive
   // keys of one head dim; in a block of 16 lanes, lane 4 e + c supplies the address of 8 bytes
   // (4 dims) of key e, and lane x receives dim x of keys 0..3.
-  unsigned kra[D / 16], vra[D / 32];
+  // (QK8: the operand of step kk is bytes 64 kk + 32 hh .. + 31 of the key's row: two 16-byte reads, kra[2 kk], kra[2 kk + 1])
+  constexpr int NKA = QK8 ? 2 * (D / 64) : D / 16;  // 16-byte K reads per lane and 32-key tile
+  unsigned kra[NKA], vra[D / 32];
+  if constexpr (QK8) {
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) kra[ks] = lds_group + ln * C::ROWB + (((2 * ks + hh) ^ k_swizzle<D>(ln)) * 16);
+    for (int u = 0; u < 2 * (D / 64); ++u)
+      kra[u] = lds_group + ln * ROWB8 + ((((u >> 1) * 4 + 2 * hh + (u & 1)) ^ k8_swizzle(ln)) * 16);
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) kra[ks] = lds_group + ln * C::ROWB + (((2 * ks + hh) ^ k_swizzle<D>(ln)) * 16);
+  }
   {
     const int blk = lane >> 4, e = (lane >> 2) & 3, c4 = lane & 3;
     const int krl = 4 * hh + e;
@@ -407,21 +445,21 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
 
   // per-lane LDS addresses of the operands of MFMA phase i: V(i) and K(i+1); computed before the
   // barrier that opens the phase
-  auto operand_addresses = [&](int i, unsigned (&va)[D / 32], unsigned (&ka)[D / 16]) {
+  auto operand_addresses = [&](int i, unsigned (&va)[D / 32], unsigned (&ka)[NKA]) {
     const unsigned vb = v_lds(i), kb = k_lds(i + 1);
 #pragma unroll
     for (int db = 0; db < D / 32; ++db) va[db] = vra[db] + vb;
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) ka[ks] = kra[ks] + kb;
+    for (int ks = 0; ks < NKA; ++ks) ka[ks] = kra[ks] + kb;
   };
 
   // MFMA phase of step i: O += V(i)^T P(i) (if PV) followed by S(i+1) = K(i+1) Q^T (if NS).
   // The LDS operand of MFMA number j is fetched LOOK MFMAs ahead of its use, so the whole
   // phase runs off a rolling window of LOOK fragments instead of stalling on every read.
-  auto mfma_phase = [&](auto do_pv, auto do_s, const unsigned (&va)[D / 32], const unsigned (&ka)[D / 16], frag (&pfr)[NT][2], auto&& side) {
+  auto mfma_phase = [&](auto do_pv, auto do_s, const unsigned (&va)[D / 32], const unsigned (&ka)[NKA], frag (&pfr)[NT][2], auto&& side) {
     constexpr bool PV = decltype(do_pv)::value, NS = decltype(do_s)::value;
     constexpr int NPV = PV ? (D / 32) * (BN / 16) : 0;
-    constexpr int NSS = NS ? (D / 16) * NT : 0;
+    constexpr int NSS = NS ? NKA * NT : 0;  // 16-byte K reads: one per 16-bit MFMA, two per 8-bit one
     constexpr int TOTAL = NPV + NSS;
     constexpr int LOOK = KV8 && D == 64 ? FWD_LOOK - 2 : FWD_LOOK;  // (the staged e4m3 bytes take the registers of two fragments)
     auto fetch = [&](int j) -> frag {
@@ -438,7 +476,11 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
         x[3] = r1[1];
         return as_frag<frag>(x);
       }
-      const int jj = j - NPV;  // jj = ks*NT + t
+      const int jj = j - NPV;  // jj = ks*NT + t;  QK8: jj = (kk*NT + t)*2 + which half of the 32 bytes
+      if constexpr (QK8) {
+        const int half = jj & 1, t = (jj >> 1) % NT, kk = (jj >> 1) / NT;
+        return as_frag<frag>(*(const __attribute__((address_space(3))) u32x4*)((const lds_u8*)(uintptr_t)ka[2 * kk + half] + t * 32 * ROWB8));
+      }
       const int t = jj % NT, ks = jj / NT;
       return as_frag<frag>(*(const __attribute__((address_space(3))) u32x4*)((const lds_u8*)(uintptr_t)ka[ks] + t * 32 * C::ROWB));
     };
@@ -447,6 +489,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     for (int j = 0; j < LOOK && j < TOTAL; ++j) win[j] = fetch(j);
     // scheduling fences keep the compiler from sinking each read back next to its use
     __builtin_amdgcn_sched_barrier(0);
+    frag klo;  // QK8: the first half of an 8-bit operand waits here for the second
 #pragma unroll
     for (int j = 0; j < TOTAL; ++j) {
       const frag a = win[j % LOOK];
@@ -455,6 +498,28 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       if (j < NPV) {
         const int db = j % (D / 32), tu = j / (D / 32);
         o[db] = M::run(a, pfr[tu >> 1][tu & 1], o[db]);
+      } else if constexpr (QK8) {
+        const int jj = j - NPV;
+        const int half = jj & 1, t = (jj >> 1) % NT, kk = (jj >> 1) / NT;
+        if (half == 0) {
+          klo = a;
+        } else {
+          const u32x4 x0 = __builtin_bit_cast(u32x4, klo), x1 = __builtin_bit_cast(u32x4, a);
+          i32x8 ka8;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            ka8[i] = (int)x0[i];
+            ka8[4 + i] = (int)x1[i];
+          }
+          f32x16 acc;
+          if (kk == 0) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+          } else {
+            acc = s[t];
+          }
+          s[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka8, qf8[kk], acc, 0, 0, 0, 0, 0, 0);  // e4m3 x e4m3, unscaled
+        }
       } else {
         const int jj = j - NPV;
         const int t = jj % NT, ks = jj / NT;
@@ -591,26 +656,26 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   ck = cv;
   cursor_next(ck);
 #pragma unroll
-  for (int q = 0; q < C::NDMA; ++q) load_one(q, 0 < n, cs.sb.krow, k_lds(0), false, 0, 0);            // K(0)
+  for (int q = 0; q < NK; ++q) load_one(q, 0 < n, cs.sb.krow, k_lds(0), false, 0, 0);                 // K(0)
 #pragma unroll
-  for (int q = 0; q < C::NDMA; ++q) load_one(C::NDMA + q, false, 0, 0, 0 < n, cs.sb.krow, v_lds(0));   // V(0)
-  if constexpr (KV8) {
+  for (int q = 0; q < C::NDMA; ++q) load_one(NK + q, false, 0, 0, 0 < n, cs.sb.krow, v_lds(0));        // V(0)
+  if constexpr (KSTAGE) {
     // K(0) goes to LDS now; V(0) stays staged together with K(1), loaded next, and both are written
     // by the first VALU phase like every later pair
 #pragma unroll
-    for (int q = 0; q < C::NDMA; ++q)
+    for (int q = 0; q < NK; ++q)
       *(__attribute__((address_space(3))) u32x4*)(lds_u8*)(uintptr_t)(lds_group + (unsigned)tg * 16 + k_lds(0) + q * (C::DTHREADS * 16)) = widen(stage[q]);
   }
 #pragma unroll
-  for (int q = 0; q < C::NDMA; ++q) load_one(q, 1 < n, cv.sb.krow, k_lds(1), false, 0, 0);            // K(1)
-  // S(0) needs Q and K(0) only: loads complete in the order of issue, so at most the 2 NDMA loads
-  // of V(0) and K(1) may still be in flight here; they are waited for before the barrier that
+  for (int q = 0; q < NK; ++q) load_one(q, 1 < n, cv.sb.krow, k_lds(1), false, 0, 0);                 // K(1)
+  // S(0) needs Q and K(0) only: loads complete in the order of issue, so at most the loads of V(0)
+  // and K(1) may still be in flight here; they are waited for before the barrier that
   // opens the first MFMA phase reading them.
-  __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * C::NDMA) & 15) | (((2 * C::NDMA) >> 4) << 14));  // vmcnt(2 NDMA)
+  __builtin_amdgcn_s_waitcnt(0x0F70 | ((NK + C::NDMA) & 15) | (((NK + C::NDMA) >> 4) << 14));  // vmcnt(loads of V(0), K(1))
   __syncthreads();
   {
     frag none[NT][2];
-    unsigned va[D / 32], ka[D / 16];
+    unsigned va[D / 32], ka[NKA];
     operand_addresses(-1, va, ka);
     mfma_phase(std::false_type{}, std::true_type{}, va, ka, none, [](int) {});  // S(0)
   }
@@ -642,11 +707,11 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       for (int q = 0; q < NLOADS; ++q) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb);
     }
     softmax_phase(cs.sb, pf);
-    unsigned va[D / 32], ka[D / 16];
+    unsigned va[D / 32], ka[NKA];
 #pragma unroll
     for (int db = 0; db < D / 32; ++db) va[db] = vra[db] + (unsigned)(2 * C::TILEB + PAR * C::TILEB);  // v_lds(i)
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) ka[ks] = kra[ks] + (unsigned)((PAR ^ 1) * C::TILEB);            // k_lds(i + 1)
+    for (int ks = 0; ks < NKA; ++ks) ka[ks] = kra[ks] + (unsigned)((PAR ^ 1) * C::TILEB);               // k_lds(i + 1)
     // Shared buffers need one barrier per step and group (after the wait for the loads: group 0
     // at the end of its VALU phase, group 1 at the end of its MFMA phase, the same physical
     // barrier); the other one only holds the two groups in step, and they drift little without it.
@@ -657,7 +722,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     if (!SHARE || !early) __syncthreads();
     __builtin_amdgcn_s_setprio(3);
     mfma_phase(std::true_type{}, std::true_type{}, va, ka, pf, [&](int j) {
-      constexpr int TOTAL = (D / 32) * (BN / 16) + (D / 16) * NT;
+      constexpr int TOTAL = (D / 32) * (BN / 16) + NKA * NT;
 #pragma unroll
       for (int q = 0; q < NLOADS; ++q)
         if ((q * TOTAL + TOTAL / 2) / NLOADS == j && !early) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb);
@@ -683,7 +748,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   {  // last sub-tile: nothing to prepare behind it
     frag pf[NT][2];
     softmax_phase(cs.sb, pf);
-    unsigned va[D / 32], ka[D / 16];
+    unsigned va[D / 32], ka[NKA];
     operand_addresses(n - 1, va, ka);
     loads_landed();
     if (!early) store_staged(k_lds(n), v_lds(n - 1));  // V(n - 1) (and whatever K(n) stands for: never read)
@@ -1234,6 +1299,26 @@ hipError_t launch16_big(const FwdParams& p, hipStream_t stream) {
   return launch<flash_fwd16_kernel<T, D, 2, false, false, false, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
 }
 
+// e4m3 q, k, v with the scores on the 8-bit matrix instruction (D = 128, plain block calls): chosen like the others.
+template <typename T>
+hipError_t launch16_qk8(FwdParams p, hipStream_t stream) {
+  constexpr int D = 128;
+  const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
+  const int force_share = spa_knob(SPA_KNOB_FWD_SHARE);
+  const bool two = force ? force == 2 : p.Sk > fwd_bn<D>();
+  if (two) {
+    const int nqt2 = fwd_tiles(p, 2 * FWD_BM);
+    const int64_t wgs = (int64_t)p.B * p.H * nqt2 * p.nranks;
+    const bool share = force_share ? force_share == 2 : wgs >= 2 * (int64_t)spa_device_cus();
+    if (share) {
+      p.nqt = nqt2;
+      return launch<flash_fwd16_kernel<T, D, 2, true, true, false, false, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, true>::SMEM, p, stream);
+    }
+    return launch<flash_fwd16_kernel<T, D, 2, false, true, false, false, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+  }
+  return launch<flash_fwd16_kernel<T, D, 1, false, true, false, false, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+}
+
 // (dtype, D) -> kernel family; the zigzag variants are instantiated beside the plain ones
 template <bool ZZ>
 hipError_t launch16_any(const FwdParams& p, int D, int dtype, hipStream_t stream) {
@@ -1263,13 +1348,20 @@ hipError_t launch16_any(const FwdParams& p, int D, int dtype, hipStream_t stream
 }  // namespace
 
 // This file makes three objects: compiled with SPA_FWD_ZIGZAG_UNIT it holds the zigzag variants of the 16-bit
-// kernel and nothing else, with SPA_FWD_BIG_UNIT the re-based variants, without either everything else (so that
-// the parts compile side by side).
+// kernel and nothing else, with SPA_FWD_BIG_UNIT the re-based variants and those with 8-bit scores, without either
+// everything else (so that the parts compile side by side).
 #if defined(SPA_FWD_ZIGZAG_UNIT)
 hipError_t spa_launch_fwd16_zigzag(const FwdParams& p, int D, int dtype, hipStream_t stream) {
   return launch16_any<true>(p, D, dtype, stream);
 }
 #elif defined(SPA_FWD_BIG_UNIT)
+hipError_t spa_launch_fwd16_qk8(const FwdParams& p, int D, int dtype, hipStream_t stream) {
+  if (D != 128 || !p.q_scale || !p.k_scale || !p.v_scale || p.zigzag || p.big || p.epi != SPA_EPI_PLAIN || p.P != 1)
+    return hipErrorInvalidValue;
+  if (dtype == 1) return launch16_qk8<__bf16>(p, stream);
+  if (dtype == 2) return launch16_qk8<_Float16>(p, stream);
+  return hipErrorInvalidValue;
+}
 hipError_t spa_launch_fwd16_big(const FwdParams& p, int D, int dtype, hipStream_t stream) {
   if (p.k_scale || p.zigzag) return hipErrorInvalidValue;  // no re-based e4m3 or zigzag variants
   if (dtype == 1) {
@@ -1286,6 +1378,7 @@ hipError_t spa_launch_fwd16_big(const FwdParams& p, int D, int dtype, hipStream_
 #else
 hipError_t spa_launch_fwd16_zigzag(const FwdParams& p, int D, int dtype, hipStream_t stream);
 hipError_t spa_launch_fwd16_big(const FwdParams& p, int D, int dtype, hipStream_t stream);
+hipError_t spa_launch_fwd16_qk8(const FwdParams& p, int D, int dtype, hipStream_t stream);
 
 // Returns hipSuccess, or hipErrorInvalidValue for an unsupported (dtype, D).
 hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream) {
@@ -1303,6 +1396,7 @@ hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t strea
     p.out = (char*)slots.out<char>(p.part, p.part_slot) - row0 * p.os.s * 2;
     p.lse = slots.lse(p.part, p.P, p.part_slot) - row0;
   }
+  if ((dtype == 1 || dtype == 2) && p.q_scale) return spa_launch_fwd16_qk8(p, D, dtype, stream);
   if (dtype == 1 || dtype == 2)
     return p.big ? spa_launch_fwd16_big(p, D, dtype, stream)
                  : p.zigzag ? spa_launch_fwd16_zigzag(p, D, dtype, stream) : launch16_any<false>(p, D, dtype, stream);

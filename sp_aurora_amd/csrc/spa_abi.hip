@@ -189,6 +189,43 @@ int spa_flash_fwd_fp8kv(const void* q, const void* k8, const void* v8, const flo
                    v_strides, o_strides, scale, mask_mode, dtype, stream);
 }
 
+int spa_flash_fwd_fp8qkv(const void* q8, const void* k8, const void* v8, const float* q_scale, const float* k_scale,
+                         const float* v_scale, void* out, float* lse, int B, int H, int Sq, int Sk, int D,
+                         const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                         const int64_t o_strides[3], float scale, int mask_mode, int dtype, void* stream) {
+  const char* what = "spa_flash_fwd_fp8qkv";
+  if (!q8 || !k8 || !v8 || !out || !lse) return fail(SPA_EINVAL, "%s: null pointer", what);
+  if (!q_scale || !k_scale || !v_scale) return fail(SPA_EINVAL, "%s: null scale pointer", what);
+  if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(SPA_EINVAL, "%s: null strides", what);
+  if (!dims_ok(B, H, Sq, D) || Sk <= 0) return fail(SPA_EINVAL, "%s: sizes must be positive (B=%d H=%d Sq=%d Sk=%d D=%d)", what, B, H, Sq, Sk, D);
+  if (dtype != SPA_BF16 && dtype != SPA_F16) return fail(dtype == SPA_F32 ? SPA_EUNSUPPORTED : SPA_EINVAL, "%s: out must be bf16 or fp16 (dtype %d)", what, dtype);
+  if (mask_mode != SPA_MASK_NONE && mask_mode != SPA_MASK_CAUSAL) return fail(SPA_EINVAL, "%s: bad mask_mode %d", what, mask_mode);
+  if (!scale_ok(scale)) return fail(SPA_EINVAL, "%s: softmax scale must be finite", what);
+  if (D != 128) return fail(SPA_EUNSUPPORTED, "%s: head dim %d, built for 128", what, D);
+  if (!aligned16(q8, q_strides, 1) || !aligned16(k8, k_strides, 1) || !aligned8(v8, v_strides, 3) || !aligned16(out, o_strides, 2) ||
+      (((uintptr_t)q_scale | (uintptr_t)k_scale | (uintptr_t)v_scale | (uintptr_t)lse) & 3) != 0)
+    return fail(SPA_EALIGN, "%s: q8, k8, out: pointers and rows 16-byte aligned; v8: 8-byte aligned", what);
+  if ((int64_t)B * H > 0x7fffffffLL || (Sq + 127) / 128 > 65535) return fail(SPA_EINVAL, "%s: grid too large", what);
+  if (!span_ok(Sk, k_strides[2], D, 1) || !span_ok(Sk, v_strides[2], D, 1))
+    return fail(SPA_EUNSUPPORTED, "%s: K/V of one (batch, head) span 2 GiB or more (not supported for e4m3 K/V)", what);
+  FwdParams p;
+  p.q = q8; p.k = k8; p.v = v8; p.out = out; p.lse = lse;
+  p.B = B; p.H = H; p.Sq = Sq; p.Sk = Sk;
+  p.qs = S3(q_strides); p.ks = S3(k_strides); p.vs = S3(v_strides); p.os = S3(o_strides);
+  p.scale = scale_eff(scale);
+  p.scale_log2 = fabsf(scale_eff(scale)) * 1.4426950408889634f;
+  p.negq = scale < 0.f;
+  p.causal = mask_mode == SPA_MASK_CAUSAL;
+  p.nqt = 0;
+  p.lse_bh = Sq;
+  p.part = nullptr; p.part_slot = 0; p.npart = 0;
+  p.epi = SPA_EPI_PLAIN;
+  p.P = 1; p.rank0 = 0; p.nranks = 1; p.t_begin = 0; p.t_count = -1;
+  p.cu_q = nullptr; p.cu_k = nullptr;
+  p.k_scale = k_scale; p.v_scale = v_scale; p.q_scale = q_scale;
+  return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), what);
+}
+
 int spa_merge(float* out_acc, float* lse_acc, const void* blk_out, const float* blk_lse, int B, int H, int Sq,
               int D, const int64_t acc_strides[3], const int64_t blk_strides[3], int blk_dtype, int init,
               void* stream) {

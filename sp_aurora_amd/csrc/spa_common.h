@@ -9,6 +9,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 struct Strides3 {
   int64_t b, h, s;  // element strides of (batch, head, seq); head-dim stride is 1
@@ -50,6 +51,8 @@ struct FwdParams {
   // V = v8 * v_scale[b*H + h], fp32, one per (batch or sequence, head); strides of k, v in bytes
   const float* k_scale;
   const float* v_scale;
+  // e4m3 q as well (null: q has the type of out): Q = q8 * q_scale[b*H + h]; strides of q in bytes
+  const float* q_scale = nullptr;
   // zigzag sharding of a causal ring (16-bit kernels; 0: contiguous chunks): the chunk of rank r holds
   // half-chunks r and 2P-1-r of the sequence, Sq/2 rows each.  Step 0 is plain causal attention on the
   // rank's own chunk; at step t >= 1 (chunk c = (r - t) mod P) every local query sees the first half of

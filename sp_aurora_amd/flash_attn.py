@@ -32,11 +32,14 @@ def intel_flash_attn_forward(q, k, v, dropout_p=0.0, softmax_scale=None, causal=
     softmax_scale None -> D ** -0.5 (:46-47).  Returns (out [B,H,Sq,D] in q.dtype, lse fp32 [B,H,Sq]).
 
     Additive: k, v may be torch.float8_e4m3fn (a quantised KV cache) with keyword arguments
-    k_scale, v_scale (fp32 [B,H]: K = k * k_scale[b,h], V = v * v_scale[b,h]); q stays bf16 / fp16.
+    k_scale, v_scale (fp32 [B,H]: K = k * k_scale[b,h], V = v * v_scale[b,h]); q stays bf16 / fp16, or is
+    torch.float8_e4m3fn too with q_scale (fp32 [B,H]) and out_dtype (bf16 / fp16): D = 128, scores on the 8-bit
+    matrix instruction.
     """
     _check_unsupported(dropout_p, window_size, alibi_slopes, return_softmax)
     return ops.flash_fwd(q, k, v, softmax_scale, bool(causal), layout="bhsd",
-                         k_scale=kwargs.get("k_scale"), v_scale=kwargs.get("v_scale"))
+                         k_scale=kwargs.get("k_scale"), v_scale=kwargs.get("v_scale"), q_scale=kwargs.get("q_scale"),
+                         out_dtype=kwargs.get("out_dtype", torch.bfloat16))
 
 
 def intel_flash_attn_backward(dout, q, k, v, out, softmax_lse, dq=None, dk=None, dv=None, dropout_p=0.0,

@@ -123,12 +123,17 @@ def prepared(fn, *args, **kwargs):
     return run, result
 
 
-def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None, lse=None, k_scale=None, v_scale=None):
+def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None, lse=None, k_scale=None, v_scale=None,
+              q_scale=None, out_dtype=torch.bfloat16):
     """Block attention forward -> (out like q, lse fp32 [B,H,Sq]).  Calls spa_flash_fwd, or
     spa_flash_fwd_fp8kv when k, v are torch.float8_e4m3fn (then k_scale, v_scale fp32 [B,H] give
-    K = k * k_scale[b,h], V = v * v_scale[b,h]; q bf16 or fp16)."""
+    K = k * k_scale[b,h], V = v * v_scale[b,h]; q bf16 or fp16), or spa_flash_fwd_fp8qkv when q is
+    torch.float8_e4m3fn as well (q_scale fp32 [B,H]; D = 128; out in `out_dtype`, bf16 or fp16): the scores
+    then run on the 8-bit matrix instruction."""
     lib = _lib.load()
     fp8 = k.dtype == FP8 or v.dtype == FP8
+    if q.dtype == FP8:
+        return _flash_fwd_fp8qkv(lib, q, k, v, softmax_scale, causal, layout, out, lse, q_scale, k_scale, v_scale, out_dtype)
     if fp8:
         q = _prep(q)
         k, v = [t if t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1]) and t.data_ptr() % 8 == 0 else t.contiguous() for t in (k, v)]
@@ -159,6 +164,40 @@ def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None
                                                out.data_ptr(), lse.data_ptr(), *tail))
         else:
             _lib.check(lib.spa_flash_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), *tail))
+    return out, lse
+
+
+def _flash_fwd_fp8qkv(lib, q, k, v, softmax_scale, causal, layout, out, lse, q_scale, k_scale, v_scale, out_dtype):
+    if k.dtype != FP8 or v.dtype != FP8:
+        raise TypeError("e4m3 q goes with e4m3 k and v")
+    if out_dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError("e4m3 q: out_dtype must be bfloat16 or float16")
+    ok16 = lambda t: t.is_cuda and t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 16 == 0 for s in t.stride()[:-1])
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        if not t.is_cuda:
+            raise ValueError("sp_aurora_amd kernels need tensors on a HIP device (got a CPU tensor)")
+    q, k, v = [t if ok16(t) else t.contiguous() for t in (q, k, v)]
+    (B, H, Sq, D), qs = _bhs(q, layout)
+    (Bk, Hk, Sk, Dk), ks = _bhs(k, layout)
+    shp_v, vs = _bhs(v, layout)
+    if (Bk, Hk, Dk) != (B, H, D) or shp_v != (Bk, Hk, Sk, Dk):
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    if q_scale is None or tuple(q_scale.shape) != (B, H):
+        raise ValueError(f"e4m3 q needs q_scale (fp32 {(B, H)})")
+    ksc, vsc = _fp8_scales(k, v, k_scale, v_scale, B, H)
+    qsc = q_scale.to(device=q.device, dtype=torch.float32).contiguous()
+    if softmax_scale is None:
+        softmax_scale = D ** (-0.5)
+    if out is None:
+        out = torch.empty(q.shape, dtype=out_dtype, device=q.device)
+    if lse is None:
+        lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    _, os_ = _bhs(out, layout)
+    with _on(q.device):
+        _lib.check(lib.spa_flash_fwd_fp8qkv(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), qsc.data_ptr(), ksc.data_ptr(), vsc.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            B, H, Sq, Sk, D, _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
+            float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(out), _stream()))
     return out, lse
 
 

@@ -11,7 +11,7 @@ import torch
 from conftest import rand
 from oracle import attn_oracle as O
 import sp_aurora_amd as spa
-from sp_aurora_amd import ops
+from sp_aurora_amd import _lib, ops
 from test_gpu_parity import DEV, check_lse, check_out
 from test_gpu_varlen import cu_of, per_sequence
 
@@ -189,3 +189,58 @@ def test_e4m3_kv_argument_checks():
         ops.flash_fwd(q, k8, q, layout="bhsd", k_scale=sc, v_scale=sc)
     with pytest.raises(spa._lib.SpaError):  # fp32 queries have no e4m3 K/V kernel
         ops.flash_fwd(q.float(), k8, k8, layout="bhsd", k_scale=sc, v_scale=sc)
+
+
+# ------------------------------------------------------------------ e4m3 q as well: scores on the 8-bit matrix instruction
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,Sq,Sk,causal", [
+    (1, 32, 1024, 1024, False),    # one block pair of benchmark config 3 (full)
+    (1, 4, 1024, 1024, True),      # config 3, diagonal
+    (1, 16, 4096, 4096, True),     # enough workgroups for the 256-row form
+    (1, 2, 130, 515, False), (2, 3, 300, 300, True), (1, 1, 77, 200, True),
+    (1, 2, 512, 129, True), (1, 1, 1, 65, False), (1, 2, 50, 40, False), (1, 1, 200, 1, False), (1, 1, 64, 64, True),
+])
+def test_block_forward_with_e4m3_q_k_v(B, H, Sq, Sk, causal, dtype):
+    """spa_flash_fwd_fp8qkv against the oracle on the dequantised q, k, v: a product of two e4m3 values is exact in
+    fp32, so the scores differ from the oracle's only by the order of the fp32 additions; same tolerances as every
+    16-bit kernel (out atol 2e-2 / rtol 1.6e-2, lse atol 1e-3).  No reference output exists for an 8-bit path."""
+    D = 128
+    q8, qsc, q_deq = quantised((B, H, Sq, D), 520, "bhsd", spread=1.2)
+    k8, ksc, k_deq = quantised((B, H, Sk, D), 521, "bhsd", spread=1.5)
+    v8, vsc, v_deq = quantised((B, H, Sk, D), 522, "bhsd", spread=0.7)
+    want_out, want_lse = O.attn_block(q_deq, k_deq, v_deq, None, causal)
+    for share, groups in ((0, 0), (1, 1), (1, 2), (2, 2)):
+        _lib.tune("fwd_share", share)
+        _lib.tune("fwd_groups", groups)
+        try:
+            out, lse = ops.flash_fwd(q8.to(DEV), k8.to(DEV), v8.to(DEV), None, causal, layout="bhsd", q_scale=qsc, k_scale=ksc,
+                                     v_scale=vsc, out_dtype=dtype)
+        finally:
+            _lib.tune("fwd_share", 0)
+            _lib.tune("fwd_groups", 0)
+        assert out.dtype == dtype and lse.dtype == torch.float32
+        check_out(out, want_out, dtype, f"share={share} groups={groups}")
+        check_lse(lse, want_lse)
+    out2, lse2 = spa.intel_flash_attn_forward(q8.to(DEV), k8.to(DEV), v8.to(DEV), causal=causal, q_scale=qsc, k_scale=ksc, v_scale=vsc,
+                                              out_dtype=dtype)
+    check_out(out2, want_out, dtype, "operator shim")
+
+
+def test_e4m3_q_k_v_public_layout_negative_scale_and_argument_checks():
+    B, S, H, D = 2, 200, 3, 128
+    q8, qsc, q_deq = quantised((B, S, H, D), 530, "bshd")
+    k8, ksc, k_deq = quantised((B, S, H, D), 531, "bshd")
+    v8, vsc, v_deq = quantised((B, S, H, D), 532, "bshd")
+    for scale in (None, -0.07, 0.0):
+        want_out, want_lse = O.full_attention(q_deq, k_deq, v_deq, scale, True)
+        out, lse = ops.flash_fwd(q8.to(DEV), k8.to(DEV), v8.to(DEV), scale, True, q_scale=qsc, k_scale=ksc, v_scale=vsc)
+        check_out(out, want_out, torch.bfloat16, f"scale {scale}")
+        check_lse(lse, want_lse)
+    with pytest.raises(ValueError):
+        ops.flash_fwd(q8.to(DEV), k8.to(DEV), v8.to(DEV), None, True, k_scale=ksc, v_scale=vsc)             # no q_scale
+    with pytest.raises(TypeError):
+        ops.flash_fwd(q8.to(DEV), k_deq.bfloat16().to(DEV), v8.to(DEV), None, True, q_scale=qsc, k_scale=ksc, v_scale=vsc)
+    q64 = q8[..., :64].contiguous()
+    with pytest.raises(_lib.SpaError):  # head dim 64: no 8-bit score variant
+        ops.flash_fwd(q64.to(DEV), k8[..., :64].contiguous().to(DEV), v8[..., :64].contiguous().to(DEV), None, True, q_scale=qsc,
+                      k_scale=ksc, v_scale=vsc)

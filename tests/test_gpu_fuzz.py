@@ -49,7 +49,7 @@ def _case(rng):
     D, H, B = rng.choice([32, 64, 128]), rng.choice([1, 2, 3]), rng.choice([1, 2])
     causal = rng.random() < 0.5
     kind = rng.choice(["block", "block", "ring", "ring_bwd", "fp8", "fp8", "fp8_ring", "varlen", "block_bwd", "block_bwd",
-                       "varlen_bwd", "varlen_bwd", "zigzag", "zigzag"])
+                       "varlen_bwd", "varlen_bwd", "zigzag", "zigzag", "fp8_qkv"])
     share, groups = rng.choice([0, 0, 1, 2, 2]), rng.choice([0, 0, 1, 2])
     _lib.tune("fwd_share", share)
     _lib.tune("fwd_groups", groups)
@@ -57,6 +57,18 @@ def _case(rng):
     mk = lambda *shape, dt=None: torch.randn(shape, generator=g).to(dt or dtype)
     atol, rtol = OUT_TOL[dtype]
     if kind in ("fp8", "fp8_ring") and (dtype == torch.float32 or D == 32):
+        return
+    if kind == "fp8_qkv":  # e4m3 q as well: scores on the 8-bit matrix instruction, D = 128
+        dt = rng.choice([torch.bfloat16, torch.float16])
+        Sq, Sk = rng.choice([1, 64, 100, 128, 256, 300, 513]), rng.choice([1, 64, 65, 128, 200, 513, 769])
+        info = (kind, dt, B, H, Sq, Sk, causal, share, groups)
+        qf, kf, vf = (mk(B, H, n_, 128, dt=torch.float32) for n_ in (Sq, Sk, Sk))
+        (q8, qs), (k8, ks), (v8, vs) = (ops.quantize_fp8_per_head(t, "bhsd") for t in (qf, kf, vf))
+        deq = lambda x8, sc: x8.double() * sc[:, :, None, None].double()
+        want_o, want_l = O.attn_block(deq(q8, qs), deq(k8, ks), deq(v8, vs), None, causal)
+        o, l = ops.flash_fwd(q8.to(DEV), k8.to(DEV), v8.to(DEV), None, causal, layout="bhsd", q_scale=qs, k_scale=ks, v_scale=vs, out_dtype=dt)
+        _close("out", o, want_o, *OUT_TOL[dt], info)
+        _close("lse", l, want_l, LSE_ATOL, 0, info)
         return
     if kind == "block":
         Sq = rng.choice([1, 7, 64, 65, 127, 128, 129, 200, 256, 300, 513, 700])
