@@ -196,6 +196,20 @@ int spa_ring_fwd_fp8kv(const void* q, const void* k8, const void* v8,
                        float scale, int mask_mode, int dtype, int fuse, void* stream);
 
 /*
+ * spa_ring_fwd with q, K, V all e4m3 as in spa_flash_fwd_fp8qkv (q_scale, k_scale, v_scale fp32 contiguous [B,H], one
+ * scale per (batch, head) for the whole sequence; D = 128; out and the ring-step slots in `dtype`, bf16 or fp16): the
+ * scores of every block pair run on the 8-bit matrix instruction.  All three `fuse` modes, contiguous chunks (no
+ * SPA_RING_ZIGZAG); workspace as for spa_ring_fwd.  The reference has no 8-bit path.
+ */
+int spa_ring_fwd_fp8qkv(const void* q8, const void* k8, const void* v8,
+                        const float* q_scale, const float* k_scale, const float* v_scale,
+                        void* out, float* lse, void* workspace,
+                        int B, int H, int S, int D, int P, int rank,
+                        const int64_t q_strides[3], const int64_t k_strides[3],
+                        const int64_t v_strides[3], const int64_t o_strides[3],
+                        float scale, int mask_mode, int dtype, int fuse, void* stream);
+
+/*
  * spa_ring_fwd for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc): the same call without the workspace
  * argument.  The scratch is a fixed buffer of SPA_STATIC_SCRATCH_BYTES inside the library's

@@ -31,6 +31,7 @@ SIGNATURES = {
     "spa_flash_fwd_fp8qkv": (_i, [_vp] * 8 + [_i] * 5 + [_s3] * 4 + [_f, _i, _i, _vp]),
     "spa_flash_fwd_varlen_fp8kv": (_i, [_vp] * 9 + [_i] * 7 + [_s3] * 4 + [_f, _i, _i, _vp]),
     "spa_ring_fwd_fp8kv": (_i, [_vp] * 8 + [_i] * 6 + [_s3] * 4 + [_f, _i, _i, _i, _vp]),
+    "spa_ring_fwd_fp8qkv": (_i, [_vp] * 9 + [_i] * 6 + [_s3] * 4 + [_f, _i, _i, _i, _vp]),
     "spa_ring_fwd_workspace_bytes": (ctypes.c_int64, [_i, _i, _i, _i, _i, _i]),
     "spa_ring_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _i, _vp]),
     "spa_static_scratch_bytes": (ctypes.c_int64, []),

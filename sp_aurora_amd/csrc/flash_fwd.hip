@@ -102,7 +102,7 @@ template <typename T, int D, int NG, bool SHARE, bool KV8 = false, bool FINALN =
           bool QK8 = false>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams pk) {
   static_assert(!(FINALN && SHARE), "the merging epilogue goes with 128-row workgroups");
-  static_assert(!QK8 || (KV8 && D == 128 && !FINALN && !ZZ && !BIG), "8-bit scores: e4m3 q, k, v, head dim 128, plain block calls");
+  static_assert(!QK8 || (KV8 && D == 128 && !ZZ && !BIG), "8-bit scores: e4m3 q, k, v, head dim 128, contiguous chunks");
   typedef typename std::conditional<KV8, unsigned char, T>::type KVT;  // element type of K / V in memory
   typedef typename std::conditional<QK8, unsigned char, T>::type QT;   // element type of q in memory
   constexpr bool KSTAGE = KV8 && !QK8;  // K tiles go through registers (widened on the way); V tiles do whenever KV8
@@ -1299,13 +1299,17 @@ hipError_t launch16_big(const FwdParams& p, hipStream_t stream) {
   return launch<flash_fwd16_kernel<T, D, 2, false, false, false, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
 }
 
-// e4m3 q, k, v with the scores on the 8-bit matrix instruction (D = 128, plain block calls): chosen like the others.
+// e4m3 q, k, v with the scores on the 8-bit matrix instruction (D = 128, block and ring calls): chosen like the others.
 template <typename T>
 hipError_t launch16_qk8(FwdParams p, hipStream_t stream) {
   constexpr int D = 128;
   const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
   const int force_share = spa_knob(SPA_KNOB_FWD_SHARE);
   const bool two = force ? force == 2 : p.Sk > fwd_bn<D>();
+  if (p.epi == SPA_EPI_FINALN) {
+    if (two) return launch<flash_fwd16_kernel<T, D, 2, false, true, true, false, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+    return launch<flash_fwd16_kernel<T, D, 1, false, true, true, false, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+  }
   if (two) {
     const int nqt2 = fwd_tiles(p, 2 * FWD_BM);
     const int64_t wgs = (int64_t)p.B * p.H * nqt2 * p.nranks;
@@ -1356,8 +1360,7 @@ hipError_t spa_launch_fwd16_zigzag(const FwdParams& p, int D, int dtype, hipStre
 }
 #elif defined(SPA_FWD_BIG_UNIT)
 hipError_t spa_launch_fwd16_qk8(const FwdParams& p, int D, int dtype, hipStream_t stream) {
-  if (D != 128 || !p.q_scale || !p.k_scale || !p.v_scale || p.zigzag || p.big || p.epi != SPA_EPI_PLAIN || p.P != 1)
-    return hipErrorInvalidValue;
+  if (D != 128 || !p.q_scale || !p.k_scale || !p.v_scale || p.zigzag || p.big || p.cu_q) return hipErrorInvalidValue;
   if (dtype == 1) return launch16_qk8<__bf16>(p, stream);
   if (dtype == 2) return launch16_qk8<_Float16>(p, stream);
   return hipErrorInvalidValue;

@@ -273,8 +273,9 @@ int static_scratch(void** ptr) {
 
 // `what` names the entry point in messages; `ws_bytes` < 0: the caller vouches for the workspace size.
 // k_scale / v_scale non-null: K and V are e4m3 bytes with one scale per (batch, head) for the whole sequence.
-int ring_fwd(const char* what, const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
-             void* out, float* lse, void* workspace,
+// q_scale non-null (with the other two): q is e4m3 as well and the scores run on the 8-bit matrix instruction (D = 128).
+int ring_fwd(const char* what, const void* q, const void* k, const void* v, const float* q_scale, const float* k_scale,
+             const float* v_scale, void* out, float* lse, void* workspace,
              int64_t ws_bytes, int B, int H, int S, int D, int P, int rank, const int64_t q_strides[3],
              const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3], float scale,
              int mask_mode, int dtype, int fuse, void* stream) {
@@ -296,10 +297,15 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   if (kv8 && (!k_scale || !v_scale)) return fail(SPA_EINVAL, "%s: null scale pointer", what);
   if (kv8 && dtype == SPA_F32) return fail(SPA_EUNSUPPORTED, "%s: e4m3 K/V go with bf16 or fp16 queries", what);
   if (kv8 && D == 32) return fail(SPA_EUNSUPPORTED, "%s: e4m3 K/V need head dim 64 or 128", what);
+  const bool qk8 = q_scale != nullptr;
+  if (qk8 && !kv8) return fail(SPA_EINVAL, "%s: e4m3 q goes with e4m3 K/V", what);
+  if (qk8 && D != 128) return fail(SPA_EUNSUPPORTED, "%s: e4m3 q: head dim %d, built for 128", what, D);
+  if (qk8 && zig_req) return fail(SPA_EUNSUPPORTED, "%s: e4m3 q has no zigzag variants", what);
   const int esz = elem_size(dtype), kesz = kv8 ? 1 : esz;
-  const bool kv_aligned = kv8 ? aligned8(k, k_strides, 3) && aligned8(v, v_strides, 3) && (((uintptr_t)k_scale | (uintptr_t)v_scale) & 3) == 0
-                              : aligned16(k, k_strides, esz) && aligned16(v, v_strides, esz);
-  if (!aligned16(q, q_strides, esz) || !kv_aligned ||
+  const bool kv_aligned = qk8   ? aligned16(k, k_strides, 1) && aligned8(v, v_strides, 3) && (((uintptr_t)q_scale | (uintptr_t)k_scale | (uintptr_t)v_scale) & 3) == 0
+                          : kv8 ? aligned8(k, k_strides, 3) && aligned8(v, v_strides, 3) && (((uintptr_t)k_scale | (uintptr_t)v_scale) & 3) == 0
+                                : aligned16(k, k_strides, esz) && aligned16(v, v_strides, esz);
+  if (!aligned16(q, q_strides, qk8 ? 1 : esz) || !kv_aligned ||
       !aligned16(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0 || ((uintptr_t)workspace & 15) != 0)
     return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned (8-byte for e4m3 K/V)", what);
   const bool big = !span_ok(S, k_strides[2], D, kesz) || !span_ok(S, v_strides[2], D, kesz);
@@ -346,7 +352,7 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   p.P = P;
   p.epi = SPA_EPI_PLAIN;
   p.cu_q = nullptr; p.cu_k = nullptr;
-  p.k_scale = k_scale; p.v_scale = v_scale;
+  p.k_scale = k_scale; p.v_scale = v_scale; p.q_scale = q_scale;
   p.zigzag = zig && dtype != SPA_F32;
   p.zz_half = 0;
   p.big = big && dtype != SPA_F32;
@@ -443,7 +449,7 @@ int spa_ring_fwd(const void* q, const void* k, const void* v, void* out, float* 
                  int H, int S, int D, int P, int rank, const int64_t q_strides[3], const int64_t k_strides[3],
                  const int64_t v_strides[3], const int64_t o_strides[3], float scale, int mask_mode, int dtype,
                  int fuse, void* stream) {
-  return ring_fwd("spa_ring_fwd", q, k, v, nullptr, nullptr, out, lse, workspace, -1, B, H, S, D, P, rank, q_strides, k_strides,
+  return ring_fwd("spa_ring_fwd", q, k, v, nullptr, nullptr, nullptr, out, lse, workspace, -1, B, H, S, D, P, rank, q_strides, k_strides,
                   v_strides, o_strides, scale, mask_mode, dtype, fuse, stream);
 }
 
@@ -452,7 +458,16 @@ int spa_ring_fwd_fp8kv(const void* q, const void* k8, const void* v8, const floa
                        const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
                        const int64_t o_strides[3], float scale, int mask_mode, int dtype, int fuse, void* stream) {
   if (!k_scale || !v_scale) return fail(SPA_EINVAL, "spa_ring_fwd_fp8kv: null scale pointer");
-  return ring_fwd("spa_ring_fwd_fp8kv", q, k8, v8, k_scale, v_scale, out, lse, workspace, -1, B, H, S, D, P, rank, q_strides,
+  return ring_fwd("spa_ring_fwd_fp8kv", q, k8, v8, nullptr, k_scale, v_scale, out, lse, workspace, -1, B, H, S, D, P, rank, q_strides,
+                  k_strides, v_strides, o_strides, scale, mask_mode, dtype, fuse, stream);
+}
+
+int spa_ring_fwd_fp8qkv(const void* q8, const void* k8, const void* v8, const float* q_scale, const float* k_scale,
+                        const float* v_scale, void* out, float* lse, void* workspace, int B, int H, int S, int D, int P, int rank,
+                        const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                        const int64_t o_strides[3], float scale, int mask_mode, int dtype, int fuse, void* stream) {
+  if (!q_scale || !k_scale || !v_scale) return fail(SPA_EINVAL, "spa_ring_fwd_fp8qkv: null scale pointer");
+  return ring_fwd("spa_ring_fwd_fp8qkv", q8, k8, v8, q_scale, k_scale, v_scale, out, lse, workspace, -1, B, H, S, D, P, rank, q_strides,
                   k_strides, v_strides, o_strides, scale, mask_mode, dtype, fuse, stream);
 }
 
@@ -470,7 +485,7 @@ int spa_ring_fwd_static(const void* q, const void* k, const void* v, void* out, 
   void* ws = nullptr;
   const int rc = static_scratch(&ws);
   if (rc != SPA_OK) return rc;
-  return ring_fwd("spa_ring_fwd_static", q, k, v, nullptr, nullptr, out, lse, ws, (int64_t)SPA_STATIC_SCRATCH_BYTES, B, H, S, D, P,
+  return ring_fwd("spa_ring_fwd_static", q, k, v, nullptr, nullptr, nullptr, out, lse, ws, (int64_t)SPA_STATIC_SCRATCH_BYTES, B, H, S, D, P,
                   rank, q_strides, k_strides, v_strides, o_strides, scale, mask_mode, dtype, fuse, stream);
 }
 

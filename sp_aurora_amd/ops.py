@@ -201,11 +201,12 @@ def _flash_fwd_fp8qkv(lib, q, k, v, softmax_scale, causal, layout, out, lse, q_s
     return out, lse
 
 
-def ring_fwd_workspace(q, ring_size, layout="bshd"):
-    """Scratch tensor spa_ring_fwd needs for this q and ring size (uint8, 16-byte aligned)."""
+def ring_fwd_workspace(q, ring_size, layout="bshd", out_dtype=None):
+    """Scratch tensor spa_ring_fwd needs for this q and ring size (uint8, 16-byte aligned); out_dtype: the type of
+    the result when q is e4m3."""
     lib = _lib.load()
     (B, H, S, D), _ = _bhs(q, layout)
-    nbytes = lib.spa_ring_fwd_workspace_bytes(B, H, S, D, int(ring_size), _dtype_code(q))
+    nbytes = lib.spa_ring_fwd_workspace_bytes(B, H, S, D, int(ring_size), _DT[out_dtype] if q.dtype == FP8 else _dtype_code(q))
     if nbytes < 0:
         raise ValueError(f"ring_size={ring_size} must divide the sequence length {S}")
     return torch.empty((nbytes,), dtype=torch.uint8, device=q.device)
@@ -215,12 +216,14 @@ RING_FUSE = {"step": _lib.SPA_RING_PER_STEP, "rank": _lib.SPA_RING_PER_RANK, "al
 
 
 def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layout="bshd", out=None, lse=None,
-             workspace=None, fuse="rank", static_scratch=False, k_scale=None, v_scale=None, sharding="contiguous"):
+             workspace=None, fuse="rank", static_scratch=False, k_scale=None, v_scale=None, sharding="contiguous",
+             q_scale=None, out_dtype=torch.bfloat16):
     """Simulated ring forward of one rank (or all, rank=-1) over the full-sequence q,k,v: one C call
     that enqueues the kernels in ring order.  Calls spa_ring_fwd.  `fuse`: "step" = one launch per
     (q chunk, kv chunk) pair, "rank" = one launch per rank walking its chunks, "all" = one launch.
     Returns (out like q, lse fp32 [B,H,S]); with rank >= 0 only that rank's rows are written.
-    k, v may be torch.float8_e4m3fn with k_scale, v_scale fp32 [B,H] (spa_ring_fwd_fp8kv).
+    k, v may be torch.float8_e4m3fn with k_scale, v_scale fp32 [B,H] (spa_ring_fwd_fp8kv); q as well, with q_scale
+    and the result's out_dtype (spa_ring_fwd_fp8qkv: D = 128, scores on the 8-bit matrix instruction).
     sharding="zigzag": the rows of q, k, v are in zigzag-sharded order (chunk r of the tensors holds
     half-chunks r and 2P-1-r of the sequence); out and lse come back in the same order.
     static_scratch=True calls spa_ring_fwd_static instead: no workspace tensor, the library's built-in
@@ -228,10 +231,19 @@ def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layo
     calls that overlap on one device race)."""
     lib = _lib.load()
     fp8 = k.dtype == FP8 or v.dtype == FP8
+    qk8 = q.dtype == FP8
+    if qk8:
+        if not fp8 or q_scale is None or out_dtype not in (torch.bfloat16, torch.float16):
+            raise ValueError("e4m3 q goes with e4m3 k, v, a q_scale and out_dtype bfloat16 or float16")
+        if not q.is_cuda:
+            raise ValueError("sp_aurora_amd kernels need tensors on a HIP device (got a CPU tensor)")
+        ok16 = lambda t: t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 16 == 0 for s in t.stride()[:-1])
+        q = q if ok16(q) else q.contiguous()
+        k = k if k.is_cuda and ok16(k) else k.contiguous()
     if fp8:
         if static_scratch:
             raise ValueError("static_scratch=True has no e4m3 K/V form")
-        q = _prep(q)
+        q = q if qk8 else _prep(q)
         k, v = [t if t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1]) and t.data_ptr() % 8 == 0 else t.contiguous() for t in (k, v)]
         if not k.is_cuda or not v.is_cuda:
             raise ValueError("sp_aurora_amd kernels need tensors on a HIP device (got a CPU tensor)")
@@ -247,7 +259,7 @@ def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layo
     if softmax_scale is None:
         softmax_scale = D ** (-0.5)
     if out is None:
-        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        out = torch.empty(q.shape, dtype=out_dtype if qk8 else q.dtype, device=q.device)
     if lse is None:
         lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
     if fuse not in RING_FUSE:
@@ -257,14 +269,22 @@ def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layo
     if static_scratch and workspace is not None:
         raise ValueError("static_scratch=True takes no workspace")
     if workspace is None and not static_scratch and (fuse == "step" or q.dtype == torch.float32):
-        workspace = ring_fwd_workspace(q, ring_size, layout)
+        workspace = ring_fwd_workspace(q, ring_size, layout, out.dtype)
     _, os_ = _bhs(out, layout)
     tail = (B, H, S, D, int(ring_size), int(rank),
             _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
             float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE,
-            _dtype_code(q), RING_FUSE[fuse] | (_lib.SPA_RING_ZIGZAG if sharding == "zigzag" else 0), _stream())
+            _dtype_code(out), RING_FUSE[fuse] | (_lib.SPA_RING_ZIGZAG if sharding == "zigzag" else 0), _stream())
     with _on(q.device):
-        if fp8:
+        if qk8:
+            ksc, vsc = _fp8_scales(k, v, k_scale, v_scale, B, H)
+            if tuple(q_scale.shape) != (B, H):
+                raise ValueError(f"q_scale must have shape {(B, H)}, got {tuple(q_scale.shape)}")
+            qsc = q_scale.to(device=q.device, dtype=torch.float32).contiguous()
+            _lib.check(lib.spa_ring_fwd_fp8qkv(q.data_ptr(), k.data_ptr(), v.data_ptr(), qsc.data_ptr(), ksc.data_ptr(), vsc.data_ptr(),
+                                               out.data_ptr(), lse.data_ptr(),
+                                               workspace.data_ptr() if workspace is not None else None, *tail))
+        elif fp8:
             ksc, vsc = _fp8_scales(k, v, k_scale, v_scale, B, H)
             _lib.check(lib.spa_ring_fwd_fp8kv(q.data_ptr(), k.data_ptr(), v.data_ptr(), ksc.data_ptr(), vsc.data_ptr(),
                                               out.data_ptr(), lse.data_ptr(),

@@ -244,3 +244,23 @@ def test_e4m3_q_k_v_public_layout_negative_scale_and_argument_checks():
     with pytest.raises(_lib.SpaError):  # head dim 64: no 8-bit score variant
         ops.flash_fwd(q64.to(DEV), k8[..., :64].contiguous().to(DEV), v8[..., :64].contiguous().to(DEV), None, True, q_scale=qsc,
                       k_scale=ksc, v_scale=vsc)
+
+
+@pytest.mark.parametrize("B,H,P,s,causal", [(1, 2, 4, 128, True), (2, 3, 3, 100, True), (1, 2, 2, 260, False), (1, 32, 8, 256, True)])
+def test_ring_forward_with_e4m3_q_k_v(B, H, P, s, causal):
+    """spa_ring_fwd_fp8qkv in its three schedules (slots and the merging epilogue included) against the oracle's full
+    attention on the dequantised tensors."""
+    D, S = 128, P * s
+    q8, qsc, q_deq = quantised((B, S, H, D), 540, "bshd", spread=1.2)
+    k8, ksc, k_deq = quantised((B, S, H, D), 541, "bshd", spread=1.5)
+    v8, vsc, v_deq = quantised((B, S, H, D), 542, "bshd", spread=0.7)
+    want_out, want_lse = O.full_attention(q_deq, k_deq, v_deq, None, causal)
+    for fuse in ("step", "rank", "all"):
+        for dtype in (torch.bfloat16, torch.float16):
+            out, lse = ops.ring_fwd(q8.to(DEV), k8.to(DEV), v8.to(DEV), P, None, causal, fuse=fuse, q_scale=qsc, k_scale=ksc, v_scale=vsc,
+                                    out_dtype=dtype)
+            assert out.dtype == dtype
+            check_out(out, want_out, dtype, f"{fuse} {dtype}")
+            check_lse(lse, want_lse)
+    with pytest.raises(_lib.SpaError):
+        ops.ring_fwd(q8.to(DEV), k8.to(DEV), v8.to(DEV), P, None, True, q_scale=qsc, k_scale=ksc, v_scale=vsc, sharding="zigzag")
