@@ -214,3 +214,36 @@ def test_varlen_backward_leaves_zeros_in_rows_of_no_sequence():
     dq, dk, dv = ops.flash_bwd_varlen_out(q, k, v, dout, lse, delta, cu, cu, 40, 40, None, True)
     for g in (dq, dk, dv):
         assert not g[used:].any() and g[:used].float().abs().max() > 0
+
+
+@pytest.mark.parametrize("P,local_lengths,H,D,dtype,causal", [
+    (2, [64, 128, 32], 2, 64, torch.bfloat16, True),
+    (4, [32, 96, 64, 48], 8, 64, torch.float16, True),     # the distributed test's batch, every sequence cut in four
+    (3, [50, 7, 130], 2, 128, torch.bfloat16, True),
+    (2, [100, 40], 2, 64, torch.float32, True),
+    (3, [20, 64], 1, 128, torch.bfloat16, False),
+])
+def test_ring_over_a_packed_batch_matches_per_sequence_attention(P, local_lengths, H, D, dtype, causal):
+    """sp_aurora_varlen_func(ring_size=P): rank r holds slice r of every sequence.  Expected: the oracle's attention of
+    every WHOLE sequence (P times the local length) alone, re-sliced into the ranks' shards; forward, lse, gradients."""
+    T = sum(local_lengths)
+    glob_q, glob_k, glob_v, glob_do = [], [], [], []
+    want_o, want_l, want_g = [], [], []
+    for i, l in enumerate(local_lengths):
+        q, k, v, do = (rand((1, P * l, H, D), 460 + 10 * i + j, dtype) for j in range(4))
+        o, ls = O.full_attention(q, k, v, None, causal)
+        g = O.attn_backward_autograd(q, k, v, do, None, causal)
+        glob_q.append(q[0]); glob_k.append(k[0]); glob_v.append(v[0]); glob_do.append(do[0])
+        want_o.append(o[0]); want_l.append(ls[0]); want_g.append([x[0] for x in g])
+    # shard r = slice r of every sequence, packed in sequence order; the shards stacked
+    stack = lambda seqs: torch.cat([torch.cat([s_[r * l:(r + 1) * l] for s_, l in zip(seqs, local_lengths)], 0) for r in range(P)], 0)
+    stack_l = lambda seqs: torch.cat([torch.cat([s_[:, r * l:(r + 1) * l] for s_, l in zip(seqs, local_lengths)], 1) for r in range(P)], 1)
+    xs = [stack(t).to(DEV).requires_grad_(True) for t in (glob_q, glob_k, glob_v)]
+    cu = cu_of(local_lengths).to(DEV)
+    out, lse, _ = spa.sp_aurora_varlen_func(*xs, cu, cu, max_seqlen=max(local_lengths), causal=causal, return_attn_probs=True, ring_size=P)
+    assert out.shape == (P * T, H, D) and lse.shape == (H, P * T)
+    check_out(out, stack(want_o), dtype)
+    check_lse(lse, stack_l(want_l))
+    out.backward(stack(glob_do).to(DEV))
+    for x, j, name in zip(xs, range(3), "qkv"):
+        check_grad(x.grad, stack([g[j] for g in want_g]), dtype, "d" + name)
