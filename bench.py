@@ -14,6 +14,9 @@ The sweep runs through the C entry point spa_ring_fwd in three schedules, same (
   rank  one launch per rank: what one GPU of a ring runs when its KV chunks are resident.
   step  one launch per (rank, ring step), the running (out, lse) in HBM, the update_out_and_lse
         merge in the kernel's epilogue: what a rank runs while chunks arrive over the wire.
+  rank_flags  (other_schedules, ring_step.flag_driven_tflops) the `rank` launches with a bounded wait for a
+        per-chunk arrival flag before a chunk's first tile is loaded (spa_ring_fwd_flags): the other way to run while
+        chunks arrive - one launch per rank, accumulators in registers across ring steps.
 `other_schedules` holds rank and step; `ring_step` repeats the step figure as the per-ring-step
 number; `roofline` carries both again as `rank_tflops` / `step_tflops`.  The line is kept below
 7.5 KB (long texts live in this docstring and in ROW_NOTES, not in the line), with `rows` ahead of
@@ -370,8 +373,8 @@ def make_row(name, ms_per_step, value, **extra):
     cfg = {"workload": workload}
     cfg.update({k2: round(v2, 2) for k2, v2 in extra.items()})
     return {"row": name, "value": round(value, 2), "unit": unit, "ms_per_step": round(ms_per_step, 4), "config": cfg,
-            "roofline": {"bound": bound, "kernel": kernel, "achieved": round(value, 2), "peak": peak, "unit": unit,
-                         "frac": round(value / peak, 4), "traffic": None}}
+            "roofline": {"bound": bound, "achieved": round(value, 2), "peak": peak, "unit": unit,
+                         "frac": round(value / peak, 4), "traffic": None}}  # (the kernel's name stays in ROW_SPECS: the line is short of room)
 
 
 def tfl(flops, m):
@@ -729,6 +732,8 @@ def assemble_line(steps, warmup, head, m_head, other, rows, cpu_head, host, traf
         line["ring_step"] = {"what": "one launch per (rank, ring step), merge in the last step's epilogue",
                              "tflops": other["step"]["tflops"], "pct_of_bf16_mfma_peak": other["step"]["pct_of_bf16_mfma_peak"],
                              "avg_launch_us": other["step"]["avg_launch_us"]}
+        if "rank_flags" in other:
+            line["ring_step"]["flag_driven_tflops"] = other["rank_flags"]["tflops"]
     line["protocol"] = {k2: m_head[k2] for k2 in ("settle_launches", "settle_ms", "settle_ended_by", "cold_ms_per_step", "timed_blocks",
                                                   "block_ms_min", "block_ms_max", "timed_region_s") if k2 in m_head}
     return line
@@ -795,6 +800,18 @@ def main():
             other[name] = {"ms_per_step": round(t, 4), "tflops": round(total_flops / (t * 1e-3) / 1e12, 2),
                            "pct_of_bf16_mfma_peak": round(100.0 * total_flops / (t * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 2),
                            "launches_per_step": launches, "avg_launch_us": round(t * 1e3 / launches, 2)}
+
+        # the schedule for chunks that arrive while a rank's one launch runs: the `rank` launches with a bounded wait for
+        # each chunk's arrival flag (all raised beforehand here: everything is resident on one GPU)
+        flags = ops.RingFlags(P, dev)
+        flags.set_all()
+        out_f = torch.empty_like(q)
+        lse_f = torch.empty((B, H, S), dtype=torch.float32, device=dev)
+        f_flags = lambda: ops.ring_fwd_flags(q, k, v, P, flags, scale, True, out=out_f, lse=lse_f)
+        mm = measure(torch, f_flags, args.steps, args.warmup, min_s=0.1, do_settle=False)
+        t = mm["ms_per_step"]
+        other["rank_flags"] = {"ms_per_step": round(t, 4), "tflops": round(total_flops / (t * 1e-3) / 1e12, 2), "launches_per_step": P,
+                               "faulted": flags.failed()}
 
     if args.traffic_leg:
         src = torch.empty(COPY_BYTES, dtype=torch.uint8, device=dev)

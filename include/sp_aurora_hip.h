@@ -210,6 +210,30 @@ int spa_ring_fwd_fp8qkv(const void* q8, const void* k8, const void* v8,
                         float scale, int mask_mode, int dtype, int fuse, void* stream);
 
 /*
+ * One launch per rank for a ring whose KV chunks ARRIVE while the launch runs (a receive buffer filled by a
+ * communication stream): spa_ring_fwd(fuse = SPA_RING_PER_RANK) whose workgroups, before they request the first tile
+ * of chunk c, wait until arrive[c] >= epoch.  The wait is an acquire load at system scope in a bounded spin: after
+ * spin_limit polls (about 0.3 us each) a wave gives up, stores 1 to *fault and goes on with whatever the buffer holds,
+ * so the grid always drains; the caller checks *fault after synchronising (and clears it before).  The query tile and
+ * the accumulators stay in registers across ring steps, i.e. the per-step loop of intel_ring_flash_attn_forward
+ * (sp_aurora/intel_ring_flash_attn.py:72-134: compute step t while chunk t+1 is in flight, :96-134) at the speed of
+ * the one-launch form, without a launch, a Q re-read and an (out, lse) round trip per step.  The producer raises a
+ * flag AFTER the chunk's bytes are visible device-wide: spa_ring_flag_set on the stream that moved the chunk, or a
+ * release store at system scope from a kernel.  Epochs let a flag array be reused without clearing (use a larger
+ * epoch per call); the rank's own chunk has a flag like the others.  bf16 / fp16, D in {64, 128}, contiguous chunks;
+ * rank >= 0 or -1 (every rank, one launch each).  arrive: uint32[P], fault: uint32[1], device memory.
+ * The reference has no counterpart (its steps are separate kernel launches around blocking waits).
+ */
+int spa_ring_fwd_flags(const void* q, const void* k, const void* v, void* out, float* lse,
+                       const uint32_t* arrive, uint32_t epoch, uint32_t spin_limit, uint32_t* fault,
+                       int B, int H, int S, int D, int P, int rank,
+                       const int64_t q_strides[3], const int64_t k_strides[3],
+                       const int64_t v_strides[3], const int64_t o_strides[3],
+                       float scale, int mask_mode, int dtype, void* stream);
+/* arrive[chunk] = epoch, ordered after everything enqueued before it on `stream` (a stream memory operation: no kernel). */
+int spa_ring_flag_set(uint32_t* arrive, int chunk, uint32_t epoch, void* stream);
+
+/*
  * spa_ring_fwd for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc): the same call without the workspace
  * argument.  The scratch is a fixed buffer of SPA_STATIC_SCRATCH_BYTES inside the library's

@@ -98,8 +98,10 @@ __device__ __forceinline__ int v_swizzle(int row) {
 // instruction (v_mfma_f32_32x32x64_f8f6f4, twice the rate of the 16-bit one; products of two e4m3 values are exact
 // in fp32): K tiles stay bytes in LDS (direct loads again, half the size), Q fragments are 32 bytes per lane and
 // 64-deep step; V is widened to T as with KV8 and P V stays a 16-bit contraction.
+// WAIT: the variant for a ring rank whose chunks arrive while its launch runs (FwdParams::arrive): a bounded wait for
+// a chunk's flag before the chunk's first tile is loaded.
 template <typename T, int D, int NG, bool SHARE, bool KV8 = false, bool FINALN = false, bool ZZ = false, bool BIG = false,
-          bool QK8 = false>
+          bool QK8 = false, bool WAIT = false>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams pk) {
   static_assert(!(FINALN && SHARE), "the merging epilogue goes with 128-row workgroups");
   static_assert(!QK8 || (KV8 && D == 128 && !ZZ && !BIG), "8-bit scores: e4m3 q, k, v, head dim 128, contiguous chunks");
@@ -143,6 +145,16 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // Ranks heaviest first: the last rank with contiguous chunks.  With zigzag shards the second half of a shard's
   // rows is heavier the lower the rank and the first half the higher, and every grid plane z holds the same work.
   const int rank = zz && zhalf ? p.rank0 + (int)blockIdx.z : p.rank0 + p.nranks - 1 - (int)blockIdx.z;
+  // WAIT: the flag of the first chunk is requested before anything else (such a load takes microseconds; it is looked
+  // at when the first tiles are about to be requested)
+  auto flag_of = [&](int ch) { return __hip_atomic_load(p.arrive + ch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM); };
+  int ahead_ch = -1;   // the chunk whose flag was fetched ahead of time, and what it read
+  unsigned ahead = 0;
+  if constexpr (WAIT) {
+    ahead_ch = rank - p.t_begin;
+    ahead_ch = ahead_ch < 0 ? ahead_ch + p.P : ahead_ch;
+    ahead = flag_of(ahead_ch);
+  }
   if (p.cu_q) {
     const int q_lo = p.cu_q[b], k_lo = p.cu_k[b];
     p.Sq = p.cu_q[b + 1] - q_lo;
@@ -276,6 +288,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     int krow;   // the same as a row of the K/V tensors
     int kend;   // one past the chunk's last row
     int klen;   // keys of the chunk this step may use (half a chunk in some steps of a zigzag ring)
+    int ch;     // the chunk's number (read by the WAIT variants only)
     bool masked;
   };
   // The loop walks the sub-tiles in order with three cursors (softmax at i, V loads at i+1,
@@ -298,6 +311,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     ch = ch < 0 ? ch + p.P : ch;
     ch = ch < 0 ? 0 : ch;  // only past the end of the schedule, where nothing is used
     c.sb.masked = c.i < n_diag;
+    c.sb.ch = ch;
     c.sb.klen = c.i >= n_diag && c.t <= zz_last_half ? klen_h : p.Sk;
     c.sb.krel = (c.j * KSTEP + (SHARE ? 0 : grp)) * BN;
     c.sb.krow = ch * p.Sk + c.sb.krel;
@@ -347,7 +361,24 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   // KV8: a thread's 8 e4m3 bytes per slot wait in registers from the MFMA phase that loads them to
   // the next VALU phase, which widens them and writes the 16-byte LDS slot (store_staged).
   u32x2 stage[KV8 ? NLOADS : 1];
-  auto load_one = [&](int q, bool kon, int k_row, unsigned kb, bool von, int v_row, unsigned vb) {
+  // (k_end / v_end: one past the chunk's last row; the WAIT variants give lanes beyond it the offset of a load that
+  // is not wanted, so that no byte of a chunk whose flag has not been seen is requested - a row past the end of a
+  // chunk is the next chunk's first - and no cache can hold a line of the receive buffer from before its arrival)
+  auto load_one = [&](int q, bool kon, int k_row, unsigned kb, bool von, int v_row, unsigned vb, int k_end = 0x7fffffff,
+                      int v_end = 0x7fffffff) {
+    if constexpr (WAIT) {
+      if (q < NK) {
+        unsigned u = kon ? (unsigned)(k_row + q * RPD_K) * krow_b : OFF_NONE;
+        if (k_row + q * RPD_K + drow >= k_end) u = OFF_NONE;
+        load_to_lds_b128(krsrc, kdoff + u, lds_wave + kb + q * (C::DTHREADS * 16));
+      } else {
+        const int r = q - NK;
+        unsigned u = von ? (unsigned)(v_row + r * C::RPD) * vrow_b : OFF_NONE;
+        if (v_row + r * C::RPD + drow >= v_end) u = OFF_NONE;
+        load_to_lds_b128(vrsrc, vdoff + u, lds_wave + vb + r * (C::DTHREADS * 16));
+      }
+      return;
+    }
     if (q < NK) {
       if constexpr (BIG) {
         // the sub-tile's first row as a 64-bit byte offset -> window descriptor + offset inside it
@@ -646,6 +677,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     int ch = rank - cs.t;
     ch = ch < 0 ? ch + p.P : ch;
     cs.sb.masked = n_diag > 0;
+    cs.sb.ch = ch;
     cs.sb.klen = n_diag == 0 && cs.t <= zz_last_half ? klen_h : p.Sk;
     cs.sb.krel = (SHARE ? 0 : grp) * BN;
     cs.sb.krow = ch * p.Sk + cs.sb.krel;
@@ -655,10 +687,36 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   cursor_next(cv);
   ck = cv;
   cursor_next(ck);
+  // WAIT: no tile of a chunk is requested before the chunk's arrival flag has been seen (each wave polls for itself;
+  // the acquire at system scope also drops cache lines that could hold the buffer's earlier contents).
+  // The flag is read with a relaxed load at system scope (it bypasses the caches; nothing is invalidated: K/V lines can
+  // not be stale, see load_one).  Such a load takes microseconds, so the flag of the chunk that follows in ring order
+  // is fetched when a chunk is entered and looked at a chunk later; only a flag that was not up yet is polled.
+  auto wait_chunk = [&](int ch) {
+    if constexpr (WAIT) {
+      unsigned seen = ch == ahead_ch ? ahead : flag_of(ch);
+      unsigned spins = 0;
+      while (__builtin_amdgcn_readfirstlane(seen) < p.epoch) {
+        if (++spins >= p.spin_limit) {  // the bound every wave reaches: note the failure and go on
+          if (lane == 0) __hip_atomic_store(p.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(8);
+        seen = flag_of(ch);
+      }
+      ahead_ch = ch > 0 ? ch - 1 : p.P - 1;
+      ahead = flag_of(ahead_ch);
+    }
+  };
+  if constexpr (WAIT) {
+    if (0 < n) wait_chunk(cs.sb.ch);
+    if (1 < n && cv.sb.ch != cs.sb.ch) wait_chunk(cv.sb.ch);
+    if (2 < n && ck.sb.ch != cv.sb.ch) wait_chunk(ck.sb.ch);
+  }
 #pragma unroll
-  for (int q = 0; q < NK; ++q) load_one(q, 0 < n, cs.sb.krow, k_lds(0), false, 0, 0);                 // K(0)
+  for (int q = 0; q < NK; ++q) load_one(q, 0 < n, cs.sb.krow, k_lds(0), false, 0, 0, cs.sb.kend, 0);     // K(0)
 #pragma unroll
-  for (int q = 0; q < C::NDMA; ++q) load_one(NK + q, false, 0, 0, 0 < n, cs.sb.krow, v_lds(0));        // V(0)
+  for (int q = 0; q < C::NDMA; ++q) load_one(NK + q, false, 0, 0, 0 < n, cs.sb.krow, v_lds(0), 0, cs.sb.kend);  // V(0)
   if constexpr (KSTAGE) {
     // K(0) goes to LDS now; V(0) stays staged together with K(1), loaded next, and both are written
     // by the first VALU phase like every later pair
@@ -667,7 +725,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       *(__attribute__((address_space(3))) u32x4*)(lds_u8*)(uintptr_t)(lds_group + (unsigned)tg * 16 + k_lds(0) + q * (C::DTHREADS * 16)) = widen(stage[q]);
   }
 #pragma unroll
-  for (int q = 0; q < NK; ++q) load_one(q, 1 < n, cv.sb.krow, k_lds(1), false, 0, 0);                 // K(1)
+  for (int q = 0; q < NK; ++q) load_one(q, 1 < n, cv.sb.krow, k_lds(1), false, 0, 0, cv.sb.kend, 0);     // K(1)
   // S(0) needs Q and K(0) only: loads complete in the order of issue, so at most the loads of V(0)
   // and K(1) may still be in flight here; they are waited for before the barrier that
   // opens the first MFMA phase reading them.
@@ -704,7 +762,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     constexpr unsigned kb = (unsigned)(PAR * C::TILEB), vb = (unsigned)(2 * C::TILEB + (PAR ^ 1) * C::TILEB);  // k_lds(i), v_lds(i + 1)
     if (early) {
 #pragma unroll
-      for (int q = 0; q < NLOADS; ++q) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb);
+      for (int q = 0; q < NLOADS; ++q) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb, ck.sb.kend, cv.sb.kend);
     }
     softmax_phase(cs.sb, pf);
     unsigned va[D / 32], ka[NKA];
@@ -719,13 +777,18 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       loads_landed();
       store_staged((unsigned)((PAR ^ 1) * C::TILEB), (unsigned)(2 * C::TILEB + PAR * C::TILEB));  // K(i + 1), V(i)
     }
+    if constexpr (WAIT) {
+      // the MFMA phase below requests K of sub-tile i + 2 (V of the same sub-tile follows one step later): its chunk's
+      // first tile?  (Here, where every load has landed anyway: looking at the flag fetched ahead waits for no other load.)
+      if (kon && ck.j == 0) wait_chunk(ck.sb.ch);
+    }
     if (!SHARE || !early) __syncthreads();
     __builtin_amdgcn_s_setprio(3);
     mfma_phase(std::true_type{}, std::true_type{}, va, ka, pf, [&](int j) {
       constexpr int TOTAL = (D / 32) * (BN / 16) + NKA * NT;
 #pragma unroll
       for (int q = 0; q < NLOADS; ++q)
-        if ((q * TOTAL + TOTAL / 2) / NLOADS == j && !early) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb);
+        if ((q * TOTAL + TOTAL / 2) / NLOADS == j && !early) load_one(q, kon, ck.sb.krow, kb, von, cv.sb.krow, vb, ck.sb.kend, cv.sb.kend);
     });
     __builtin_amdgcn_s_setprio(0);
     cursor_next(cs);
@@ -1323,6 +1386,15 @@ hipError_t launch16_qk8(FwdParams p, hipStream_t stream) {
   return launch<flash_fwd16_kernel<T, D, 1, false, true, false, false, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
 }
 
+// One launch for a rank whose chunks arrive while it runs: 128-row workgroups, one or two wave groups.
+template <typename T, int D>
+hipError_t launch16_wait(const FwdParams& p, hipStream_t stream) {
+  const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
+  const bool two = force ? force == 2 : p.Sk > fwd_bn<D>();
+  if (two) return launch<flash_fwd16_kernel<T, D, 2, false, false, false, false, false, false, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+  return launch<flash_fwd16_kernel<T, D, 1, false, false, false, false, false, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+}
+
 // (dtype, D) -> kernel family; the zigzag variants are instantiated beside the plain ones
 template <bool ZZ>
 hipError_t launch16_any(const FwdParams& p, int D, int dtype, hipStream_t stream) {
@@ -1352,7 +1424,7 @@ hipError_t launch16_any(const FwdParams& p, int D, int dtype, hipStream_t stream
 }  // namespace
 
 // This file makes three objects: compiled with SPA_FWD_ZIGZAG_UNIT it holds the zigzag variants of the 16-bit
-// kernel and nothing else, with SPA_FWD_BIG_UNIT the re-based variants and those with 8-bit scores, without either
+// kernel and nothing else, with SPA_FWD_BIG_UNIT the re-based variants, those with 8-bit scores and those that wait for chunk arrival flags, without either
 // everything else (so that the parts compile side by side).
 #if defined(SPA_FWD_ZIGZAG_UNIT)
 hipError_t spa_launch_fwd16_zigzag(const FwdParams& p, int D, int dtype, hipStream_t stream) {
@@ -1363,6 +1435,17 @@ hipError_t spa_launch_fwd16_qk8(const FwdParams& p, int D, int dtype, hipStream_
   if (D != 128 || !p.q_scale || !p.k_scale || !p.v_scale || p.zigzag || p.big || p.cu_q) return hipErrorInvalidValue;
   if (dtype == 1) return launch16_qk8<__bf16>(p, stream);
   if (dtype == 2) return launch16_qk8<_Float16>(p, stream);
+  return hipErrorInvalidValue;
+}
+hipError_t spa_launch_fwd16_wait(const FwdParams& p, int D, int dtype, hipStream_t stream) {
+  if (!p.arrive || !p.fault || p.k_scale || p.zigzag || p.big || p.epi != SPA_EPI_PLAIN || p.cu_q) return hipErrorInvalidValue;
+  if (dtype == 1) {
+    if (D == 128) return launch16_wait<__bf16, 128>(p, stream);
+    if (D == 64) return launch16_wait<__bf16, 64>(p, stream);
+  } else if (dtype == 2) {
+    if (D == 128) return launch16_wait<_Float16, 128>(p, stream);
+    if (D == 64) return launch16_wait<_Float16, 64>(p, stream);
+  }
   return hipErrorInvalidValue;
 }
 hipError_t spa_launch_fwd16_big(const FwdParams& p, int D, int dtype, hipStream_t stream) {
@@ -1382,6 +1465,7 @@ hipError_t spa_launch_fwd16_big(const FwdParams& p, int D, int dtype, hipStream_
 hipError_t spa_launch_fwd16_zigzag(const FwdParams& p, int D, int dtype, hipStream_t stream);
 hipError_t spa_launch_fwd16_big(const FwdParams& p, int D, int dtype, hipStream_t stream);
 hipError_t spa_launch_fwd16_qk8(const FwdParams& p, int D, int dtype, hipStream_t stream);
+hipError_t spa_launch_fwd16_wait(const FwdParams& p, int D, int dtype, hipStream_t stream);
 
 // Returns hipSuccess, or hipErrorInvalidValue for an unsupported (dtype, D).
 hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream) {
@@ -1399,6 +1483,7 @@ hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t strea
     p.out = (char*)slots.out<char>(p.part, p.part_slot) - row0 * p.os.s * 2;
     p.lse = slots.lse(p.part, p.P, p.part_slot) - row0;
   }
+  if ((dtype == 1 || dtype == 2) && p.arrive) return spa_launch_fwd16_wait(p, D, dtype, stream);
   if ((dtype == 1 || dtype == 2) && p.q_scale) return spa_launch_fwd16_qk8(p, D, dtype, stream);
   if (dtype == 1 || dtype == 2)
     return p.big ? spa_launch_fwd16_big(p, D, dtype, stream)

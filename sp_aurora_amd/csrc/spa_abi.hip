@@ -273,12 +273,19 @@ int static_scratch(void** ptr) {
 
 // `what` names the entry point in messages; `ws_bytes` < 0: the caller vouches for the workspace size.
 // k_scale / v_scale non-null: K and V are e4m3 bytes with one scale per (batch, head) for the whole sequence.
+// What the flag variant adds to a ring call: null `arrive` = none.
+struct RingFlags {
+  const unsigned* arrive = nullptr;
+  unsigned epoch = 0, spin_limit = 0;
+  unsigned* fault = nullptr;
+};
+
 // q_scale non-null (with the other two): q is e4m3 as well and the scores run on the 8-bit matrix instruction (D = 128).
 int ring_fwd(const char* what, const void* q, const void* k, const void* v, const float* q_scale, const float* k_scale,
              const float* v_scale, void* out, float* lse, void* workspace,
              int64_t ws_bytes, int B, int H, int S, int D, int P, int rank, const int64_t q_strides[3],
              const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3], float scale,
-             int mask_mode, int dtype, int fuse, void* stream) {
+             int mask_mode, int dtype, int fuse, void* stream, const RingFlags flags = RingFlags()) {
   if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "%s: null pointer", what);
   if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(SPA_EINVAL, "%s: null strides", what);
   if (!dims_ok(B, H, S, D)) return fail(SPA_EINVAL, "%s: sizes must be positive", what);
@@ -356,6 +363,11 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   p.zigzag = zig && dtype != SPA_F32;
   p.zz_half = 0;
   p.big = big && dtype != SPA_F32;
+  if (flags.arrive) {
+    if (fuse != SPA_RING_PER_RANK || dtype == SPA_F32 || kv8 || zig || big || D == 32)
+      return fail(SPA_EUNSUPPORTED, "%s: built for one launch per rank, bf16 / fp16, head dim 64 or 128, contiguous chunks below 2 GiB", what);
+    p.arrive = flags.arrive; p.epoch = flags.epoch; p.spin_limit = flags.spin_limit; p.fault = flags.fault;
+  }
 
   if (fuse == SPA_RING_ALL_RANKS) {  // one launch: every requested rank, every step
     p.rank0 = r_lo; p.nranks = r_hi - r_lo; p.t_begin = 0; p.t_count = -1;
@@ -460,6 +472,26 @@ int spa_ring_fwd_fp8kv(const void* q, const void* k8, const void* v8, const floa
   if (!k_scale || !v_scale) return fail(SPA_EINVAL, "spa_ring_fwd_fp8kv: null scale pointer");
   return ring_fwd("spa_ring_fwd_fp8kv", q, k8, v8, nullptr, k_scale, v_scale, out, lse, workspace, -1, B, H, S, D, P, rank, q_strides,
                   k_strides, v_strides, o_strides, scale, mask_mode, dtype, fuse, stream);
+}
+
+int spa_ring_fwd_flags(const void* q, const void* k, const void* v, void* out, float* lse, const uint32_t* arrive,
+                       uint32_t epoch, uint32_t spin_limit, uint32_t* fault, int B, int H, int S, int D, int P, int rank,
+                       const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                       const int64_t o_strides[3], float scale, int mask_mode, int dtype, void* stream) {
+  if (!arrive || !fault) return fail(SPA_EINVAL, "spa_ring_fwd_flags: null flag pointer");
+  if ((((uintptr_t)arrive | (uintptr_t)fault) & 3) != 0) return fail(SPA_EALIGN, "spa_ring_fwd_flags: flags must be 4-byte aligned");
+  if (spin_limit == 0) return fail(SPA_EINVAL, "spa_ring_fwd_flags: spin_limit must be positive");
+  RingFlags f;
+  f.arrive = arrive; f.epoch = epoch; f.spin_limit = spin_limit; f.fault = fault;
+  return ring_fwd("spa_ring_fwd_flags", q, k, v, nullptr, nullptr, nullptr, out, lse, nullptr, -1, B, H, S, D, P, rank, q_strides,
+                  k_strides, v_strides, o_strides, scale, mask_mode, dtype, SPA_RING_PER_RANK, stream, f);
+}
+
+int spa_ring_flag_set(uint32_t* arrive, int chunk, uint32_t epoch, void* stream) {
+  if (!arrive || chunk < 0) return fail(SPA_EINVAL, "spa_ring_flag_set: null pointer or negative chunk");
+  const hipError_t e = hipStreamWriteValue32((hipStream_t)stream, arrive + chunk, epoch, 0);
+  if (e != hipSuccess) return fail(SPA_ELAUNCH, "spa_ring_flag_set: %s", hipGetErrorString(e));
+  return SPA_OK;
 }
 
 int spa_ring_fwd_fp8qkv(const void* q8, const void* k8, const void* v8, const float* q_scale, const float* k_scale,

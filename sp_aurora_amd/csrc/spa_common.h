@@ -61,6 +61,13 @@ struct FwdParams {
   // the second half only (a step with c > r that is not the rank's last).
   int zigzag = 0;
   int zz_half = 0;
+  // Chunk arrival flags (the variants for a ring rank whose K/V chunks land while its one launch runs): before a
+  // workgroup loads the first tile of chunk c it waits until arrive[c] >= epoch (an acquire load at system scope in
+  // a bounded spin: after spin_limit polls the wave gives up, sets *fault = 1 and goes on, so the grid always drains).
+  const unsigned* arrive = nullptr;
+  unsigned epoch = 0;
+  unsigned spin_limit = 0;
+  unsigned* fault = nullptr;
   // K / V rows of one (batch, head) span 2 GiB or more: the launcher takes the kernel variants that re-base their
   // buffer descriptors per tile (16-bit kernels; the fp32 kernels address with 64-bit pointers anyway)
   int big = 0;

@@ -297,6 +297,64 @@ def ring_fwd(q, k, v, ring_size, softmax_scale=None, causal=False, rank=-1, layo
     return out, lse
 
 
+class RingFlags:
+    """Arrival flags of a ring's KV chunks for ring_fwd_flags: uint32 flag per chunk and a fault word, on the device.
+    `epoch` is what a flag must reach; next_epoch() starts a new round without clearing the array."""
+
+    def __init__(self, ring_size, device):
+        self.arrive = torch.zeros((int(ring_size),), dtype=torch.int32, device=device)
+        self.fault = torch.zeros((1,), dtype=torch.int32, device=device)
+        self.epoch = 1
+
+    def next_epoch(self):
+        self.epoch += 1
+        return self.epoch
+
+    def set(self, chunk, stream=None):
+        """arrive[chunk] = epoch after everything enqueued so far on `stream` (default: the current one)."""
+        st = _stream() if stream is None else stream.cuda_stream
+        _lib.check(_lib.load().spa_ring_flag_set(self.arrive.data_ptr(), int(chunk), self.epoch, st))
+
+    def set_all(self, stream=None):
+        for c in range(self.arrive.numel()):
+            self.set(c, stream)
+
+    def failed(self):
+        """True when some wave gave up waiting (reads the fault word: synchronises)."""
+        return bool(self.fault.item())
+
+
+def ring_fwd_flags(q, k, v, ring_size, flags, softmax_scale=None, causal=False, rank=-1, layout="bshd", out=None, lse=None,
+                   spin_limit=1 << 20):
+    """ring_fwd(fuse="rank") for chunks that arrive while the launch runs: a workgroup waits for flags.arrive[c] >=
+    flags.epoch (bounded by spin_limit polls) before it touches chunk c.  Calls spa_ring_fwd_flags."""
+    lib = _lib.load()
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise TypeError("q, k, v must share a dtype")
+    (B, H, S, D), qs = _bhs(q, layout)
+    shp_k, ks = _bhs(k, layout)
+    shp_v, vs = _bhs(v, layout)
+    if shp_k != (B, H, S, D) or shp_v != (B, H, S, D):
+        raise ValueError(f"ring attention needs q, k, v of one shape, got {tuple(q.shape)} {tuple(k.shape)} {tuple(v.shape)}")
+    if flags.arrive.numel() != int(ring_size) or flags.arrive.device != q.device:
+        raise ValueError("flags must hold one entry per chunk on q's device")
+    if softmax_scale is None:
+        softmax_scale = D ** (-0.5)
+    if out is None:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    if lse is None:
+        lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
+    _, os_ = _bhs(out, layout)
+    with _on(q.device):
+        _lib.check(lib.spa_ring_fwd_flags(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), flags.arrive.data_ptr(), flags.epoch,
+            int(spin_limit), flags.fault.data_ptr(), B, H, S, D, int(ring_size), int(rank), _lib.strides3(qs), _lib.strides3(ks),
+            _lib.strides3(vs), _lib.strides3(os_), float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE,
+            _dtype_code(q), _stream()))
+    return out, lse
+
+
 def merge(out_acc, lse_acc, blk_out, blk_lse, layout="bshd", init=False):
     """In-place merge of (blk_out, blk_lse) into fp32 (out_acc, lse_acc).  Calls spa_merge."""
     lib = _lib.load()

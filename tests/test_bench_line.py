@@ -16,6 +16,7 @@ def _fake_line():
               "cold_ms_per_step": 0.9312, "timed_blocks": 200, "block_ms_min": 0.4801, "block_ms_max": 0.4999, "timed_region_s": 0.213}
     other = {name: {"ms_per_step": 0.8123, "tflops": 1234.56, "pct_of_bf16_mfma_peak": 49.38, "launches_per_step": 36, "avg_launch_us": 22.56}
              for name in ("rank", "step")}
+    other["rank_flags"] = {"ms_per_step": 0.5612, "tflops": 1234.56, "launches_per_step": 8, "faulted": False}
     cpu = {"value": 0.3513, "unit": "TFLOP/s", "cores": 128, "kind": "port",
            "sample": "backward pairs [1,2048,16,128]: 1 d 1289 ms + 1 f 1250 ms measured, x 16 d + 120 f = 1134.6 s"}
     rows = {}
@@ -48,6 +49,7 @@ def test_schedule_figures_come_last_and_rows_are_complete():
         assert k in line, k
     assert line["roofline"]["rank_tflops"] == 1234.56 and line["roofline"]["step_tflops"] == 1234.56
     assert line["protocol"]["settle_ended_by"] in ("converged", "cap")
+    assert line["ring_step"]["flag_driven_tflops"] == 1234.56
 
 
 def test_more_than_one_gpu_is_refused():

@@ -1,0 +1,82 @@
+"""One launch per rank for a ring whose KV chunks arrive while the launch runs (spa_ring_fwd_flags): with the flags
+raised beforehand the result is that of the plain one-launch form, bit for bit; with a second stream filling the
+receive buffer and raising the flags while the kernel runs it is still that result; with flags that never come every
+wave gives up at its spin limit, the launch ends and the fault word says so."""
+import time
+
+import pytest
+import torch
+
+from conftest import rand_qkv
+from oracle import attn_oracle as O
+from sp_aurora_amd import ops
+from test_gpu_parity import DEV, check_lse, check_out
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("B,H,P,s,D,dtype,causal", [
+    (1, 4, 4, 256, 128, torch.bfloat16, True),
+    (2, 2, 3, 100, 64, torch.float16, True),
+    (1, 2, 4, 64, 128, torch.bfloat16, False),     # one wave group per workgroup
+    (1, 32, 8, 1024, 128, torch.bfloat16, True),   # benchmark config 3
+])
+def test_flags_raised_beforehand_give_the_one_launch_result(B, H, P, s, D, dtype, causal):
+    q, k, v = (t.to(DEV) for t in rand_qkv((B, P * s, H, D), 800, dtype, 0.5))
+    want_o, want_l = ops.ring_fwd(q, k, v, P, None, causal, fuse="rank")
+    flags = ops.RingFlags(P, q.device)
+    flags.set_all()
+    out, lse = ops.ring_fwd_flags(q, k, v, P, flags, None, causal)
+    torch.cuda.synchronize()
+    assert not flags.failed()
+    assert torch.equal(out, want_o) and torch.equal(lse, want_l)
+    # a new round on the same flag array: nothing raised yet for the new epoch, a tiny spin limit -> every wave gives up
+    flags.next_epoch()
+    ops.ring_fwd_flags(q, k, v, P, flags, None, causal, spin_limit=4)
+    torch.cuda.synchronize()
+    assert flags.failed()
+
+
+def test_chunks_that_arrive_while_the_launch_runs():
+    """Rank P-1 of a causal ring: its own chunk is there, the others are copied into a poisoned receive buffer by a second
+    stream, each followed by its flag, while the rank's launch is already running and waiting."""
+    B, H, P, s, D, dtype = 1, 8, 4, 512, 128, torch.bfloat16
+    r = P - 1
+    q, k, v = (t.to(DEV) for t in rand_qkv((B, P * s, H, D), 801, dtype, 0.5))
+    (qc, kc, vc) = (t.cpu() for t in (q, k, v))
+    want_o, want_l = O.full_attention(qc, kc, vc, None, True)
+    rows = slice(r * s, (r + 1) * s)
+    kbuf, vbuf = torch.full_like(k, float("nan")), torch.full_like(v, float("nan"))
+    kbuf[:, rows], vbuf[:, rows] = k[:, rows], v[:, rows]
+    flags = ops.RingFlags(P, q.device)
+    out = torch.zeros_like(q)
+    lse = torch.zeros((B, H, P * s), dtype=torch.float32, device=DEV)
+    torch.cuda.synchronize()
+    comm = torch.cuda.Stream()
+    flags.set(r)                                     # the rank's own chunk
+    ops.ring_fwd_flags(q, kbuf, vbuf, P, flags, None, True, rank=r, out=out, lse=lse, spin_limit=1 << 21)
+    with torch.cuda.stream(comm):
+        for c in range(r - 1, -1, -1):               # ring order: chunk r-1 lands first
+            time.sleep(0.002)
+            cs = slice(c * s, (c + 1) * s)
+            kbuf[:, cs].copy_(k[:, cs])
+            vbuf[:, cs].copy_(v[:, cs])
+            flags.set(c, stream=comm)
+    torch.cuda.synchronize()
+    assert not flags.failed(), "a wave gave up waiting for a chunk"
+    check_out(out[:, rows], want_o[:, rows], dtype)
+    check_lse(lse[:, :, rows], want_l[:, :, rows])
+    assert not out[:, :r * s].any()
+
+
+def test_flag_entry_refuses_what_it_is_not_built_for():
+    from sp_aurora_amd import _lib
+    q, k, v = (t.to(DEV) for t in rand_qkv((1, 256, 2, 32), 802, torch.bfloat16))
+    flags = ops.RingFlags(2, q.device)
+    with pytest.raises(_lib.SpaError):   # head dim 32
+        ops.ring_fwd_flags(q, k, v, 2, flags, None, True)
+    q, k, v = (t.to(DEV) for t in rand_qkv((1, 256, 2, 64), 803, torch.float32))
+    with pytest.raises(_lib.SpaError):   # fp32
+        ops.ring_fwd_flags(q, k, v, 2, flags, None, True)
+    with pytest.raises(ValueError):      # one flag per chunk
+        ops.ring_fwd_flags(q.bfloat16(), k.bfloat16(), v.bfloat16(), 4, flags, None, True)
