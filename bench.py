@@ -48,6 +48,8 @@ Two helper modes for the HBM traffic figure (roofline.traffic):
                          both the attention kernel and a calibration kernel
   --pmc-summary F W      reads the two counter_collection.csv files of such runs and writes
                          profiles/flash_fwd_traffic.json (no GPU needed)
+  --pmc-summary-rows F W the same for the re-layout and merge kernels, from two runs of
+                         `--workload hbm --traffic-leg`: writes profiles/hbm_rows_traffic.json
 `--transient` prints, instead of the benchmark, the per-launch durations of the first 120 launches
 after 3 s of idle together with the clock and board power read from sysfs (what the settle phase
 is for).
@@ -74,6 +76,7 @@ SEED = 2
 INPUT_SCALE = 0.5
 COPY_BYTES = 1 << 30  # calibration copy of the traffic leg: reads and writes this many bytes
 TRAFFIC_JSON = os.path.join(ROOT, "profiles", "flash_fwd_traffic.json")
+ROWS_TRAFFIC_JSON = os.path.join(ROOT, "profiles", "hbm_rows_traffic.json")  # the same for the HBM-bound rows
 MIN_TIMED_S = 0.2
 MAX_BLOCKS = 200
 
@@ -374,7 +377,22 @@ def make_row(name, ms_per_step, value, **extra):
     cfg.update({k2: round(v2, 2) for k2, v2 in extra.items()})
     return {"row": name, "value": round(value, 2), "unit": unit, "ms_per_step": round(ms_per_step, 4), "config": cfg,
             "roofline": {"bound": bound, "achieved": round(value, 2), "peak": peak, "unit": unit,
-                         "frac": round(value / peak, 4), "traffic": None}}  # (the kernel's name stays in ROW_SPECS: the line is short of room)
+                         "frac": round(value / peak, 4), "traffic": row_traffic(name)}}  # (the kernel's name stays in ROW_SPECS: the line is short of room)
+
+
+_ROW_TRAFFIC = None
+
+
+def row_traffic(name):
+    """HBM bytes per launch of a row's kernel as recorded by --pmc-summary-rows, or None."""
+    global _ROW_TRAFFIC
+    if _ROW_TRAFFIC is None:
+        try:
+            _ROW_TRAFFIC = json.load(open(ROWS_TRAFFIC_JSON))
+        except (OSError, ValueError):
+            _ROW_TRAFFIC = {}
+    t = _ROW_TRAFFIC.get(name, {}).get("hbm_bytes_per_launch")
+    return round(t) if t else None
 
 
 def tfl(flops, m):
@@ -629,6 +647,15 @@ def transient(torch, spa, idle_s=3.0, launches=120):
 
 
 # ------------------------------------------------------------------------------------ traffic helper
+def calibration_copy(torch, dev):
+    """A plain device copy of COPY_BYTES: what FETCH_SIZE / WRITE_SIZE read for it scales the kernels' readings."""
+    src = torch.empty(COPY_BYTES, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
 def pmc_summary(fetch_dir, write_dir):
     """FETCH_SIZE / WRITE_SIZE (KiB per dispatch) of the attention kernel, each scaled by what the
     same counter reads for the calibration copy of COPY_BYTES."""
@@ -676,9 +703,48 @@ def pmc_summary(fetch_dir, write_dir):
     print(json.dumps(res, indent=1))
 
 
+def pmc_summary_rows(fetch_dir, write_dir):
+    """The same for the kernels of the HBM-bound rows (two runs of `--workload hbm --traffic-leg`): FETCH_SIZE and
+    WRITE_SIZE per dispatch, each scaled by the calibration copy of the same run."""
+    kernels = {"config4_relayout_s2h": ("relayout_kernel<16, true>", 268435456),
+               "config4_relayout_h2s": ("relayout_kernel<16, false>", 268435456),
+               "merge_update_out_and_lse": ("merge_kernelIDF16bLb0E", 42336256)}  # (the profiler leaves bf16 names mangled)
+
+    def read(d, counter):
+        files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
+        if not files:
+            raise SystemExit(f"no counter_collection.csv under {d}")
+        per, copy = {n: [] for n in kernels}, []
+        for f in files:
+            for row in csv.DictReader(open(f)):
+                if row.get("Counter_Name") != counter:
+                    continue
+                name, val = row["Kernel_Name"], float(row["Counter_Value"])
+                for n, (pat, _) in kernels.items():
+                    if pat in name:
+                        per[n].append(val)
+                if "copybuffer" in name.lower():
+                    copy.append(val)
+        if not copy or not all(per.values()):
+            raise SystemExit(f"{counter}: a kernel or the calibration copy is missing in {d}")
+        return per, max(copy)
+
+    f_per, f_copy = read(fetch_dir, "FETCH_SIZE")
+    w_per, w_copy = read(write_dir, "WRITE_SIZE")
+    f_factor, w_factor = (COPY_BYTES / 1024.0) / f_copy, (COPY_BYTES / 1024.0) / w_copy
+    res = {"copy_bytes": COPY_BYTES, "copy_fetch_size_kib": f_copy, "copy_write_size_kib": w_copy, "fetch_factor": f_factor, "write_factor": w_factor}
+    for n, (_, alg) in kernels.items():
+        fa, wa = statistics.median(f_per[n]), statistics.median(w_per[n])
+        res[n] = {"dispatches": len(f_per[n]), "fetch_size_kib_per_dispatch": fa, "write_size_kib_per_dispatch": wa,
+                  "hbm_fetch_bytes_per_launch": fa * f_factor * 1024.0, "hbm_write_bytes_per_launch": wa * w_factor * 1024.0,
+                  "hbm_bytes_per_launch": (fa * f_factor + wa * w_factor) * 1024.0, "algorithmic_bytes_per_launch": alg}
+    json.dump(res, open(ROWS_TRAFFIC_JSON, "w"), indent=1)
+    print(json.dumps(res, indent=1))
+
+
 # ------------------------------------------------------------------------------------ main
 ROW_SETS = {"fp8kv": {"fp8kv"}, "relayout": {"config4"}, "ulysses": {"config4"}, "merge": {"merge"}, "backward": {"config5"},
-            "config1": {"config1"}, "config2": {"config2"}, "zigzag": {"zigzag"}}
+            "config1": {"config1"}, "config2": {"config2"}, "zigzag": {"zigzag"}, "hbm": {"config4", "merge"}}
 ALL_ROWS = {"config1", "config2", "zigzag", "config4", "fp8kv", "merge", "config5"}
 LINE_LIMIT = 7500  # bytes of the printed line: readers that keep only the end of the output keep 8 KB
 
@@ -751,12 +817,17 @@ def main():
                     help="which schedule --only-all runs (profiling runs); `value` is always the `all` schedule otherwise")
     ap.add_argument("--traffic-leg", action="store_true", help="also run the calibration copy (for --pmc runs)")
     ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"))
+    ap.add_argument("--pmc-summary-rows", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="the same for the re-layout and merge kernels (runs of --workload hbm --traffic-leg): writes profiles/hbm_rows_traffic.json")
     ap.add_argument("--transient", action="store_true",
                     help="instead of the benchmark: per-launch durations of the first 120 launches after 3 s of idle, with clock / power samples")
     ap.add_argument("--workload", default="config3", choices=["config3"] + sorted(ROW_SETS))
     args = ap.parse_args()
     if args.pmc_summary:
         pmc_summary(*args.pmc_summary)
+        return
+    if args.pmc_summary_rows:
+        pmc_summary_rows(*args.pmc_summary_rows)
         return
     if args.gpus != 1:
         print("bench.py: this build measures one GPU (the ring is simulated on it, no collectives); --gpus must be 1", file=sys.stderr)
@@ -777,6 +848,8 @@ def main():
         return
     if args.workload != "config3":
         rows = gpu_rows(torch, spa, ops, ROW_SETS[args.workload], args.steps, args.warmup)
+        if args.traffic_leg:
+            calibration_copy(torch, dev)
         if not args.no_cpu_baseline:
             attach_cpu(rows, CpuLegs(torch))
         print(json.dumps({"rows": list(rows.values())}))
@@ -814,11 +887,7 @@ def main():
                                "faulted": flags.failed()}
 
     if args.traffic_leg:
-        src = torch.empty(COPY_BYTES, dtype=torch.uint8, device=dev)
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(torch, dev)
 
     traffic = traffic_src = None
     if os.path.exists(TRAFFIC_JSON):
