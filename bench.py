@@ -319,7 +319,7 @@ class CpuLegs:
 # ------------------------------------------------------------------------------------ rows
 # What each row of `rows` runs (the line itself carries a short `workload` only).
 ROW_NOTES = {
-    "config1_fp32_block_forward": "config 1: fp32 B=1 S=512 H=8 D=64 non-causal block forward, out + lse (flash_fwd32_kernel<64>)",
+    "config1_fp32_block_forward": "config 1: fp32 B=1 S=512 H=8 D=64 non-causal block forward, out + lse (flash_fwd32_splitk_kernel<64,8>)",
     "config2_ring_rank2_of_4": "config 2: bf16 B=2 S=4096 (P=4 chunks of 1024) H=32 D=64 causal, rank 2: diagonal chunk 2, then chunks 1, 0, "
                                "merged; value = one launch for the rank, step_tflops = one launch per ring step (3 launches)",
     "config3_zigzag_ring": "config 3 tensors with zigzag sharding (rank r holds half-chunks r and 15-r): every rank runs 1 diagonal "
@@ -348,7 +348,7 @@ ROW_NOTES = {
 
 # name -> (short workload text, unit, roofline bound, kernel, peak, extra config keys)
 ROW_SPECS = {
-    "config1_fp32_block_forward": ("config 1: fp32 [1,512,8,64] block forward", "TFLOP/s", "mfma", "flash_fwd32<64>", MFMA_F32_PEAK_TFLOPS, ()),
+    "config1_fp32_block_forward": ("config 1: fp32 [1,512,8,64] block forward", "TFLOP/s", "mfma", "flash_fwd32_splitk<64,8>", MFMA_F32_PEAK_TFLOPS, ()),
     "config2_ring_rank2_of_4": ("config 2: bf16 D=64, rank 2 of P=4, 1 launch", "TFLOP/s", "mfma", "flash_fwd16<bf16,64>", MFMA_BF16_PEAK_TFLOPS,
                                 ("step_tflops",)),
     "config3_zigzag_ring": ("config 3, zigzag shards, 1 launch per rank", "TFLOP/s", "mfma", "flash_fwd16<bf16,128>", MFMA_BF16_PEAK_TFLOPS,

@@ -416,8 +416,10 @@ int spa_flash_bwd_varlen_out(const void* q, const void* k, const void* v, const 
  *                                  2 = 256-row workgroups sharing one set of buffers
  *   SPA_TUNE_BWD_DQ_WAVES  4 | 8   waves per workgroup of the backward's dq kernel
  *   SPA_TUNE_BWD_DKDV_FORM 1       compiler-scheduled MFMAs in the D = 128 dk/dv kernel
+ *   SPA_TUNE_FWD32_SPLIT  1 | 2    never / whenever D <= 64: the fp32 forward with 32-row workgroups whose waves share
+ *                                  the key tiles (the library takes it when 128-row workgroups would leave half the CUs idle)
  */
-enum { SPA_TUNE_FWD_GROUPS = 0, SPA_TUNE_FWD_SHARE = 1, SPA_TUNE_BWD_DQ_WAVES = 2, SPA_TUNE_BWD_DKDV_FORM = 3 };
+enum { SPA_TUNE_FWD_GROUPS = 0, SPA_TUNE_FWD_SHARE = 1, SPA_TUNE_BWD_DQ_WAVES = 2, SPA_TUNE_BWD_DKDV_FORM = 3, SPA_TUNE_FWD32_SPLIT = 4 };
 int spa_tune(int knob, int value);
 
 #ifdef __cplusplus

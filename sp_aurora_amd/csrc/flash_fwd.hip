@@ -1287,6 +1287,187 @@ __global__ void __launch_bounds__(FWD_THREADS, 1) flash_fwd32_kernel(const FwdPa
   }
 }
 
+
+// ---------------------------------------------------------------------------------
+// fp32, few query rows: a launch of the kernel above with fewer workgroups than CUs lasts as long as one wave's
+// chain of fp32 MFMAs over all key tiles (64 MFMAs of 64 cycles per 32 keys).  Here a workgroup owns 32 query rows
+// and its NW waves take every NW-th key tile, each through an LDS tile pair of its own (no workgroup barrier in the
+// loop); the waves' (O, m, l) are combined through LDS at the end.  Same arithmetic per tile as above.
+// ---------------------------------------------------------------------------------
+template <int D, int NW>
+struct Fwd32SplitCfg {
+  static constexpr int PITCH = D + 4;
+  static constexpr int TILE = F32_BN * PITCH;          // floats per K or V tile
+  static constexpr int WAVE = 2 * TILE;                // one wave's K and V tile
+  static constexpr int SMEM = NW * WAVE * 4;           // the combine reuses it: NW x (32 x D + 64) floats fit
+  static constexpr int CPR = D / 4;                    // 16-byte chunks per row
+  static constexpr int RPP = 64 / CPR;                 // rows a wave fetches per pass
+  static constexpr int PASS = F32_BN / RPP;
+  static_assert(D <= 64, "built for head dims whose tile pair fits a wave's registers");
+};
+
+template <int D, int NW>
+__global__ void __launch_bounds__(64 * NW, 1) flash_fwd32_splitk_kernel(const FwdParams p) {
+  typedef Fwd32SplitCfg<D, NW> C;
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* const sm = (float*)smem;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ln = lane & 31;
+  const int hh = lane >> 5;
+  const int h = blockIdx.x % p.H;
+  const int b = blockIdx.x / p.H;
+  const int qt = p.nqt - 1 - (int)blockIdx.y;
+  const int q0 = qt * 32;
+  const float* qp = (const float*)p.q + b * p.qs.b + h * p.qs.h;
+  const float* kp = (const float*)p.k + b * p.ks.b + h * p.ks.h;
+  const float* vp = (const float*)p.v + b * p.vs.b + h * p.vs.h;
+  const int qrow = q0 + ln;
+  const int qrow_c = qrow < p.Sq ? qrow : p.Sq - 1;
+  f32x4 qf[D / 8];
+#pragma unroll
+  for (int g = 0; g < D / 8; ++g) {
+    qf[g] = *(const f32x4*)(qp + (int64_t)qrow_c * p.qs.s + 8 * g + 4 * hh);
+    if (p.negq) qf[g] = -qf[g];
+  }
+  const int kv_end = p.causal ? (q0 + 32 < p.Sk ? q0 + 32 : p.Sk) : p.Sk;
+  const int nt = (kv_end + F32_BN - 1) / F32_BN;
+  float* const kb = sm + w * C::WAVE;  // this wave's tiles
+  float* const vb = kb + C::TILE;
+  const int cc = lane % C::CPR, cr = lane / C::CPR;
+  f32x4 kreg[C::PASS], vreg[C::PASS];
+  auto gload = [&](int it) {
+    const int key0 = it * F32_BN;
+#pragma unroll
+    for (int i = 0; i < C::PASS; ++i) {
+      int r = key0 + cr + i * C::RPP;
+      r = r < p.Sk ? r : p.Sk - 1;
+      kreg[i] = *(const f32x4*)(kp + (int64_t)r * p.ks.s + cc * 4);
+      vreg[i] = *(const f32x4*)(vp + (int64_t)r * p.vs.s + cc * 4);
+    }
+  };
+  auto lstore = [&]() {
+#pragma unroll
+    for (int i = 0; i < C::PASS; ++i) {
+      const int lr = cr + i * C::RPP;
+      *(f32x4*)(kb + lr * C::PITCH + cc * 4) = kreg[i];
+      *(f32x4*)(vb + lr * C::PITCH + cc * 4) = vreg[i];
+    }
+  };
+  f32x16 o[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[i][v] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const float c = p.scale_log2;
+  if (w < nt) gload(w);
+  for (int it = w; it < nt; it += NW) {
+    const int key0 = it * F32_BN;
+    // the tile is this wave's alone: its own LDS reads of the tile before are done (in order), and a wave's LDS
+    // writes are visible to its own later reads
+    lstore();
+    if (it + NW < nt) gload(it + NW);
+    f32x16 s;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+    for (int g = 0; g < D / 8; ++g) {
+      const f32x4 a = *(const f32x4*)(kb + ln * C::PITCH + 8 * g + 4 * hh);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], qf[g][e], s, 0, 0, 0);
+    }
+    const bool need_mask = (p.causal && key0 + F32_BN - 1 > q0) || (key0 + F32_BN > p.Sk);
+    if (need_mask) {
+      const int lim = p.causal ? (qrow < p.Sk - 1 ? qrow : p.Sk - 1) : p.Sk - 1;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = key0 + 8 * (v >> 2) + 4 * hh + (v & 3);
+        if (key > lim) s[v] = -INFINITY;
+      }
+    }
+    float mx = s[0];
+#pragma unroll
+    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
+    mx = halves_max(mx);
+    const float m_new = fmaxf(m_run, mx);
+    // (a row past the last key of a causal tile that starts beyond it has seen nothing yet: -inf - -inf)
+    const float alpha = m_new == -INFINITY ? 1.f : fast_exp2((m_run - m_new) * c);
+    const float mc = m_new == -INFINITY ? 0.f : m_new * c;
+    m_run = m_new;
+    float ps = 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float e = fast_exp2(__builtin_fmaf(s[v], c, -mc));
+      s[v] = e;
+      ps += e;
+    }
+    l_run = l_run * alpha + ps;
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o[i][v] *= alpha;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int kl = 8 * (v >> 2) + 4 * hh + (v & 3);
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db) {
+        const float a = vb[kl * C::PITCH + db * 32 + ln];
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s[v], o[db], 0, 0, 0);
+      }
+    }
+  }
+  // ---- combine: every wave leaves its unscaled O (lane-private order) and (m, l); wave j then finishes the
+  // 16-byte pieces j, j + NW, ... of every row ----
+  constexpr int NPC = D / 8;           // 16-byte pieces per lane: (db, g)
+  constexpr int REC = 64 * NPC * 4;    // floats of one wave's O
+  const float l_own = halves_sum(l_run);
+  __syncthreads();                     // every wave is done with its tiles
+  float* const orec = sm + w * (REC + 128);
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      f32x4 st;
+      st[0] = o[db][4 * g + 0]; st[1] = o[db][4 * g + 1]; st[2] = o[db][4 * g + 2]; st[3] = o[db][4 * g + 3];
+      *(f32x4*)(orec + ((db * 4 + g) * 64 + lane) * 4) = st;
+    }
+  if (hh == 0) {
+    orec[REC + ln] = m_run;
+    orec[REC + 32 + ln] = l_own;
+  }
+  __syncthreads();
+  float mw[NW], m_all = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < NW; ++j) {
+    mw[j] = sm[j * (REC + 128) + REC + ln];
+    m_all = fmaxf(m_all, mw[j]);
+  }
+  float aw[NW], l_all = 0.f;
+#pragma unroll
+  for (int j = 0; j < NW; ++j) {
+    aw[j] = mw[j] == -INFINITY ? 0.f : fast_exp2((mw[j] - m_all) * c);  // a wave without a visible key
+    l_all += aw[j] * sm[j * (REC + 128) + REC + 32 + ln];
+  }
+  const float inv = 1.f / l_all;
+  if (qrow < p.Sq) {
+    float* const op = (float*)p.out + b * p.os.b + h * p.os.h + (int64_t)qrow * p.os.s;
+    for (int pc = w; pc < NPC; pc += NW) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < NW; ++j) {
+        const f32x4 x = *(const f32x4*)(sm + j * (REC + 128) + (pc * 64 + lane) * 4);
+        acc[0] += aw[j] * x[0]; acc[1] += aw[j] * x[1]; acc[2] += aw[j] * x[2]; acc[3] += aw[j] * x[3];
+      }
+      acc[0] *= inv; acc[1] *= inv; acc[2] *= inv; acc[3] *= inv;
+      const int db = pc / 4, g = pc % 4;
+      *(f32x4*)(op + db * 32 + 8 * g + 4 * hh) = acc;
+    }
+    if (w == 0 && hh == 0) p.lse[((int64_t)b * p.H + h) * p.lse_bh + qrow] = (m_all * c + fast_log2(l_all)) * 0.6931471805599453f;
+  }
+}
+
 template <auto kernel>
 hipError_t launch(int threads, int smem, const FwdParams& p, hipStream_t stream) {
   const hipError_t e = spa_allow_dynamic_lds<kernel>(smem);
@@ -1490,6 +1671,16 @@ hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t strea
                  : p.zigzag ? spa_launch_fwd16_zigzag(p, D, dtype, stream) : launch16_any<false>(p, D, dtype, stream);
   if (dtype == 0) {
     if (p.epi != SPA_EPI_PLAIN) return hipErrorInvalidValue;  // fp32 ring steps merge with the separate kernel
+    // Few 128-row workgroups (fewer than half the CUs), a head dim whose tile pair fits a wave's registers: 32-row
+    // workgroups whose 8 waves share the key tiles.  spa_tune("fwd32_split"): 1 never, 2 whenever D <= 64.
+    const int knob = spa_knob(SPA_KNOB_FWD32_SPLIT);
+    const bool few = 2 * (int64_t)p.B * p.H * p.nqt <= spa_device_cus() && p.Sk > 4 * F32_BN;
+    if (D <= 64 && !p.cu_q && p.nranks == 1 && p.P == 1 && knob != 1 && (few || knob == 2)) {
+      FwdParams ps = p;
+      ps.nqt = (p.Sq + 31) / 32;
+      if (D == 64) return launch<flash_fwd32_splitk_kernel<64, 8>>(512, Fwd32SplitCfg<64, 8>::SMEM, ps, stream);
+      return launch<flash_fwd32_splitk_kernel<32, 8>>(512, Fwd32SplitCfg<32, 8>::SMEM, ps, stream);
+    }
     if (D == 128) return launch<flash_fwd32_kernel<128>>(FWD_THREADS, Fwd32Cfg<128>::SMEM, p, stream);
     if (D == 64) return launch<flash_fwd32_kernel<64>>(FWD_THREADS, Fwd32Cfg<64>::SMEM, p, stream);
     if (D == 32) return launch<flash_fwd32_kernel<32>>(FWD_THREADS, Fwd32Cfg<32>::SMEM, p, stream);
