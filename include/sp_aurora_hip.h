@@ -212,9 +212,12 @@ int spa_ring_fwd_fp8qkv(const void* q8, const void* k8, const void* v8,
 /*
  * One launch per rank for a ring whose KV chunks ARRIVE while the launch runs (a receive buffer filled by a
  * communication stream): spa_ring_fwd(fuse = SPA_RING_PER_RANK) whose workgroups, before they request the first tile
- * of chunk c, wait until arrive[c] >= epoch.  The wait is an acquire load at system scope in a bounded spin: after
- * spin_limit polls (about 0.3 us each) a wave gives up, stores 1 to *fault and goes on with whatever the buffer holds,
- * so the grid always drains; the caller checks *fault after synchronising (and clears it before).  The query tile and
+ * of chunk c, wait until arrive[c] >= epoch.  The flag is read past the caches (a relaxed load at system scope) in a
+ * bounded spin: after spin_limit polls (about 1 us each) a wave gives up, stores 1 to *fault and goes on with whatever
+ * the buffer holds, so the grid always drains; the caller checks *fault after synchronising (and clears it before).
+ * The kernel requests no byte of a chunk before it has seen the chunk's flag, so no cache can hold the buffer's earlier
+ * contents; for that to hold per cache line, every K / V chunk of every (batch, head) must start on a 128-byte boundary
+ * (SPA_EALIGN otherwise).  The query tile and
  * the accumulators stay in registers across ring steps, i.e. the per-step loop of intel_ring_flash_attn_forward
  * (sp_aurora/intel_ring_flash_attn.py:72-134: compute step t while chunk t+1 is in flight, :96-134) at the speed of
  * the one-launch form, without a launch, a Q re-read and an (out, lse) round trip per step.  The producer raises a

@@ -367,15 +367,21 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   auto load_one = [&](int q, bool kon, int k_row, unsigned kb, bool von, int v_row, unsigned vb, int k_end = 0x7fffffff,
                       int v_end = 0x7fffffff) {
     if constexpr (WAIT) {
+      // the descriptor's range ends with the chunk (a scalar per load instead of a compare per lane): what lies past
+      // it arrives as zeros like everything past the tensor
       if (q < NK) {
-        unsigned u = kon ? (unsigned)(k_row + q * RPD_K) * krow_b : OFF_NONE;
-        if (k_row + q * RPD_K + drow >= k_end) u = OFF_NONE;
-        load_to_lds_b128(krsrc, kdoff + u, lds_wave + kb + q * (C::DTHREADS * 16));
+        const unsigned u = kon ? (unsigned)(k_row + q * RPD_K) * krow_b : OFF_NONE;
+        u32x4 rs = krsrc;
+        const unsigned lim = (unsigned)k_end * krow_b;
+        rs[2] = lim < krsrc[2] ? lim : krsrc[2];
+        load_to_lds_b128(rs, kdoff + u, lds_wave + kb + q * (C::DTHREADS * 16));
       } else {
         const int r = q - NK;
-        unsigned u = von ? (unsigned)(v_row + r * C::RPD) * vrow_b : OFF_NONE;
-        if (v_row + r * C::RPD + drow >= v_end) u = OFF_NONE;
-        load_to_lds_b128(vrsrc, vdoff + u, lds_wave + vb + r * (C::DTHREADS * 16));
+        const unsigned u = von ? (unsigned)(v_row + r * C::RPD) * vrow_b : OFF_NONE;
+        u32x4 rs = vrsrc;
+        const unsigned lim = (unsigned)v_end * vrow_b;
+        rs[2] = lim < vrsrc[2] ? lim : vrsrc[2];
+        load_to_lds_b128(rs, vdoff + u, lds_wave + vb + r * (C::DTHREADS * 16));
       }
       return;
     }

@@ -481,6 +481,17 @@ int spa_ring_fwd_flags(const void* q, const void* k, const void* v, void* out, f
   if (!arrive || !fault) return fail(SPA_EINVAL, "spa_ring_fwd_flags: null flag pointer");
   if ((((uintptr_t)arrive | (uintptr_t)fault) & 3) != 0) return fail(SPA_EALIGN, "spa_ring_fwd_flags: flags must be 4-byte aligned");
   if (spin_limit == 0) return fail(SPA_EINVAL, "spa_ring_fwd_flags: spin_limit must be positive");
+  // No cache line may hold bytes of two chunks: a line fetched with one chunk would keep the other's bytes from before
+  // their arrival.  Every chunk of every (batch, head) must therefore start on a 128-byte boundary.
+  if (k && v && k_strides && v_strides && P > 0 && S > 0 && S % P == 0 && (dtype == SPA_BF16 || dtype == SPA_F16)) {
+    const int64_t chunk = S / P;
+    auto lines_ok = [&](const void* base, const int64_t st[3]) {
+      return ((uintptr_t)base & 127) == 0 && (P == 1 || (chunk * st[2] * 2) % 128 == 0) && (B == 1 || (st[0] * 2) % 128 == 0) &&
+             (H == 1 || (st[1] * 2) % 128 == 0);
+    };
+    if (!lines_ok(k, k_strides) || !lines_ok(v, v_strides))
+      return fail(SPA_EALIGN, "spa_ring_fwd_flags: every K / V chunk of every (batch, head) must start on a 128-byte boundary");
+  }
   RingFlags f;
   f.arrive = arrive; f.epoch = epoch; f.spin_limit = spin_limit; f.fault = fault;
   return ring_fwd("spa_ring_fwd_flags", q, k, v, nullptr, nullptr, nullptr, out, lse, nullptr, -1, B, H, S, D, P, rank, q_strides,

@@ -78,5 +78,10 @@ def test_flag_entry_refuses_what_it_is_not_built_for():
     q, k, v = (t.to(DEV) for t in rand_qkv((1, 256, 2, 64), 803, torch.float32))
     with pytest.raises(_lib.SpaError):   # fp32
         ops.ring_fwd_flags(q, k, v, 2, flags, None, True)
+    qb, kb, vb = (t.bfloat16() for t in (q, k, v))
+    pad = torch.zeros(kb.numel() + 64, dtype=torch.bfloat16, device=DEV)
+    k_off = pad[32:32 + kb.numel()].view_as(kb).copy_(kb)      # 64 bytes off a line boundary
+    with pytest.raises(_lib.SpaError):   # a cache line would hold bytes of two chunks
+        ops.ring_fwd_flags(qb, k_off, vb, 2, flags, None, True)
     with pytest.raises(ValueError):      # one flag per chunk
         ops.ring_fwd_flags(q.bfloat16(), k.bfloat16(), v.bfloat16(), 4, flags, None, True)
