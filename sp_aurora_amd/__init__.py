@@ -62,7 +62,8 @@ from .ulysses import (  # noqa: F401
     ulysses_flash_attn_qkvpacked_func,
 )
 from .utils import flatten_varlen_lse, unflatten_varlen_lse, update_out_and_lse  # noqa: F401
-from .varlen import VarlenFlashAttnFunc, ring_flash_attn_varlen_func, sp_aurora_varlen_func  # noqa: F401
+from .varlen import (VarlenFlashAttnFunc, ring_flash_attn_varlen_func, sp_aurora_varlen_func,  # noqa: F401
+                     zigzag_sp_aurora_varlen_func, zigzag_varlen_order)
 
 SeqAllToAll4D_v2 = SeqAllToAll4D  # sp_aurora/__init__.py:77
 

@@ -247,3 +247,48 @@ def test_ring_over_a_packed_batch_matches_per_sequence_attention(P, local_length
     out.backward(stack(glob_do).to(DEV))
     for x, j, name in zip(xs, range(3), "qkv"):
         check_grad(x.grad, stack([g[j] for g in want_g]), dtype, "d" + name)
+
+
+@pytest.mark.parametrize("P,local_lengths,H,D,dtype", [
+    (2, [64, 128], 2, 64, torch.bfloat16),
+    (4, [32, 0, 96, 2], 2, 128, torch.float16),     # an empty sequence and one with a single row per half
+    (3, [100, 36], 3, 32, torch.float32),
+    (2, [130, 62, 8], 1, 64, torch.bfloat16),
+])
+def test_zigzag_ring_over_a_packed_batch(P, local_lengths, H, D, dtype):
+    """zigzag_sp_aurora_varlen_func(ring_size=P): rank r holds half-slices r and 2P-1-r of every sequence.  Expected: the
+    oracle's causal attention of every whole sequence alone, brought into the shards' order; forward, lse, gradients."""
+    T = sum(local_lengths)
+    seq_lens = [P * l for l in local_lengths]
+    parts = {name: [] for name in ("q", "k", "v", "do", "o", "l", "dq", "dk", "dv")}
+    for i, n in enumerate(seq_lens):
+        q, k, v, do = (rand((1, n, H, D), 560 + 10 * i + j, dtype) for j in range(4))
+        if n:
+            o, ls = O.full_attention(q, k, v, None, True)
+            g = O.attn_backward_autograd(q, k, v, do, None, True)
+        else:
+            o, ls, g = q.float(), torch.zeros((1, H, 0)), (q.float(), k.float(), v.float())
+        for name, t in zip(("q", "k", "v", "do", "o", "dq", "dk", "dv"), (q, k, v, do, o, *g)):
+            parts[name].append(t[0])
+        parts["l"].append(ls[0])
+    idx = spa.zigzag_varlen_order(seq_lens, P)
+    nat = {name: torch.cat(ts, 1 if name == "l" else 0) for name, ts in parts.items()}
+    xs = [nat[name][idx].to(DEV).requires_grad_(True) for name in "qkv"]
+    cu = cu_of(local_lengths).to(DEV)
+    out, lse, _ = spa.zigzag_sp_aurora_varlen_func(*xs, cu, cu, max_seqlen=max(local_lengths), causal=True, return_attn_probs=True,
+                                                   ring_size=P)
+    assert out.shape == (P * T, H, D) and lse.shape == (H, P * T)
+    check_out(out, nat["o"][idx], dtype)
+    check_lse(lse, nat["l"][:, idx])
+    out.backward(nat["do"][idx].to(DEV))
+    for x, name in zip(xs, "qkv"):
+        check_grad(x.grad, nat["d" + name][idx], dtype, "d" + name)
+    # without a mask the sharding does not matter: the contiguous ring's result on the same rows
+    a = spa.zigzag_sp_aurora_varlen_func(*[x.detach() for x in xs], cu, cu, max_seqlen=max(local_lengths), causal=False, ring_size=P)
+    b = spa.sp_aurora_varlen_func(*[x.detach() for x in xs], cu, cu, max_seqlen=max(local_lengths), causal=False, ring_size=P)
+    assert torch.equal(a, b)
+    # an odd share of a shard cannot be halved
+    if T:
+        bad = cu_of([T - 1, 1]).to(DEV)
+        with pytest.raises(ValueError):
+            spa.zigzag_sp_aurora_varlen_func(*[x.detach() for x in xs], bad, bad, max_seqlen=T, causal=True, ring_size=P)
