@@ -335,7 +335,8 @@ ROW_NOTES = {
                          "peak = the mix of the two rates for equal FLOPs, 2 / (1/5000 + 1/2500); kv_only_tflops = bf16 q with e4m3 K / V "
                          "(spa_flash_fwd_fp8kv, both contractions 16-bit), bf16_tflops = the same call with bf16 q, K, V; "
                          "ring_rank_tflops / ring_step_tflops = the config-3 ring sweep (P = 8) on the e4m3 tensors, one launch per rank / "
-                         "per (rank, step) (spa_ring_fwd_fp8qkv)",
+                         "per (rank, step) (spa_ring_fwd_fp8qkv); ring_flags_tflops = one launch per rank that waits for each chunk's arrival "
+                         "flag, all raised beforehand (spa_ring_fwd_flags_fp8qkv)",
     "merge_update_out_and_lse": "update_out_and_lse: merge of a bf16 block into the fp32 running (out, lse) of one config-3 rank "
                                 "[1,1024,32,128], 8 operand sets in turn, recorded calls replayed; host cost of the call included",
     "config5_ring_forward": "config 5 forward: bf16 qkv [1,32768,3,16,128] (strided views) causal, ring of 16 chunks of 2048, 16 diagonal + "
@@ -358,7 +359,7 @@ ROW_SPECS = {
     "config4_ulysses_forward": ("config 4: 3 re-layouts, attention, 1 re-layout", "TFLOP/s", "mfma", "relayout x4 + flash_fwd16<bf16,128>",
                                 MFMA_BF16_PEAK_TFLOPS, ("views_tflops",)),
     "block_forward_fp8": ("causal block forward [1,8192,32,128], e4m3 q/K/V, 8-bit scores", "TFLOP/s", "mfma", "flash_fwd16<bf16,128,e4m3 q/K/V>",
-                          MFMA_FP8_BF16_MIX_PEAK_TFLOPS, ("kv_only_tflops", "bf16_tflops", "ring_rank_tflops", "ring_step_tflops")),
+                          MFMA_FP8_BF16_MIX_PEAK_TFLOPS, ("kv_only_tflops", "bf16_tflops", "ring_rank_tflops", "ring_step_tflops", "ring_flags_tflops")),
     "merge_update_out_and_lse": ("merge of a bf16 block [1,1024,32,128] into fp32 (out, lse), 42.3 MB", "GB/s", "hbm", "merge<bf16>",
                                  HBM_PEAK_GBPS, ()),
     "config5_ring_forward": ("config 5 forward, P=16, 1 launch", "TFLOP/s", "mfma", "flash_fwd16<bf16,128>", MFMA_BF16_PEAK_TFLOPS,
@@ -510,8 +511,14 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
             fr = lambda fuse=fuse: ops.ring_fwd(q8, k8, v8, P, None, True, out=out, lse=lse, workspace=ws, fuse=fuse, q_scale=qsc,
                                                 k_scale=ksc, v_scale=vsc)
             ring8[fuse] = tfl(flops, measure(torch, fr, 20, 5, **light))
+        flags8 = ops.RingFlags(P, dev)
+        flags8.set_all()
+        ff = lambda: ops.ring_fwd_flags(q8, k8, v8, P, flags8, None, True, out=out, lse=lse, q_scale=qsc, k_scale=ksc, v_scale=vsc)
+        ring8["flags"] = tfl(flops, measure(torch, ff, 20, 5, **light))
+        if flags8.failed():
+            raise RuntimeError("bench.py: a wave of the flag-driven e4m3 ring gave up waiting with every flag raised")
         finish("block_forward_fp8", m, tf, kv_only_tflops=tfl(flops, mkv), bf16_tflops=tfl(flops, m16),
-               ring_rank_tflops=ring8["rank"], ring_step_tflops=ring8["step"])
+               ring_rank_tflops=ring8["rank"], ring_step_tflops=ring8["step"], ring_flags_tflops=ring8["flags"])
         del q, k, v, q8, k8, v8
     if "merge" in which:
         Bn, sn, Hn, Dn = 1, 1024, 32, 128

@@ -233,6 +233,13 @@ int spa_ring_fwd_flags(const void* q, const void* k, const void* v, void* out, f
                        const int64_t q_strides[3], const int64_t k_strides[3],
                        const int64_t v_strides[3], const int64_t o_strides[3],
                        float scale, int mask_mode, int dtype, void* stream);
+/* The same for e4m3 q, k, v (spa_ring_fwd_fp8qkv's tensors and scales: D = 128, scores on the 8-bit matrix instruction,
+ * out in `dtype`; strides of q, k, v in bytes). */
+int spa_ring_fwd_flags_fp8qkv(const void* q8, const void* k8, const void* v8, const float* q_scale, const float* k_scale,
+                              const float* v_scale, void* out, float* lse, const uint32_t* arrive, uint32_t epoch,
+                              uint32_t spin_limit, uint32_t* fault, int B, int H, int S, int D, int P, int rank,
+                              const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                              const int64_t o_strides[3], float scale, int mask_mode, int dtype, void* stream);
 /* arrive[chunk] = epoch, ordered after everything enqueued before it on `stream` (a stream memory operation: no kernel). */
 int spa_ring_flag_set(uint32_t* arrive, int chunk, uint32_t epoch, void* stream);
 

@@ -33,6 +33,7 @@ SIGNATURES = {
     "spa_ring_fwd_fp8kv": (_i, [_vp] * 8 + [_i] * 6 + [_s3] * 4 + [_f, _i, _i, _i, _vp]),
     "spa_ring_fwd_fp8qkv": (_i, [_vp] * 9 + [_i] * 6 + [_s3] * 4 + [_f, _i, _i, _i, _vp]),
     "spa_ring_fwd_flags": (_i, [_vp] * 6 + [ctypes.c_uint32, ctypes.c_uint32, _vp] + [_i] * 6 + [_s3] * 4 + [_f, _i, _i, _vp]),
+    "spa_ring_fwd_flags_fp8qkv": (_i, [_vp] * 9 + [ctypes.c_uint32, ctypes.c_uint32, _vp] + [_i] * 6 + [_s3] * 4 + [_f, _i, _i, _vp]),
     "spa_ring_flag_set": (_i, [_vp, _i, ctypes.c_uint32, _vp]),
     "spa_ring_fwd_workspace_bytes": (ctypes.c_int64, [_i, _i, _i, _i, _i, _i]),
     "spa_ring_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _i, _vp]),

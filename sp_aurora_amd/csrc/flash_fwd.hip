@@ -374,17 +374,29 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
       // it arrives as zeros like everything past the tensor
       if (q < NK) {
         const unsigned u = kon ? (unsigned)(k_row + q * RPD_K) * krow_b : OFF_NONE;
-        u32x4 rs = krsrc;
-        const unsigned lim = (unsigned)k_end * krow_b;
-        rs[2] = lim < krsrc[2] ? lim : krsrc[2];
-        load_to_lds_b128(rs, kdoff + u, lds_wave + kb + q * (C::DTHREADS * 16));
+        const unsigned end = (unsigned)k_end * krow_b;
+        const unsigned lim = end < krsrc[2] ? end : krsrc[2];
+        if constexpr (KSTAGE) {
+          stage[q] = __builtin_bit_cast(
+              u32x2, __builtin_amdgcn_raw_buffer_load_b64(__builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, (int)lim, 0x00020000), kdoff + u, 0, 0));
+        } else {
+          u32x4 rs = krsrc;
+          rs[2] = lim;
+          load_to_lds_b128(rs, kdoff + u, lds_wave + kb + q * (C::DTHREADS * 16));
+        }
       } else {
         const int r = q - NK;
         const unsigned u = von ? (unsigned)(v_row + r * C::RPD) * vrow_b : OFF_NONE;
-        u32x4 rs = vrsrc;
-        const unsigned lim = (unsigned)v_end * vrow_b;
-        rs[2] = lim < vrsrc[2] ? lim : vrsrc[2];
-        load_to_lds_b128(rs, vdoff + u, lds_wave + vb + r * (C::DTHREADS * 16));
+        const unsigned end = (unsigned)v_end * vrow_b;
+        const unsigned lim = end < vrsrc[2] ? end : vrsrc[2];
+        if constexpr (KV8) {
+          stage[q] = __builtin_bit_cast(
+              u32x2, __builtin_amdgcn_raw_buffer_load_b64(__builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, (int)lim, 0x00020000), vdoff + u, 0, 0));
+        } else {
+          u32x4 rs = vrsrc;
+          rs[2] = lim;
+          load_to_lds_b128(rs, vdoff + u, lds_wave + vb + r * (C::DTHREADS * 16));
+        }
       }
       return;
     }
@@ -1585,6 +1597,16 @@ hipError_t launch16_wait(const FwdParams& p, hipStream_t stream) {
   return launch<flash_fwd16_kernel<T, D, 1, false, false, false, false, false, false, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
 }
 
+// The same for e4m3 q, k, v with the scores on the 8-bit matrix instruction (D = 128).
+template <typename T>
+hipError_t launch16_wait_qk8(const FwdParams& p, hipStream_t stream) {
+  constexpr int D = 128;
+  const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
+  const bool two = force ? force == 2 : p.Sk > fwd_bn<D>();
+  if (two) return launch<flash_fwd16_kernel<T, D, 2, false, true, false, false, false, true, true>>(2 * FWD_THREADS, Fwd16Cfg<D, 2, false>::SMEM, p, stream);
+  return launch<flash_fwd16_kernel<T, D, 1, false, true, false, false, false, true, true>>(FWD_THREADS, Fwd16Cfg<D, 1, false>::SMEM, p, stream);
+}
+
 // (dtype, D) -> kernel family; the zigzag variants are instantiated beside the plain ones
 template <bool ZZ>
 hipError_t launch16_any(const FwdParams& p, int D, int dtype, hipStream_t stream) {
@@ -1628,7 +1650,13 @@ hipError_t spa_launch_fwd16_qk8(const FwdParams& p, int D, int dtype, hipStream_
   return hipErrorInvalidValue;
 }
 hipError_t spa_launch_fwd16_wait(const FwdParams& p, int D, int dtype, hipStream_t stream) {
-  if (!p.arrive || !p.fault || p.k_scale || p.zigzag || p.big || p.epi != SPA_EPI_PLAIN || p.cu_q) return hipErrorInvalidValue;
+  if (!p.arrive || !p.fault || p.zigzag || p.big || p.epi != SPA_EPI_PLAIN || p.cu_q) return hipErrorInvalidValue;
+  if (p.k_scale || p.v_scale || p.q_scale) {  // e4m3 tensors: all three, 8-bit scores
+    if (!p.k_scale || !p.v_scale || !p.q_scale || D != 128) return hipErrorInvalidValue;
+    if (dtype == 1) return launch16_wait_qk8<__bf16>(p, stream);
+    if (dtype == 2) return launch16_wait_qk8<_Float16>(p, stream);
+    return hipErrorInvalidValue;
+  }
   if (dtype == 1) {
     if (D == 128) return launch16_wait<__bf16, 128>(p, stream);
     if (D == 64) return launch16_wait<__bf16, 64>(p, stream);

@@ -271,6 +271,15 @@ int static_scratch(void** ptr) {
   return SPA_OK;
 }
 
+// The flag-driven launches: no cache line may hold bytes of two chunks (a line fetched with one chunk would keep the
+// other's bytes from before their arrival), so every chunk of every (batch, head) must start on a 128-byte boundary.
+// Strides in elements of `esz` bytes.
+bool chunk_lines_ok(const void* base, const int64_t st[3], int esz, int B, int H, int S, int P) {
+  const int64_t chunk = S / P;
+  return ((uintptr_t)base & 127) == 0 && (P == 1 || (chunk * st[2] * esz) % 128 == 0) && (B == 1 || (st[0] * esz) % 128 == 0) &&
+         (H == 1 || (st[1] * esz) % 128 == 0);
+}
+
 // `what` names the entry point in messages; `ws_bytes` < 0: the caller vouches for the workspace size.
 // k_scale / v_scale non-null: K and V are e4m3 bytes with one scale per (batch, head) for the whole sequence.
 // What the flag variant adds to a ring call: null `arrive` = none.
@@ -364,8 +373,8 @@ int ring_fwd(const char* what, const void* q, const void* k, const void* v, cons
   p.zz_half = 0;
   p.big = big && dtype != SPA_F32;
   if (flags.arrive) {
-    if (fuse != SPA_RING_PER_RANK || dtype == SPA_F32 || kv8 || zig || big || D == 32)
-      return fail(SPA_EUNSUPPORTED, "%s: built for one launch per rank, bf16 / fp16, head dim 64 or 128, contiguous chunks below 2 GiB", what);
+    if (fuse != SPA_RING_PER_RANK || dtype == SPA_F32 || (kv8 && !qk8) || zig || big || D == 32)
+      return fail(SPA_EUNSUPPORTED, "%s: built for one launch per rank, bf16 / fp16 (or e4m3 q, k, v), head dim 64 or 128, contiguous chunks below 2 GiB", what);
     p.arrive = flags.arrive; p.epoch = flags.epoch; p.spin_limit = flags.spin_limit; p.fault = flags.fault;
   }
 
@@ -481,21 +490,32 @@ int spa_ring_fwd_flags(const void* q, const void* k, const void* v, void* out, f
   if (!arrive || !fault) return fail(SPA_EINVAL, "spa_ring_fwd_flags: null flag pointer");
   if ((((uintptr_t)arrive | (uintptr_t)fault) & 3) != 0) return fail(SPA_EALIGN, "spa_ring_fwd_flags: flags must be 4-byte aligned");
   if (spin_limit == 0) return fail(SPA_EINVAL, "spa_ring_fwd_flags: spin_limit must be positive");
-  // No cache line may hold bytes of two chunks: a line fetched with one chunk would keep the other's bytes from before
-  // their arrival.  Every chunk of every (batch, head) must therefore start on a 128-byte boundary.
-  if (k && v && k_strides && v_strides && P > 0 && S > 0 && S % P == 0 && (dtype == SPA_BF16 || dtype == SPA_F16)) {
-    const int64_t chunk = S / P;
-    auto lines_ok = [&](const void* base, const int64_t st[3]) {
-      return ((uintptr_t)base & 127) == 0 && (P == 1 || (chunk * st[2] * 2) % 128 == 0) && (B == 1 || (st[0] * 2) % 128 == 0) &&
-             (H == 1 || (st[1] * 2) % 128 == 0);
-    };
-    if (!lines_ok(k, k_strides) || !lines_ok(v, v_strides))
-      return fail(SPA_EALIGN, "spa_ring_fwd_flags: every K / V chunk of every (batch, head) must start on a 128-byte boundary");
-  }
+  if (k && v && k_strides && v_strides && P > 0 && S > 0 && S % P == 0 && (dtype == SPA_BF16 || dtype == SPA_F16) &&
+      (!chunk_lines_ok(k, k_strides, 2, B, H, S, P) || !chunk_lines_ok(v, v_strides, 2, B, H, S, P)))
+    return fail(SPA_EALIGN, "spa_ring_fwd_flags: every K / V chunk of every (batch, head) must start on a 128-byte boundary");
   RingFlags f;
   f.arrive = arrive; f.epoch = epoch; f.spin_limit = spin_limit; f.fault = fault;
   return ring_fwd("spa_ring_fwd_flags", q, k, v, nullptr, nullptr, nullptr, out, lse, nullptr, -1, B, H, S, D, P, rank, q_strides,
                   k_strides, v_strides, o_strides, scale, mask_mode, dtype, SPA_RING_PER_RANK, stream, f);
+}
+
+int spa_ring_fwd_flags_fp8qkv(const void* q8, const void* k8, const void* v8, const float* q_scale, const float* k_scale,
+                              const float* v_scale, void* out, float* lse, const uint32_t* arrive, uint32_t epoch,
+                              uint32_t spin_limit, uint32_t* fault, int B, int H, int S, int D, int P, int rank,
+                              const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                              const int64_t o_strides[3], float scale, int mask_mode, int dtype, void* stream) {
+  const char* what = "spa_ring_fwd_flags_fp8qkv";
+  if (!q_scale || !k_scale || !v_scale) return fail(SPA_EINVAL, "%s: null scale pointer", what);
+  if (!arrive || !fault) return fail(SPA_EINVAL, "%s: null flag pointer", what);
+  if ((((uintptr_t)arrive | (uintptr_t)fault) & 3) != 0) return fail(SPA_EALIGN, "%s: flags must be 4-byte aligned", what);
+  if (spin_limit == 0) return fail(SPA_EINVAL, "%s: spin_limit must be positive", what);
+  if (k8 && v8 && k_strides && v_strides && P > 0 && S > 0 && S % P == 0 &&
+      (!chunk_lines_ok(k8, k_strides, 1, B, H, S, P) || !chunk_lines_ok(v8, v_strides, 1, B, H, S, P)))
+    return fail(SPA_EALIGN, "%s: every K / V chunk of every (batch, head) must start on a 128-byte boundary", what);
+  RingFlags f;
+  f.arrive = arrive; f.epoch = epoch; f.spin_limit = spin_limit; f.fault = fault;
+  return ring_fwd(what, q8, k8, v8, q_scale, k_scale, v_scale, out, lse, nullptr, -1, B, H, S, D, P, rank, q_strides, k_strides,
+                  v_strides, o_strides, scale, mask_mode, dtype, SPA_RING_PER_RANK, stream, f);
 }
 
 int spa_ring_flag_set(uint32_t* arrive, int chunk, uint32_t epoch, void* stream) {

@@ -325,13 +325,23 @@ class RingFlags:
 
 
 def ring_fwd_flags(q, k, v, ring_size, flags, softmax_scale=None, causal=False, rank=-1, layout="bshd", out=None, lse=None,
-                   spin_limit=1 << 20):
+                   spin_limit=1 << 20, q_scale=None, k_scale=None, v_scale=None, out_dtype=torch.bfloat16):
     """ring_fwd(fuse="rank") for chunks that arrive while the launch runs: a workgroup waits for flags.arrive[c] >=
-    flags.epoch (bounded by spin_limit polls) before it touches chunk c.  Calls spa_ring_fwd_flags."""
+    flags.epoch (bounded by spin_limit polls) before it touches chunk c.  Calls spa_ring_fwd_flags, or, for e4m3 q, k, v
+    with their [B,H] scales (D = 128, result in out_dtype), spa_ring_fwd_flags_fp8qkv."""
     lib = _lib.load()
-    q, k, v = _prep(q), _prep(k), _prep(v)
-    if not (q.dtype == k.dtype == v.dtype):
-        raise TypeError("q, k, v must share a dtype")
+    fp8 = q.dtype == FP8
+    if fp8:
+        if k.dtype != FP8 or v.dtype != FP8 or q_scale is None or out_dtype not in (torch.bfloat16, torch.float16):
+            raise ValueError("e4m3 q goes with e4m3 k, v, the three scales and out_dtype bfloat16 or float16")
+        if not (q.is_cuda and k.is_cuda and v.is_cuda):
+            raise ValueError("sp_aurora_amd kernels need tensors on a HIP device (got a CPU tensor)")
+        ok16 = lambda t: t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s_ % 16 == 0 for s_ in t.stride()[:-1])
+        q, k, v = (t if ok16(t) else t.contiguous() for t in (q, k, v))
+    else:
+        q, k, v = _prep(q), _prep(k), _prep(v)
+        if not (q.dtype == k.dtype == v.dtype):
+            raise TypeError("q, k, v must share a dtype")
     (B, H, S, D), qs = _bhs(q, layout)
     shp_k, ks = _bhs(k, layout)
     shp_v, vs = _bhs(v, layout)
@@ -342,16 +352,23 @@ def ring_fwd_flags(q, k, v, ring_size, flags, softmax_scale=None, causal=False, 
     if softmax_scale is None:
         softmax_scale = D ** (-0.5)
     if out is None:
-        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        out = torch.empty(q.shape, dtype=out_dtype if fp8 else q.dtype, device=q.device)
     if lse is None:
         lse = torch.empty((B, H, S), dtype=torch.float32, device=q.device)
     _, os_ = _bhs(out, layout)
+    tail = (flags.arrive.data_ptr(), flags.epoch, int(spin_limit), flags.fault.data_ptr(), B, H, S, D, int(ring_size), int(rank),
+            _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_), float(softmax_scale),
+            _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(out), _stream())
     with _on(q.device):
-        _lib.check(lib.spa_ring_fwd_flags(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), flags.arrive.data_ptr(), flags.epoch,
-            int(spin_limit), flags.fault.data_ptr(), B, H, S, D, int(ring_size), int(rank), _lib.strides3(qs), _lib.strides3(ks),
-            _lib.strides3(vs), _lib.strides3(os_), float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE,
-            _dtype_code(q), _stream()))
+        if fp8:
+            ksc, vsc = _fp8_scales(k, v, k_scale, v_scale, B, H)
+            if tuple(q_scale.shape) != (B, H):
+                raise ValueError(f"q_scale must have shape {(B, H)}, got {tuple(q_scale.shape)}")
+            qsc = q_scale.to(device=q.device, dtype=torch.float32).contiguous()
+            _lib.check(lib.spa_ring_fwd_flags_fp8qkv(q.data_ptr(), k.data_ptr(), v.data_ptr(), qsc.data_ptr(), ksc.data_ptr(), vsc.data_ptr(),
+                                                     out.data_ptr(), lse.data_ptr(), *tail))
+        else:
+            _lib.check(lib.spa_ring_fwd_flags(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), *tail))
     return out, lse
 
 
