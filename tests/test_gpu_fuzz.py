@@ -1,6 +1,6 @@
 """A bounded, fixed-seed sweep of random shapes through every entry of the HIP path against the
-float64 oracle: block forward, ring forward in its three schedules (contiguous and zigzag shards), e4m3 K/V (block and ring),
-packed variable-length batches, and the three backward forms.  Shapes are drawn from lists that
+float64 oracle: block forward, ring forward in its three schedules (contiguous and zigzag shards) and with arrival flags,
+e4m3 K/V (block and ring), packed variable-length batches, and the three backward forms.  Shapes are drawn from lists that
 straddle the kernels' tile sizes (1, 63..65, 127..130, 255..257, ragged tails) and the
 workgroup-form overrides are drawn as well, so that every kernel variant sees awkward sizes.
 The sweep stops at its first failure and names the case."""
@@ -49,10 +49,11 @@ def _case(rng):
     D, H, B = rng.choice([32, 64, 128]), rng.choice([1, 2, 3]), rng.choice([1, 2])
     causal = rng.random() < 0.5
     kind = rng.choice(["block", "block", "ring", "ring_bwd", "fp8", "fp8", "fp8_ring", "varlen", "block_bwd", "block_bwd",
-                       "varlen_bwd", "varlen_bwd", "zigzag", "zigzag", "fp8_qkv"])
+                       "varlen_bwd", "varlen_bwd", "zigzag", "zigzag", "fp8_qkv", "flags"])
     share, groups = rng.choice([0, 0, 1, 2, 2]), rng.choice([0, 0, 1, 2])
     _lib.tune("fwd_share", share)
     _lib.tune("fwd_groups", groups)
+    _lib.tune("fwd32_split", rng.choice([0, 0, 1, 2]))
     g = torch.Generator().manual_seed(rng.randrange(1 << 30))
     mk = lambda *shape, dt=None: torch.randn(shape, generator=g).to(dt or dtype)
     atol, rtol = OUT_TOL[dtype]
@@ -69,6 +70,20 @@ def _case(rng):
         o, l = ops.flash_fwd(q8.to(DEV), k8.to(DEV), v8.to(DEV), None, causal, layout="bhsd", q_scale=qs, k_scale=ks, v_scale=vs, out_dtype=dt)
         _close("out", o, want_o, *OUT_TOL[dt], info)
         _close("lse", l, want_l, LSE_ATOL, 0, info)
+        return
+    if kind == "flags":  # one launch per rank behind arrival flags (all raised): 16-bit types, D = 64 or 128
+        if dtype == torch.float32 or D == 32:
+            return
+        P, s = rng.choice([2, 3, 4, 5]), rng.choice([32, 64, 100, 128, 192, 260])
+        info = (kind, dtype, B, H, P, s, D, causal, groups)
+        q, k, v = (mk(B, P * s, H, D) for _ in range(3))
+        want_o, want_l = O.full_attention(q, k, v, None, causal)
+        flags = ops.RingFlags(P, torch.device(DEV))
+        flags.set_all()
+        o, l = ops.ring_fwd_flags(q.to(DEV), k.to(DEV), v.to(DEV), P, flags, None, causal)
+        _close("out", o, want_o, atol, rtol, info)
+        _close("lse", l, want_l, LSE_ATOL, 0, info)
+        assert not flags.failed(), info
         return
     if kind == "block":
         Sq = rng.choice([1, 7, 64, 65, 127, 128, 129, 200, 256, 300, 513, 700])
@@ -183,3 +198,4 @@ def test_fixed_seed_sweep_of_random_shapes_against_the_oracle():
     finally:
         _lib.tune("fwd_share", 0)
         _lib.tune("fwd_groups", 0)
+        _lib.tune("fwd32_split", 0)
