@@ -369,9 +369,22 @@ ROW_SPECS = {
 }
 
 
+# Rows that `--workload` can print and the default line leaves out (the line is short of room).
+EXTRA_ROW_NOTES = {
+    "decode_key_split": "a decode step against a long cache: bf16 q [1,1,32,128] (one new token) x K, V [1,32768,32,128], no mask; the keys "
+                        "are cut into chunks that run side by side (spa_flash_fwd_splitkv, as many as the library suggests); value = K and V "
+                        "bytes per call time; plain_gbps = the same call as one launch of 32 workgroups (spa_flash_fwd); e4m3_gbps = the "
+                        "split call on an e4m3 cache (half the bytes per key); q128_tflops = the split call with 128 query rows",
+}
+EXTRA_ROW_SPECS = {
+    "decode_key_split": ("decode: q [1,1,32,128] x K/V [1,32768,32,128] bf16, keys split", "GB/s", "hbm", "flash_fwd16<bf16,128,split keys>",
+                         HBM_PEAK_GBPS, ("plain_gbps", "e4m3_gbps", "q128_tflops", "chunks")),
+}
+
+
 def make_row(name, ms_per_step, value, **extra):
     """One entry of `rows` (without cpu_baseline) from the table above."""
-    workload, unit, bound, kernel, peak, keys = ROW_SPECS[name]
+    workload, unit, bound, kernel, peak, keys = (ROW_SPECS.get(name) or EXTRA_ROW_SPECS[name])
     if set(extra) != set(keys):
         raise KeyError(f"{name}: expected extras {keys}, got {sorted(extra)}")
     cfg = {"workload": workload}
@@ -379,6 +392,11 @@ def make_row(name, ms_per_step, value, **extra):
     return {"row": name, "value": round(value, 2), "unit": unit, "ms_per_step": round(ms_per_step, 4), "config": cfg,
             "roofline": {"bound": bound, "achieved": round(value, 2), "peak": peak, "unit": unit,
                          "frac": round(value / peak, 4), "traffic": row_traffic(name)}}  # (the kernel's name stays in ROW_SPECS: the line is short of room)
+
+
+def _lib_mod():
+    from sp_aurora_amd import _lib
+    return _lib
 
 
 _ROW_TRAFFIC = None
@@ -542,6 +560,28 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
         gb = nbytes / (m["ms_per_step"] * 1e-3) / 1e9
         finish("merge_update_out_and_lse", m, gb)
         del sets
+    if "decode" in which:
+        Bn, Hn, Skn, Dn = 1, 32, 32768, 128
+        k, v = rand_tensors(torch, (Bn, Skn, Hn, Dn), 7, 2, 1.0, torch.bfloat16, dev)
+        k8, ksc = ops.quantize_fp8_per_head(k.float())
+        v8, vsc = ops.quantize_fp8_per_head(v.float())
+        kv_bytes = 2.0 * Bn * Skn * Hn * Dn * 2
+        res = {}
+        for sq in (1, 128):
+            (q,) = rand_tensors(torch, (Bn, sq, Hn, Dn), 8, 1, 1.0, torch.bfloat16, dev)
+            out = torch.empty_like(q)
+            lse = torch.empty((Bn, Hn, sq), dtype=torch.float32, device=dev)
+            n = _lib_mod().load().spa_flash_fwd_splitkv_suggest(Bn, Hn, sq, Skn, Dn, 0, 1)
+            ws = ops.flash_fwd_splitkv_workspace(q, max(n, 1))
+            f_split = lambda: ops.flash_fwd(q, k, v, None, False, out=out, lse=lse, split_kv=n, workspace=ws)
+            f_plain = lambda: ops.flash_fwd(q, k, v, None, False, out=out, lse=lse, split_kv=None)
+            f_e4m3 = lambda: ops.flash_fwd(q, k8, v8, None, False, out=out, lse=lse, k_scale=ksc, v_scale=vsc, split_kv=n, workspace=ws)
+            res[sq] = (n, measure(torch, f_split, 20, 5, **light), measure(torch, f_plain, 20, 5, **light), measure(torch, f_e4m3, 20, 5, **light))
+        n1, m_split, m_plain, m_e4 = res[1]
+        gbps = lambda nbytes, m: nbytes / (m["ms_per_step"] * 1e-3) / 1e9
+        finish("decode_key_split", m_split, gbps(kv_bytes, m_split), plain_gbps=gbps(kv_bytes, m_plain), e4m3_gbps=gbps(kv_bytes / 2, m_e4),
+               q128_tflops=tfl(4.0 * Bn * Hn * 128 * Skn * Dn, res[128][1]), chunks=n1)
+        del k, v, k8, v8
     if "config5" in which:
         Bn, Sn, Hn, Dn, Pn = 1, 32768, 16, 128, 16
         qkv, = rand_tensors(torch, (Bn, Sn, 3, Hn, Dn), 4, 1, 1.0, torch.bfloat16, dev)
@@ -751,7 +791,7 @@ def pmc_summary_rows(fetch_dir, write_dir):
 
 # ------------------------------------------------------------------------------------ main
 ROW_SETS = {"fp8kv": {"fp8kv"}, "relayout": {"config4"}, "ulysses": {"config4"}, "merge": {"merge"}, "backward": {"config5"},
-            "config1": {"config1"}, "config2": {"config2"}, "zigzag": {"zigzag"}, "hbm": {"config4", "merge"}}
+            "config1": {"config1"}, "config2": {"config2"}, "zigzag": {"zigzag"}, "hbm": {"config4", "merge"}, "decode": {"decode"}}
 ALL_ROWS = {"config1", "config2", "zigzag", "config4", "fp8kv", "merge", "config5"}
 LINE_LIMIT = 7500  # bytes of the printed line: readers that keep only the end of the output keep 8 KB
 

@@ -102,6 +102,31 @@ int spa_flash_fwd_fp8kv(const void* q, const void* k8, const void* v8,
                         float scale, int mask_mode, int dtype, void* stream);
 
 /*
+ * The block forward for calls with few query rows and many keys (a decode step against a KV cache: the call sites that hand
+ * the operator a cache, adapters/hf_adapter.py:141-155): without a mask the keys can be cut into nsplit chunks that run
+ * side by side on the same query rows (grid planes of one launch), each leaving its block result (out in q's type, lse)
+ * in the workspace; a second kernel applies update_out_and_lse (sp_aurora/utils.py:103-104) to all of them.  The plain
+ * launch has B * H * ceil(Sq / 128) workgroups however long the keys are, which leaves most of the 256 CUs idle for such a call.
+ * spa_flash_fwd_splitkv_suggest returns the number of chunks the library would take for a shape (1: do not split);
+ * nsplit = 1 is spa_flash_fwd.  Chunks hold a multiple of 128 keys, so fewer than nsplit may run.  bf16 / fp16, D in
+ * {64, 128}, mask none, K/V below 2 GiB per (batch, head).  workspace: spa_flash_fwd_splitkv_workspace_bytes() bytes, 16-byte
+ * aligned, the caller's.  _fp8kv: K / V as e4m3 bytes with scales, as for spa_flash_fwd_fp8kv.
+ */
+int64_t spa_flash_fwd_splitkv_workspace_bytes(int B, int H, int Sq, int D, int nsplit, int dtype);
+int spa_flash_fwd_splitkv_suggest(int B, int H, int Sq, int Sk, int D, int mask_mode, int dtype);
+int spa_flash_fwd_splitkv(const void* q, const void* k, const void* v, void* out, float* lse, void* workspace,
+                          int B, int H, int Sq, int Sk, int D, int nsplit,
+                          const int64_t q_strides[3], const int64_t k_strides[3],
+                          const int64_t v_strides[3], const int64_t o_strides[3],
+                          float scale, int dtype, void* stream);
+int spa_flash_fwd_splitkv_fp8kv(const void* q, const void* k8, const void* v8, const float* k_scale, const float* v_scale,
+                                void* out, float* lse, void* workspace,
+                                int B, int H, int Sq, int Sk, int D, int nsplit,
+                                const int64_t q_strides[3], const int64_t k_strides[3],
+                                const int64_t v_strides[3], const int64_t o_strides[3],
+                                float scale, int dtype, void* stream);
+
+/*
  * spa_flash_fwd_fp8kv with q held as e4m3 as well: Q = q8 * q_scale[b*H + h] (fp32 contiguous [B,H], positive),
  * q8 [B,H,Sq,D] by strides in bytes, rows of q8 and k8 16-byte aligned, rows of v8 8-byte aligned; out (and the
  * softmax) in `dtype` (SPA_BF16 or SPA_F16); D = 128.  The scores q8 . k8 are formed on the 8-bit matrix

@@ -36,6 +36,10 @@ SIGNATURES = {
     "spa_ring_fwd_flags_fp8qkv": (_i, [_vp] * 9 + [ctypes.c_uint32, ctypes.c_uint32, _vp] + [_i] * 6 + [_s3] * 4 + [_f, _i, _i, _vp]),
     "spa_ring_flag_set": (_i, [_vp, _i, ctypes.c_uint32, _vp]),
     "spa_ring_fwd_workspace_bytes": (ctypes.c_int64, [_i, _i, _i, _i, _i, _i]),
+    "spa_flash_fwd_splitkv_workspace_bytes": (ctypes.c_int64, [_i, _i, _i, _i, _i, _i]),
+    "spa_flash_fwd_splitkv_suggest": (_i, [_i, _i, _i, _i, _i, _i, _i]),
+    "spa_flash_fwd_splitkv": (_i, [_vp] * 6 + [_i] * 6 + [_s3] * 4 + [_f, _i, _vp]),
+    "spa_flash_fwd_splitkv_fp8kv": (_i, [_vp] * 8 + [_i] * 6 + [_s3] * 4 + [_f, _i, _vp]),
     "spa_ring_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _s3, _s3, _s3, _s3, _f, _i, _i, _i, _vp]),
     "spa_static_scratch_bytes": (ctypes.c_int64, []),
     "spa_static_scratch_init": (_i, []),
@@ -65,7 +69,7 @@ class SpaError(RuntimeError):
 
 
 # entry points that return an int but launch nothing: they run as they are while recording
-_QUERIES = ("spa_abi_version", "spa_tune", "spa_device_info", "spa_static_scratch_init")
+_QUERIES = ("spa_abi_version", "spa_tune", "spa_device_info", "spa_static_scratch_init", "spa_flash_fwd_splitkv_suggest")
 
 
 class _Recorder:

@@ -20,6 +20,7 @@ UNITS = [
     ("flash_fwd.hip", "flash_fwd.o", _FWD),
     ("flash_fwd.hip", "flash_fwd_zigzag.o", _FWD + ["-DSPA_FWD_ZIGZAG_UNIT"]),
     ("flash_fwd.hip", "flash_fwd_big.o", _FWD + ["-DSPA_FWD_BIG_UNIT"]),
+    ("flash_fwd.hip", "flash_fwd_splitkv.o", _FWD + ["-DSPA_FWD_SPLITKV_UNIT"]),
     ("flash_bwd.hip", "flash_bwd.o", []),
     ("flash_bwd.hip", "flash_bwd_big.o", ["-DSPA_BWD_BIG_UNIT"]),
     ("spa_abi.hip", "spa_abi.o", []),

@@ -100,10 +100,14 @@ __device__ __forceinline__ int v_swizzle(int row) {
 // 64-deep step; V is widened to T as with KV8 and P V stays a 16-bit contraction.
 // WAIT: the variant for a ring rank whose chunks arrive while its launch runs (FwdParams::arrive): a bounded wait for
 // a chunk's flag before the chunk's first tile is loaded.
+// KS: the variant that splits the KEYS of a call with few query rows over grid.z (FwdParams::sk_last): "rank" z takes
+// chunk z of the keys for the SAME query rows and writes its block result to rows z * Sq .. of (out, lse), which the
+// launcher points at a scratch tensor; a second kernel merges the z results.
 template <typename T, int D, int NG, bool SHARE, bool KV8 = false, bool FINALN = false, bool ZZ = false, bool BIG = false,
-          bool QK8 = false, bool WAIT = false>
+          bool QK8 = false, bool WAIT = false, bool KS = false>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams pk) {
   static_assert(!(FINALN && SHARE), "the merging epilogue goes with 128-row workgroups");
+  static_assert(!KS || (!SHARE && !FINALN && !ZZ && !BIG && !QK8 && !WAIT), "split keys: 128-row workgroups, plain results");
   static_assert(!QK8 || (KV8 && D == 128 && !ZZ && !BIG), "8-bit scores: e4m3 q, k, v, head dim 128, contiguous chunks");
   typedef typename std::conditional<KV8, unsigned char, T>::type KVT;  // element type of K / V in memory
   typedef typename std::conditional<QK8, unsigned char, T>::type QT;   // element type of q in memory
@@ -182,7 +186,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const int qw0 = q0 + (SHARE ? grp * FWD_BM : 0) + w * 32;
   const int64_t qoff = (int64_t)rank * p.Sq;  // first row of this rank's query chunk
 
-  const QT* qp = (const QT*)p.q + b * p.qs.b + h * p.qs.h + qoff * p.qs.s;
+  const QT* qp = (const QT*)p.q + b * p.qs.b + h * p.qs.h + (KS ? 0 : qoff * p.qs.s);  // (KS: every chunk of keys meets the same rows)
   const KVT* kp = (const KVT*)p.k + b * p.ks.b + h * p.ks.h;
   const KVT* vp = (const KVT*)p.v + b * p.vs.b + h * p.vs.h;
 
@@ -228,7 +232,9 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const bool diag = p.causal && p.t_begin == 0;
   const int kv_end = q0 + C::BMW < p.Sk ? q0 + C::BMW : p.Sk;  // keys of the diagonal chunk in use
   const int n_diag = diag ? (kv_end + TILE - 1) / TILE : 0;
-  const int npc = (p.Sk + TILE - 1) / TILE;                    // sub-tiles per full chunk
+  // (KS: one step, the rank's own chunk; the last chunk of the keys may be shorter than the others)
+  const int ks_klen = KS && rank == p.P - 1 ? p.sk_last : p.Sk;
+  const int npc = ((KS ? ks_klen : p.Sk) + TILE - 1) / TILE;   // sub-tiles per full chunk
   const int zz_last_half = zz ? rank : -1;
   const int klen_h = zz ? zz_hs : p.Sk;                        // keys of a half step
   const int npc_h = (klen_h + TILE - 1) / TILE;                // sub-tiles of a half step
@@ -312,7 +318,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     ch = ch < 0 ? 0 : ch;  // only past the end of the schedule, where nothing is used
     c.sb.masked = c.i < n_diag;
     c.sb.ch = ch;
-    c.sb.klen = c.i >= n_diag && c.t <= zz_last_half ? klen_h : p.Sk;
+    c.sb.klen = KS ? ks_klen : c.i >= n_diag && c.t <= zz_last_half ? klen_h : p.Sk;
     c.sb.krel = (c.j * KSTEP + (SHARE ? 0 : grp)) * BN;
     c.sb.krow = ch * p.Sk + c.sb.krel;
     c.sb.kend = ch * p.Sk + p.Sk;
@@ -345,7 +351,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const unsigned vdoff = (unsigned)((drow * p.vs.s + ((dpos ^ v_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(KVT));
   const unsigned krow_b = (unsigned)(p.ks.s * (int64_t)sizeof(KVT));  // bytes per K row
   const unsigned vrow_b = (unsigned)(p.vs.s * (int64_t)sizeof(KVT));
-  const int64_t rows_all = (int64_t)p.P * p.Sk;
+  const int64_t rows_all = KS ? (int64_t)(p.P - 1) * p.Sk + p.sk_last : (int64_t)p.P * p.Sk;
   const unsigned long long kbytes = (unsigned long long)(((rows_all - 1) * p.ks.s + D) * (int64_t)sizeof(KVT));
   const unsigned long long vbytes = (unsigned long long)(((rows_all - 1) * p.vs.s + D) * (int64_t)sizeof(KVT));
   static_assert(!(BIG && KV8), "the re-based variants are built for 16-bit K / V");
@@ -699,7 +705,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     ch = ch < 0 ? ch + p.P : ch;
     cs.sb.masked = n_diag > 0;
     cs.sb.ch = ch;
-    cs.sb.klen = n_diag == 0 && cs.t <= zz_last_half ? klen_h : p.Sk;
+    cs.sb.klen = KS ? ks_klen : n_diag == 0 && cs.t <= zz_last_half ? klen_h : p.Sk;
     cs.sb.krel = (SHARE ? 0 : grp) * BN;
     cs.sb.krow = ch * p.Sk + cs.sb.krel;
     cs.sb.kend = ch * p.Sk + p.Sk;
@@ -1635,10 +1641,30 @@ hipError_t launch16_any(const FwdParams& p, int D, int dtype, hipStream_t stream
 
 }  // namespace
 
-// This file makes three objects: compiled with SPA_FWD_ZIGZAG_UNIT it holds the zigzag variants of the 16-bit
-// kernel and nothing else, with SPA_FWD_BIG_UNIT the re-based variants, those with 8-bit scores and those that wait for chunk arrival flags, without either
+// This file makes four objects: compiled with SPA_FWD_ZIGZAG_UNIT it holds the zigzag variants of the 16-bit
+// kernel and nothing else, with SPA_FWD_SPLITKV_UNIT those that split the keys over the grid, with SPA_FWD_BIG_UNIT the
+// re-based variants, those with 8-bit scores and those that wait for chunk arrival flags, without any of them
 // everything else (so that the parts compile side by side).
-#if defined(SPA_FWD_ZIGZAG_UNIT)
+#if defined(SPA_FWD_SPLITKV_UNIT)
+// Keys split over grid.z (the caller has set P, Sk, sk_last, nranks = P and pointed out / lse at the scratch tensors).
+hipError_t spa_launch_fwd16_splitkv(FwdParams p, int D, int dtype, hipStream_t stream) {
+  if (p.causal || p.P < 2 || p.nranks != p.P || p.rank0 != 0 || p.t_begin != 0 || p.t_count != 1 || p.sk_last <= 0 || p.sk_last > p.Sk ||
+      p.Sk <= fwd_bn<128>() || p.zigzag || p.big || p.arrive || p.q_scale || p.cu_q || p.epi != SPA_EPI_PLAIN || (p.k_scale && !p.v_scale))
+    return hipErrorInvalidValue;
+  p.nqt = fwd_tiles(p, FWD_BM);
+#define SPA_KS(T, DD, KV8) \
+  launch<flash_fwd16_kernel<T, DD, 2, false, KV8, false, false, false, false, false, true>>(2 * FWD_THREADS, Fwd16Cfg<DD, 2, false>::SMEM, p, stream)
+  if (p.k_scale) {
+    if (dtype == 1) { if (D == 128) return SPA_KS(__bf16, 128, true); if (D == 64) return SPA_KS(__bf16, 64, true); }
+    if (dtype == 2) { if (D == 128) return SPA_KS(_Float16, 128, true); if (D == 64) return SPA_KS(_Float16, 64, true); }
+    return hipErrorInvalidValue;
+  }
+  if (dtype == 1) { if (D == 128) return SPA_KS(__bf16, 128, false); if (D == 64) return SPA_KS(__bf16, 64, false); }
+  if (dtype == 2) { if (D == 128) return SPA_KS(_Float16, 128, false); if (D == 64) return SPA_KS(_Float16, 64, false); }
+#undef SPA_KS
+  return hipErrorInvalidValue;
+}
+#elif defined(SPA_FWD_ZIGZAG_UNIT)
 hipError_t spa_launch_fwd16_zigzag(const FwdParams& p, int D, int dtype, hipStream_t stream) {
   return launch16_any<true>(p, D, dtype, stream);
 }
@@ -1724,4 +1750,4 @@ hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t strea
   }
   return hipErrorInvalidValue;
 }
-#endif  // SPA_FWD_ZIGZAG_UNIT / SPA_FWD_BIG_UNIT
+#endif  // SPA_FWD_SPLITKV_UNIT / SPA_FWD_ZIGZAG_UNIT / SPA_FWD_BIG_UNIT

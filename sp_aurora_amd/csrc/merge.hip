@@ -162,6 +162,40 @@ __global__ void __launch_bounds__(256) finalize_kernel(T* __restrict__ out, cons
     if (on[k]) Load8<T>::st(op[k], x[k]);
 }
 
+// Merge of the n block results a key-split forward left behind (rows j * Sq .. of `part`, [B, n * Sq, H, D] in T, and of
+// part_lse, [B, H, n * Sq]): update_out_and_lse (sp_aurora/utils.py:103-104) over all of them at once, as a running
+// (weighted sum, weight sum) relative to the largest lse so far.  All lse are finite (every chunk holds a key).
+template <typename T>
+__global__ void __launch_bounds__(256) splitkv_combine_kernel(T* __restrict__ out, float* __restrict__ lse, const T* __restrict__ part,
+                                                              const float* __restrict__ part_lse, int n, int H, int Sq, int D,
+                                                              int cpr_shift, unsigned nrows, Strides3 os, int64_t lse_bh) {
+  const unsigned gid = blockIdx.x * 256u + threadIdx.x;
+  const unsigned row = gid >> cpr_shift;
+  const int ch = (int)(gid & ((1u << cpr_shift) - 1u));
+  if (row >= nrows) return;
+  const RowIdx r = decode_row(row, H);
+  const int64_t prow = (int64_t)H * D;                                  // elements between rows of `part`
+  const T* pp = part + ((int64_t)r.b * n * Sq + r.s) * prow + r.h * D + ch * 8;
+  const float* pl = part_lse + ((int64_t)r.b * H + r.h) * ((int64_t)n * Sq) + r.s;
+  float x[8], xb[8], lb = pl[0], wsum = 1.f;
+  Load8<T>::ld(pp, x);
+  for (int j = 1; j < n; ++j) {
+    Load8<T>::ld(pp + (int64_t)j * Sq * prow, xb);
+    const float lj = pl[(int64_t)j * Sq];
+    const float mx = fmaxf(lb, lj);
+    const float wa = __expf(lb - mx), wb = __expf(lj - mx);
+    wsum = wsum * wa + wb;
+    lb = mx;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = x[i] * wa + xb[i] * wb;
+  }
+  const float inv = 1.f / wsum;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) x[i] *= inv;
+  Load8<T>::st(out + r.b * os.b + r.h * os.h + (int64_t)r.s * os.s + ch * 8, x);
+  if (ch == 0) lse[((int64_t)r.b * H + r.h) * lse_bh + r.s] = lb + __logf(wsum);
+}
+
 // delta[b,h,s] = sum_d dout*out; the D/8 lanes of a row reduce with DPP-free shuffles.
 template <typename T>
 __global__ void __launch_bounds__(256) delta_kernel(const T* __restrict__ out, const T* __restrict__ dout,
@@ -256,6 +290,21 @@ hipError_t spa_launch_delta(const void* out, const void* dout, float* delta, int
     hipLaunchKernelGGL((delta_kernel<__bf16>), g.grid, dim3(256), 0, stream, (const __bf16*)out, (const __bf16*)dout, delta, H, Sq, g.cpr_shift, g.nrows, g.half, os, ds);
   else if (dtype == 2)
     hipLaunchKernelGGL((delta_kernel<_Float16>), g.grid, dim3(256), 0, stream, (const _Float16*)out, (const _Float16*)dout, delta, H, Sq, g.cpr_shift, g.nrows, g.half, os, ds);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+hipError_t spa_launch_splitkv_combine(void* out, float* lse, const void* part, const float* part_lse, int n, int B, int H, int Sq,
+                                      int D, Strides3 os, int64_t lse_bh, int dtype, hipStream_t stream) {
+  const RowGrid g = row_grid(B, H, Sq, D);
+  if (!g.ok || n < 1) return hipErrorInvalidValue;
+  if (dtype == 1)
+    hipLaunchKernelGGL((splitkv_combine_kernel<__bf16>), g.grid, dim3(256), 0, stream, (__bf16*)out, lse, (const __bf16*)part, part_lse, n, H,
+                       Sq, D, g.cpr_shift, g.nrows, os, lse_bh);
+  else if (dtype == 2)
+    hipLaunchKernelGGL((splitkv_combine_kernel<_Float16>), g.grid, dim3(256), 0, stream, (_Float16*)out, lse, (const _Float16*)part,
+                       part_lse, n, H, Sq, D, g.cpr_shift, g.nrows, os, lse_bh);
   else
     return hipErrorInvalidValue;
   return hipGetLastError();

@@ -71,6 +71,9 @@ struct FwdParams {
   // K / V rows of one (batch, head) span 2 GiB or more: the launcher takes the kernel variants that re-base their
   // buffer descriptors per tile (16-bit kernels; the fp32 kernels address with 64-bit pointers anyway)
   int big = 0;
+  // Keys split over grid.z for calls with few query rows (the KS variants): K / V hold P chunks of Sk keys, the last
+  // one sk_last keys; plane z computes the block (all Sq query rows) x (chunk z) and writes it to rows z * Sq .. of out / lse.
+  int sk_last = 0;
 };
 
 // Layout of the ring-step slots of one rank in the caller's workspace (16-bit inputs, ring of P):

@@ -124,12 +124,17 @@ def prepared(fn, *args, **kwargs):
 
 
 def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None, lse=None, k_scale=None, v_scale=None,
-              q_scale=None, out_dtype=torch.bfloat16):
+              q_scale=None, out_dtype=torch.bfloat16, split_kv="auto", workspace=None):
     """Block attention forward -> (out like q, lse fp32 [B,H,Sq]).  Calls spa_flash_fwd, or
     spa_flash_fwd_fp8kv when k, v are torch.float8_e4m3fn (then k_scale, v_scale fp32 [B,H] give
     K = k * k_scale[b,h], V = v * v_scale[b,h]; q bf16 or fp16), or spa_flash_fwd_fp8qkv when q is
     torch.float8_e4m3fn as well (q_scale fp32 [B,H]; D = 128; out in `out_dtype`, bf16 or fp16): the scores
-    then run on the 8-bit matrix instruction."""
+    then run on the 8-bit matrix instruction.
+    split_kv: for calls without a mask whose few query rows would leave most CUs idle (a decode step against a long
+    cache) the keys are cut into chunks that run side by side (spa_flash_fwd_splitkv[_fp8kv]): "auto" = as many as
+    the library suggests, an int = that many, None or 1 = never.  The chunks' results wait in `workspace` (a uint8 tensor
+    of flash_fwd_splitkv_workspace(...) bytes; allocated here when not given, except while the stream is being captured,
+    where "auto" then does not split)."""
     lib = _lib.load()
     fp8 = k.dtype == FP8 or v.dtype == FP8
     if q.dtype == FP8:
@@ -155,6 +160,32 @@ def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None
     if lse is None:
         lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
     _, os_ = _bhs(out, layout)
+    nsplit = 1
+    if split_kv is not None and split_kv != 1 and not causal and q.dtype in (torch.bfloat16, torch.float16) and D in (64, 128):
+        if split_kv == "auto":
+            nsplit = lib.spa_flash_fwd_splitkv_suggest(B, H, Sq, Sk, D, _lib.SPA_MASK_NONE, _dtype_code(q))
+            if nsplit > 1 and workspace is None and q.is_cuda and torch.cuda.is_current_stream_capturing():
+                nsplit = 1
+        else:
+            nsplit = int(split_kv)
+            if nsplit < 1:
+                raise ValueError(f"split_kv must be 'auto', None or a positive int, got {split_kv!r}")
+    if nsplit > 1:
+        need = lib.spa_flash_fwd_splitkv_workspace_bytes(B, H, Sq, D, nsplit, _dtype_code(q))
+        if workspace is None:
+            workspace = torch.empty((need,), dtype=torch.uint8, device=q.device)
+        elif workspace.numel() * workspace.element_size() < need or workspace.device != q.device:
+            raise ValueError(f"split_kv={nsplit}: the workspace must hold {need} bytes on q's device")
+        stail = (workspace.data_ptr(), B, H, Sq, Sk, D, nsplit, _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
+                 float(softmax_scale), _dtype_code(q), _stream())
+        with _on(q.device):
+            if fp8:
+                ksc, vsc = _fp8_scales(k, v, k_scale, v_scale, B, H)
+                _lib.check(lib.spa_flash_fwd_splitkv_fp8kv(q.data_ptr(), k.data_ptr(), v.data_ptr(), ksc.data_ptr(), vsc.data_ptr(),
+                                                           out.data_ptr(), lse.data_ptr(), *stail))
+            else:
+                _lib.check(lib.spa_flash_fwd_splitkv(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), *stail))
+        return out, lse
     tail = (B, H, Sq, Sk, D, _lib.strides3(qs), _lib.strides3(ks), _lib.strides3(vs), _lib.strides3(os_),
             float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(q), _stream())
     with _on(q.device):
@@ -165,6 +196,15 @@ def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None
         else:
             _lib.check(lib.spa_flash_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), *tail))
     return out, lse
+
+
+def flash_fwd_splitkv_workspace(q, nsplit, layout="bshd"):
+    """Scratch tensor (uint8) for flash_fwd(..., split_kv=nsplit) on this q."""
+    (B, H, Sq, D), _ = _bhs(q, layout)
+    need = _lib.load().spa_flash_fwd_splitkv_workspace_bytes(B, H, Sq, D, int(nsplit), _dtype_code(q))
+    if need < 0:
+        raise ValueError("the key split is built for bf16 / fp16 queries")
+    return torch.empty((need,), dtype=torch.uint8, device=q.device)
 
 
 def _flash_fwd_fp8qkv(lib, q, k, v, softmax_scale, causal, layout, out, lse, q_scale, k_scale, v_scale, out_dtype):

@@ -88,10 +88,11 @@ def _case(rng):
     if kind == "block":
         Sq = rng.choice([1, 7, 64, 65, 127, 128, 129, 200, 256, 300, 513, 700])
         Sk = rng.choice([1, 3, 64, 65, 128, 130, 255, 256, 400, 769])
-        info = (kind, dtype, B, H, Sq, Sk, D, causal, share, groups)
+        split = rng.choice(["auto", "auto", 2, 3, 5])   # keys cut into chunks that run side by side (calls without a mask, 16-bit, D >= 64)
+        info = (kind, dtype, B, H, Sq, Sk, D, causal, share, groups, split)
         q, k, v = mk(B, H, Sq, D), mk(B, H, Sk, D), mk(B, H, Sk, D)
         want_o, want_l = O.attn_block(q, k, v, None, causal)
-        o, l = ops.flash_fwd(q.to(DEV), k.to(DEV), v.to(DEV), None, causal, layout="bhsd")
+        o, l = ops.flash_fwd(q.to(DEV), k.to(DEV), v.to(DEV), None, causal, layout="bhsd", split_kv=split)
         _close("out", o, want_o, atol, rtol, info)
         _close("lse", l, want_l, LSE_ATOL, 0, info)
     elif kind == "ring":

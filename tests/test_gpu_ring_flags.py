@@ -15,6 +15,24 @@ from test_gpu_parity import DEV, check_lse, check_out
 pytestmark = pytest.mark.gpu
 
 
+def independent_stream():
+    """A stream whose work runs while a kernel on the current stream waits.  Streams share a few hardware queues; a
+    producer queued behind the waiting kernel on the same queue would only run once that kernel has given up.  Probed
+    with a tiny launch and a short spin limit: the flag of its second chunk is raised on the candidate stream."""
+    q, k, v = (t.to(DEV) for t in rand_qkv((1, 256, 1, 64), 899, torch.bfloat16))
+    for _ in range(8):
+        cand = torch.cuda.Stream()
+        flags = ops.RingFlags(2, q.device)
+        flags.set(1)
+        torch.cuda.synchronize()
+        ops.ring_fwd_flags(q, k, v, 2, flags, None, True, rank=1, spin_limit=40000)
+        flags.set(0, stream=cand)
+        torch.cuda.synchronize()
+        if not flags.failed():
+            return cand
+    pytest.skip("no stream on a hardware queue of its own")
+
+
 @pytest.mark.parametrize("B,H,P,s,D,dtype,causal", [
     (1, 4, 4, 256, 128, torch.bfloat16, True),
     (2, 2, 3, 100, 64, torch.float16, True),
@@ -51,8 +69,8 @@ def test_chunks_that_arrive_while_the_launch_runs():
     flags = ops.RingFlags(P, q.device)
     out = torch.zeros_like(q)
     lse = torch.zeros((B, H, P * s), dtype=torch.float32, device=DEV)
+    comm = independent_stream()
     torch.cuda.synchronize()
-    comm = torch.cuda.Stream()
     flags.set(r)                                     # the rank's own chunk
     ops.ring_fwd_flags(q, kbuf, vbuf, P, flags, None, True, rank=r, out=out, lse=lse, spin_limit=1 << 21)
     with torch.cuda.stream(comm):
@@ -118,8 +136,8 @@ def test_e4m3_tensors_with_flags(B, H, P, s, causal):
     flags.next_epoch()
     out2 = torch.zeros((B, S, H, D), dtype=torch.bfloat16, device=DEV)
     lse2 = torch.zeros((B, H, S), dtype=torch.float32, device=DEV)
+    comm = independent_stream()
     torch.cuda.synchronize()
-    comm = torch.cuda.Stream()
     flags.set(r)
     ops.ring_fwd_flags(q8, kbuf, vbuf, P, flags, None, True, rank=r, out=out2, lse=lse2, spin_limit=1 << 21, **scales)
     with torch.cuda.stream(comm):
