@@ -247,7 +247,10 @@ int spa_ring_fwd_fp8qkv(const void* q8, const void* k8, const void* v8,
  * (sp_aurora/intel_ring_flash_attn.py:72-134: compute step t while chunk t+1 is in flight, :96-134) at the speed of
  * the one-launch form, without a launch, a Q re-read and an (out, lse) round trip per step.  The producer raises a
  * flag AFTER the chunk's bytes are visible device-wide: spa_ring_flag_set on the stream that moved the chunk, or a
- * release store at system scope from a kernel.  Epochs let a flag array be reused without clearing (use a larger
+ * release store at system scope from a kernel.  The producer must be able to run while the launch waits: HIP streams share
+ * a few hardware queues, and work queued behind the waiting launch on the same queue starts only when the launch has
+ * given up (use a stream seen to run beside the consumer's, another process or a peer).
+ * Epochs let a flag array be reused without clearing (use a larger
  * epoch per call); the rank's own chunk has a flag like the others.  bf16 / fp16, D in {64, 128}, contiguous chunks;
  * rank >= 0 or -1 (every rank, one launch each).  arrive: uint32[P], fault: uint32[1], device memory.
  * The reference has no counterpart (its steps are separate kernel launches around blocking waits).
