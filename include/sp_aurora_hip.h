@@ -398,6 +398,20 @@ int spa_flash_fwd_varlen(const void* q, const void* k, const void* v, void* out,
                          float scale, int mask_mode, int dtype, void* stream);
 
 /*
+ * The ring over a packed variable-length batch in one launch per rank (or one for all ranks): the reference's varlen test
+ * runs its function under a process group (test/flash_attention/test_intel_ring_flash_attn_varlen.py:150-215), i.e. every
+ * rank holds the r-th of P equal slices of EVERY sequence, packed alike on every rank.  q, k, v, out: the P shards stacked,
+ * [P * shard_rows, H, D]; cu_seqlens [nseq + 1] describes one shard; lse [H, P * shard_rows].  Rank r walks the shards
+ * r, r-1, ... as spa_ring_fwd does (the causal mask inside each sequence at step 0 only), the query tile and the accumulators
+ * in registers across the shards.  fuse = SPA_RING_PER_RANK or SPA_RING_ALL_RANKS; rank >= 0 or -1; bf16 / fp16.
+ */
+int spa_ring_fwd_varlen(const void* q, const void* k, const void* v, void* out, float* lse,
+                        const int32_t* cu_seqlens, int nseq, int H, int shard_rows, int max_seqlen, int D, int P, int rank,
+                        const int64_t q_strides[2], const int64_t k_strides[2],
+                        const int64_t v_strides[2], const int64_t o_strides[2],
+                        float scale, int mask_mode, int dtype, int fuse, void* stream);
+
+/*
  * spa_flash_fwd_varlen with e4m3 K / V as in spa_flash_fwd_fp8kv: k8, v8 [total_k, H, D] by
  * (head, row) strides in bytes, k_scale / v_scale fp32 contiguous [nseq, H] (one scale per
  * sequence and head).  Same call sites as spa_flash_fwd_fp8kv.

@@ -53,6 +53,7 @@ SIGNATURES = {
     "spa_flash_bwd": (_i, [_vp] * 9 + [_i] * 5 + [_s3] * 7 + [_f, _i, _i, _vp]),
     "spa_flash_bwd_out": (_i, [_vp] * 9 + [_i] * 5 + [_s3] * 7 + [_f, _i, _i, _vp]),
     "spa_flash_fwd_varlen": (_i, [_vp] * 7 + [_i] * 7 + [_s3] * 4 + [_f, _i, _i, _vp]),
+    "spa_ring_fwd_varlen": (_i, [_vp] * 6 + [_i] * 7 + [_s3] * 4 + [_f, _i, _i, _i, _vp]),
     "spa_flash_bwd_varlen": (_i, [_vp] * 11 + [_i] * 7 + [_s3] * 7 + [_f, _i, _i, _vp]),
     "spa_flash_bwd_varlen_out": (_i, [_vp] * 11 + [_i] * 7 + [_s3] * 7 + [_f, _i, _i, _vp]),
 }

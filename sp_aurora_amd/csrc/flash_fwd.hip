@@ -103,8 +103,10 @@ __device__ __forceinline__ int v_swizzle(int row) {
 // KS: the variant that splits the KEYS of a call with few query rows over grid.z (FwdParams::sk_last): "rank" z takes
 // chunk z of the keys for the SAME query rows and writes its block result to rows z * Sq .. of (out, lse), which the
 // launcher points at a scratch tensor; a second kernel merges the z results.
+// VR: the variant for a ring over a packed variable-length batch (FwdParams::chunk_rows, rank_rows): chunks and ranks
+// lie a shard apart, not a sequence length apart.
 template <typename T, int D, int NG, bool SHARE, bool KV8 = false, bool FINALN = false, bool ZZ = false, bool BIG = false,
-          bool QK8 = false, bool WAIT = false, bool KS = false>
+          bool QK8 = false, bool WAIT = false, bool KS = false, bool VR = false>
 __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const FwdParams pk) {
   static_assert(!(FINALN && SHARE), "the merging epilogue goes with 128-row workgroups");
   static_assert(!KS || (!SHARE && !FINALN && !ZZ && !BIG && !QK8 && !WAIT), "split keys: 128-row workgroups, plain results");
@@ -184,7 +186,8 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   }
   const int q_lim = zz && !zhalf ? zz_hs : p.Sq;  // one past the last row this workgroup may own
   const int qw0 = q0 + (SHARE ? grp * FWD_BM : 0) + w * 32;
-  const int64_t qoff = (int64_t)rank * p.Sq;  // first row of this rank's query chunk
+  const int64_t qoff = (int64_t)rank * (VR ? p.rank_rows : p.Sq);  // first row of this rank's query chunk
+  const int crow = VR ? p.chunk_rows : p.Sk;                         // rows from one K / V chunk to the next
 
   const QT* qp = (const QT*)p.q + b * p.qs.b + h * p.qs.h + (KS ? 0 : qoff * p.qs.s);  // (KS: every chunk of keys meets the same rows)
   const KVT* kp = (const KVT*)p.k + b * p.ks.b + h * p.ks.h;
@@ -320,8 +323,8 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     c.sb.ch = ch;
     c.sb.klen = KS ? ks_klen : c.i >= n_diag && c.t <= zz_last_half ? klen_h : p.Sk;
     c.sb.krel = (c.j * KSTEP + (SHARE ? 0 : grp)) * BN;
-    c.sb.krow = ch * p.Sk + c.sb.krel;
-    c.sb.kend = ch * p.Sk + p.Sk;
+    c.sb.krow = ch * crow + c.sb.krel;
+    c.sb.kend = ch * crow + p.Sk;
   };
   // ---- global -> LDS: direct loads, no registers in between ----
   // Thread tg of the group owns slot tg of every round of 256 16-byte slots; round j of a
@@ -351,7 +354,7 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
   const unsigned vdoff = (unsigned)((drow * p.vs.s + ((dpos ^ v_swizzle<D>(drow)) * 8)) * (int64_t)sizeof(KVT));
   const unsigned krow_b = (unsigned)(p.ks.s * (int64_t)sizeof(KVT));  // bytes per K row
   const unsigned vrow_b = (unsigned)(p.vs.s * (int64_t)sizeof(KVT));
-  const int64_t rows_all = KS ? (int64_t)(p.P - 1) * p.Sk + p.sk_last : (int64_t)p.P * p.Sk;
+  const int64_t rows_all = KS ? (int64_t)(p.P - 1) * p.Sk + p.sk_last : (int64_t)(p.P - 1) * crow + p.Sk;
   const unsigned long long kbytes = (unsigned long long)(((rows_all - 1) * p.ks.s + D) * (int64_t)sizeof(KVT));
   const unsigned long long vbytes = (unsigned long long)(((rows_all - 1) * p.vs.s + D) * (int64_t)sizeof(KVT));
   static_assert(!(BIG && KV8), "the re-based variants are built for 16-bit K / V");
@@ -707,8 +710,8 @@ __global__ void __launch_bounds__(FWD_THREADS * NG, 1) flash_fwd16_kernel(const 
     cs.sb.ch = ch;
     cs.sb.klen = KS ? ks_klen : n_diag == 0 && cs.t <= zz_last_half ? klen_h : p.Sk;
     cs.sb.krel = (SHARE ? 0 : grp) * BN;
-    cs.sb.krow = ch * p.Sk + cs.sb.krel;
-    cs.sb.kend = ch * p.Sk + p.Sk;
+    cs.sb.krow = ch * crow + cs.sb.krel;
+    cs.sb.kend = ch * crow + p.Sk;
   }
   cv = cs;
   cursor_next(cv);
@@ -1642,7 +1645,8 @@ hipError_t launch16_any(const FwdParams& p, int D, int dtype, hipStream_t stream
 }  // namespace
 
 // This file makes four objects: compiled with SPA_FWD_ZIGZAG_UNIT it holds the zigzag variants of the 16-bit
-// kernel and nothing else, with SPA_FWD_SPLITKV_UNIT those that split the keys over the grid, with SPA_FWD_BIG_UNIT the
+// kernel and nothing else, with SPA_FWD_SPLITKV_UNIT those that split the keys over the grid and those for a ring over a
+// packed variable-length batch, with SPA_FWD_BIG_UNIT the
 // re-based variants, those with 8-bit scores and those that wait for chunk arrival flags, without any of them
 // everything else (so that the parts compile side by side).
 #if defined(SPA_FWD_SPLITKV_UNIT)
@@ -1662,6 +1666,22 @@ hipError_t spa_launch_fwd16_splitkv(FwdParams p, int D, int dtype, hipStream_t s
   if (dtype == 1) { if (D == 128) return SPA_KS(__bf16, 128, false); if (D == 64) return SPA_KS(__bf16, 64, false); }
   if (dtype == 2) { if (D == 128) return SPA_KS(_Float16, 128, false); if (D == 64) return SPA_KS(_Float16, 64, false); }
 #undef SPA_KS
+  return hipErrorInvalidValue;
+}
+// A ring over a packed variable-length batch (cu_q, P > 1, chunk_rows / rank_rows = rows of a shard): 128-row workgroups.
+hipError_t spa_launch_fwd16_varlen_ring(FwdParams p, int D, int dtype, hipStream_t stream) {
+  if (!p.cu_q || !p.cu_k || p.chunk_rows <= 0 || p.rank_rows <= 0 || p.zigzag || p.big || p.arrive || p.k_scale || p.q_scale ||
+      p.epi != SPA_EPI_PLAIN)
+    return hipErrorInvalidValue;
+  p.nqt = fwd_tiles(p, FWD_BM);
+  const int force = spa_knob(SPA_KNOB_FWD_GROUPS);
+  const bool two = force ? force == 2 : p.Sk > fwd_bn<128>();
+#define SPA_VR(T, DD)                                                                                                                     \
+  (two ? launch<flash_fwd16_kernel<T, DD, 2, false, false, false, false, false, false, false, false, true>>(2 * FWD_THREADS, Fwd16Cfg<DD, 2, false>::SMEM, p, stream) \
+       : launch<flash_fwd16_kernel<T, DD, 1, false, false, false, false, false, false, false, false, true>>(FWD_THREADS, Fwd16Cfg<DD, 1, false>::SMEM, p, stream))
+  if (dtype == 1) { if (D == 128) return SPA_VR(__bf16, 128); if (D == 64) return SPA_VR(__bf16, 64); if (D == 32) return SPA_VR(__bf16, 32); }
+  if (dtype == 2) { if (D == 128) return SPA_VR(_Float16, 128); if (D == 64) return SPA_VR(_Float16, 64); if (D == 32) return SPA_VR(_Float16, 32); }
+#undef SPA_VR
   return hipErrorInvalidValue;
 }
 #elif defined(SPA_FWD_ZIGZAG_UNIT)
@@ -1710,6 +1730,7 @@ hipError_t spa_launch_fwd16_zigzag(const FwdParams& p, int D, int dtype, hipStre
 hipError_t spa_launch_fwd16_big(const FwdParams& p, int D, int dtype, hipStream_t stream);
 hipError_t spa_launch_fwd16_qk8(const FwdParams& p, int D, int dtype, hipStream_t stream);
 hipError_t spa_launch_fwd16_wait(const FwdParams& p, int D, int dtype, hipStream_t stream);
+hipError_t spa_launch_fwd16_varlen_ring(FwdParams p, int D, int dtype, hipStream_t stream);
 
 // Returns hipSuccess, or hipErrorInvalidValue for an unsupported (dtype, D).
 hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream) {
@@ -1727,6 +1748,7 @@ hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t strea
     p.out = (char*)slots.out<char>(p.part, p.part_slot) - row0 * p.os.s * 2;
     p.lse = slots.lse(p.part, p.P, p.part_slot) - row0;
   }
+  if ((dtype == 1 || dtype == 2) && p.chunk_rows) return spa_launch_fwd16_varlen_ring(p, D, dtype, stream);
   if ((dtype == 1 || dtype == 2) && p.arrive) return spa_launch_fwd16_wait(p, D, dtype, stream);
   if ((dtype == 1 || dtype == 2) && p.q_scale) return spa_launch_fwd16_qk8(p, D, dtype, stream);
   if (dtype == 1 || dtype == 2)

@@ -785,7 +785,10 @@ int flash_fwd_varlen(const char* what, const void* q, const void* k, const void*
                      const float* v_scale, void* out, float* lse, const int32_t* cu_seqlens_q,
                      const int32_t* cu_seqlens_k, int nseq, int H, int total_q, int total_k, int max_sq, int max_sk,
                      int D, const int64_t q_strides[2], const int64_t k_strides[2], const int64_t v_strides[2],
-                     const int64_t o_strides[2], float scale, int mask_mode, int dtype, void* stream) {
+                     const int64_t o_strides[2], float scale, int mask_mode, int dtype, void* stream, int P = 1, int rank = -1,
+                     int fuse = SPA_RING_PER_RANK) {
+  // P > 1: a ring over the packed batch.  The tensors are P stacked shards of total_q = total_k rows, every shard
+  // packed as cu_seqlens_q says; rank r (or every rank, -1) walks the shards in ring order, one launch per rank or one for all.
   const bool kv8 = k_scale || v_scale;
   if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "%s: null pointer", what);
   if (kv8 && (!k_scale || !v_scale)) return fail(SPA_EINVAL, "%s: null scale pointer", what);
@@ -793,6 +796,14 @@ int flash_fwd_varlen(const char* what, const void* q, const void* k, const void*
   const int rc = varlen_sizes_ok(what, cu_seqlens_q, cu_seqlens_k, nseq, H, total_q, total_k, max_sq, max_sk, D, dtype,
                                  mask_mode, scale);
   if (rc != SPA_OK) return rc;
+  if (P < 1 || rank < -1 || rank >= P) return fail(SPA_EINVAL, "%s: ring size %d, rank %d", what, P, rank);
+  if (P > 1) {
+    if (fuse != SPA_RING_PER_RANK && fuse != SPA_RING_ALL_RANKS) return fail(SPA_EINVAL, "%s: one launch per rank or one for all ranks", what);
+    if (dtype == SPA_F32 || kv8) return fail(SPA_EUNSUPPORTED, "%s: the ring over a packed batch is built for bf16 / fp16 tensors", what);
+    if (cu_seqlens_q != cu_seqlens_k || total_q != total_k || max_sq != max_sk)
+      return fail(SPA_EINVAL, "%s: a ring over a packed batch has one cu_seqlens for queries and keys", what);
+    if ((int64_t)P * total_q > 0x7fffffffLL || P > 65535) return fail(SPA_EINVAL, "%s: grid too large", what);
+  }
   if (kv8 && dtype == SPA_F32) return fail(SPA_EUNSUPPORTED, "%s: e4m3 K/V go with bf16 or fp16 queries", what);
   if (kv8 && D == 32) return fail(SPA_EUNSUPPORTED, "%s: e4m3 K/V need head dim 64 or 128", what);
   const int esz = elem_size(dtype), kesz = kv8 ? 1 : esz;
@@ -800,10 +811,12 @@ int flash_fwd_varlen(const char* what, const void* q, const void* k, const void*
                               : aligned16v(k, k_strides, esz) && aligned16v(v, v_strides, esz);
   if (!aligned16v(q, q_strides, esz) || !kv_aligned || !aligned16v(out, o_strides, esz) || ((uintptr_t)lse & 3) != 0)
     return fail(SPA_EALIGN, "%s: pointers and row strides must be 16-byte aligned (8-byte for e4m3 K/V)", what);
-  const bool big = !span_ok(max_sk, k_strides[1], D, kesz) || !span_ok(max_sk, v_strides[1], D, kesz);
-  if (big && big_kv_obstacle(kv8, dtype, k_strides[1], v_strides[1], esz))
+  // (a sequence's keys reach from its slice in the first shard to its slice in the last)
+  const int64_t key_span = (int64_t)(P - 1) * total_k + max_sk;
+  const bool big = key_span > 0x7fffffffLL || !span_ok((int)key_span, k_strides[1], D, kesz) || !span_ok((int)key_span, v_strides[1], D, kesz);
+  if (big && (P > 1 || big_kv_obstacle(kv8, dtype, k_strides[1], v_strides[1], esz)))
     return fail(SPA_EUNSUPPORTED, "%s: K/V of one (sequence, head) span 2 GiB or more (%s)", what,
-                big_kv_obstacle(kv8, dtype, k_strides[1], v_strides[1], esz));
+                P > 1 ? "not supported for a ring over a packed batch" : big_kv_obstacle(kv8, dtype, k_strides[1], v_strides[1], esz));
   FwdParams p;
   p.big = big && dtype != SPA_F32;
   p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
@@ -814,12 +827,26 @@ int flash_fwd_varlen(const char* what, const void* q, const void* k, const void*
   p.negq = scale < 0.f;
   p.causal = mask_mode == SPA_MASK_CAUSAL;
   p.nqt = 0;
-  p.lse_bh = total_q;
+  p.lse_bh = (int64_t)P * total_q;
   p.part = nullptr; p.part_slot = 0; p.npart = 0;
   p.epi = SPA_EPI_PLAIN;
   p.P = 1; p.rank0 = 0; p.nranks = 1; p.t_begin = 0; p.t_count = -1;
   p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
   p.k_scale = k_scale; p.v_scale = v_scale;
+  if (P > 1) {
+    p.P = P; p.chunk_rows = total_k; p.rank_rows = total_q;
+    const int r_lo = rank < 0 ? 0 : rank, r_hi = rank < 0 ? P : rank + 1;
+    if (fuse == SPA_RING_ALL_RANKS) {
+      p.rank0 = r_lo; p.nranks = r_hi - r_lo;
+      return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), what);
+    }
+    for (int r = r_lo; r < r_hi; ++r) {
+      p.rank0 = r; p.nranks = 1;
+      const hipError_t e = spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream);
+      if (e != hipSuccess) return launch_result(e, what);
+    }
+    return SPA_OK;
+  }
   return launch_result(spa_launch_flash_fwd(p, D, dtype, (hipStream_t)stream), what);
 }
 
@@ -875,6 +902,15 @@ int spa_flash_fwd_varlen(const void* q, const void* k, const void* v, void* out,
   return flash_fwd_varlen("spa_flash_fwd_varlen", q, k, v, nullptr, nullptr, out, lse, cu_seqlens_q, cu_seqlens_k, nseq, H,
                           total_q, total_k, max_sq, max_sk, D, q_strides, k_strides, v_strides, o_strides, scale,
                           mask_mode, dtype, stream);
+}
+
+int spa_ring_fwd_varlen(const void* q, const void* k, const void* v, void* out, float* lse, const int32_t* cu_seqlens, int nseq,
+                        int H, int shard_rows, int max_seqlen, int D, int P, int rank, const int64_t q_strides[2],
+                        const int64_t k_strides[2], const int64_t v_strides[2], const int64_t o_strides[2], float scale,
+                        int mask_mode, int dtype, int fuse, void* stream) {
+  return flash_fwd_varlen("spa_ring_fwd_varlen", q, k, v, nullptr, nullptr, out, lse, cu_seqlens, cu_seqlens, nseq, H, shard_rows,
+                          shard_rows, max_seqlen, max_seqlen, D, q_strides, k_strides, v_strides, o_strides, scale, mask_mode, dtype,
+                          stream, P, rank, fuse);
 }
 
 int spa_flash_fwd_varlen_fp8kv(const void* q, const void* k8, const void* v8, const float* k_scale,

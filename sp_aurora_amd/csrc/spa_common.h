@@ -74,6 +74,11 @@ struct FwdParams {
   // Keys split over grid.z for calls with few query rows (the KS variants): K / V hold P chunks of Sk keys, the last
   // one sk_last keys; plane z computes the block (all Sq query rows) x (chunk z) and writes it to rows z * Sq .. of out / lse.
   int sk_last = 0;
+  // A ring over a packed variable-length batch (cu_q set, P > 1): the tensors are P stacked shards of chunk_rows rows,
+  // every shard packed as cu_q says, so chunk c of a sequence's keys starts chunk_rows rows after chunk c - 1 and rank
+  // r's queries rank_rows rows after rank r - 1's (0: chunks and ranks follow each other, Sk and Sq rows apart).
+  int chunk_rows = 0;
+  int rank_rows = 0;
 };
 
 // Layout of the ring-step slots of one rank in the caller's workspace (16-bit inputs, ring of P):

@@ -685,6 +685,41 @@ def flash_fwd_varlen(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seql
     return out, lse
 
 
+def ring_fwd_varlen(q, k, v, cu_seqlens, max_seqlen, ring_size, softmax_scale=None, causal=False, rank=-1, fuse="rank", out=None,
+                    lse=None):
+    """Ring forward over a packed variable-length batch: q, k, v [P * T, H, D] = P stacked shards (rank r holds the r-th of
+    P equal slices of every sequence), cu_seqlens int32 [nseq + 1] the layout of one shard of T rows.  One launch per
+    rank (fuse="rank") or one for all ranks ("all").  Returns (out like q, lse fp32 [H, P * T]).  Calls spa_ring_fwd_varlen
+    (bf16 / fp16)."""
+    lib = _lib.load()
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    if not (q.dtype == k.dtype == v.dtype):
+        raise TypeError("q, k, v must share a dtype")
+    (PT, H, D), qs = _thd(q, "q")
+    shp_k, ks = _thd(k, "k")
+    shp_v, vs = _thd(v, "v")
+    P = int(ring_size)
+    if shp_k != (PT, H, D) or shp_v != (PT, H, D) or P < 1 or PT % P:
+        raise ValueError(f"ring over a packed batch: q, k, v of one shape whose rows ring_size={P} divides, got {tuple(q.shape)} "
+                         f"{tuple(k.shape)} {tuple(v.shape)}")
+    if fuse not in ("rank", "all"):
+        raise ValueError(f"fuse must be 'rank' or 'all', got {fuse!r}")
+    cu = _cu(cu_seqlens, q.device, "cu_seqlens")
+    if softmax_scale is None:
+        softmax_scale = D ** (-0.5)
+    if out is None:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    if lse is None:
+        lse = torch.empty((H, PT), dtype=torch.float32, device=q.device)
+    _, os_ = _thd(out, "out")
+    with _on(q.device):
+        _lib.check(lib.spa_ring_fwd_varlen(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), cu.data_ptr(), cu.numel() - 1, H, PT // P,
+            int(max_seqlen), D, P, int(rank), _lib.strides2(qs), _lib.strides2(ks), _lib.strides2(vs), _lib.strides2(os_),
+            float(softmax_scale), _lib.SPA_MASK_CAUSAL if causal else _lib.SPA_MASK_NONE, _dtype_code(q), RING_FUSE[fuse], _stream()))
+    return out, lse
+
+
 def _flash_bwd_varlen(name, q, k, v, dout, lse, delta, dq, dk, dv, grad_dtype, cu_seqlens_q, cu_seqlens_k,
                       max_seqlen_q, max_seqlen_k, softmax_scale, causal):
     if not (q.dtype == k.dtype == v.dtype == dout.dtype):

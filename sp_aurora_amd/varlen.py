@@ -59,14 +59,20 @@ class VarlenFlashAttnFunc(torch.autograd.Function):
         return dq, dk, dv, None, None, None, None, None, None, None, None
 
 
-def ring_varlen_forward(q, k, v, cu_seqlens, max_seqlen, softmax_scale, causal, ring_size):
+def ring_varlen_forward(q, k, v, cu_seqlens, max_seqlen, softmax_scale, causal, ring_size, fuse="rank"):
     """All ranks of a simulated ring over a packed batch (see the module docstring): q, k, v [P * T, H, D] =
     P stacked shards of T rows, cu_seqlens [nseq + 1] the layout of one shard.  Returns out like q and
-    lse fp32 [H, P * T]."""
+    lse fp32 [H, P * T].  fuse="rank" / "all": one launch per rank / for all ranks, the rank's query tile and accumulators
+    in registers across its shards (spa_ring_fwd_varlen; bf16 / fp16); "step" (and fp32): one variable-length block launch
+    per visited shard pair, merged with update_out_and_lse as separate passes."""
     P = int(ring_size)
     PT, H, D = q.shape
     if P < 1 or PT % P or k.shape != q.shape or v.shape != q.shape:
         raise ValueError(f"ring_size={P} must divide the packed rows {PT}, and k, v must have q's shape")
+    if fuse not in ("step", "rank", "all"):
+        raise ValueError(f"fuse must be 'step', 'rank' or 'all', got {fuse!r}")
+    if fuse != "step" and q.dtype in (torch.bfloat16, torch.float16) and P > 1:
+        return ops.ring_fwd_varlen(q, k, v, cu_seqlens, max_seqlen, P, softmax_scale, causal, fuse=fuse)
     T = PT // P
     out = torch.empty_like(q)
     lse = torch.empty((H, PT), dtype=torch.float32, device=q.device)

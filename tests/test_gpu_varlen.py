@@ -247,6 +247,21 @@ def test_ring_over_a_packed_batch_matches_per_sequence_attention(P, local_length
     out.backward(stack(glob_do).to(DEV))
     for x, j, name in zip(xs, range(3), "qkv"):
         check_grad(x.grad, stack([g[j] for g in want_g]), dtype, "d" + name)
+    # the three launch forms (per shard pair with separate merges; one launch per rank; one launch) agree with the oracle,
+    # and a single rank writes its rows only
+    from sp_aurora_amd import varlen as V
+    det = [x.detach() for x in xs]
+    for fuse in ("step", "rank", "all"):
+        o2, l2 = V.ring_varlen_forward(*det, cu, max(local_lengths), None, causal, P, fuse=fuse)
+        check_out(o2, stack(want_o), dtype, fuse)
+        check_lse(l2, stack_l(want_l))
+    if dtype != torch.float32:
+        r = P - 1
+        o3 = torch.full_like(det[0], 7.0)
+        l3 = torch.full((H, P * T), 7.0, dtype=torch.float32, device=DEV)
+        ops.ring_fwd_varlen(*det, cu, max(local_lengths), P, None, causal, rank=r, out=o3, lse=l3)
+        assert torch.equal(o3[r * T:], o2[r * T:]) or (o3[r * T:].float() - o2[r * T:].float()).abs().max() < 2e-2
+        assert (o3[:r * T] == 7.0).all() and (l3[:, :r * T] == 7.0).all()
 
 
 @pytest.mark.parametrize("P,local_lengths,H,D,dtype", [
