@@ -20,7 +20,7 @@ import torch
 
 from conftest import rand_qkv
 import sp_aurora_amd as spa
-from sp_aurora_amd import ops
+from sp_aurora_amd import _lib, ops
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -317,3 +317,29 @@ def test_rows_of_one_head_spanning_more_than_2_gib():
         ref = ref.float()
         bad = (got.float() - ref).abs() > 3e-2 * ref.abs().max() + 3e-2 * ref.abs()
         assert torch.isfinite(got).all() and not bad.any(), f"{name}: {int(bad.sum())} out of tolerance"
+
+
+def test_decode_step_against_a_long_cache_with_the_keys_split():
+    """The shape of `bench.py --workload decode`: one new token (and a block of 128) per head against 32768 cached keys, the
+    library's own choice of chunks.  Every head against the fp32 reference on the GPU, rows of two heads against the fp64
+    oracle; the e4m3 cache the same way on its dequantised values."""
+    B, H, Sk, D = 1, 32, 32768, 128
+    k, v = config_qkv((B, Sk, H, D), 7, n=2)
+    assert _lib.load().spa_flash_fwd_splitkv_suggest(B, H, 1, Sk, D, 0, _lib.SPA_BF16) > 1
+    for sq in (1, 128):
+        (q,) = config_qkv((B, sq, H, D), 8, n=1)
+        out, lse = ops.flash_fwd(q, k, v, None, False)                      # split_kv="auto"
+        for h in range(H):
+            ro, rl = ref_head(q[0, :, h], k[0, :, h], v[0, :, h], D ** -0.5, False)
+            assert_out(out[0, :, h], ro, f"decode Sq={sq} head {h}")
+            assert_lse(lse[0, h], rl, f"decode Sq={sq} head {h}")
+        for h in (0, H - 1):
+            spot_check_rows(out[0, :, h], lse[0, h], q[0, :, h], k[0, :, h], v[0, :, h], D ** -0.5, False, f"decode Sq={sq} head {h}", n_rows=3)
+        k8, ksc = ops.quantize_fp8_per_head(k.float())
+        v8, vsc = ops.quantize_fp8_per_head(v.float())
+        out8, lse8 = ops.flash_fwd(q, k8, v8, None, False, k_scale=ksc, v_scale=vsc)
+        kd, vd = k8.float() * ksc[:, None, :, None], v8.float() * vsc[:, None, :, None]
+        for h in (3, 17):
+            ro, rl = ref_head(q[0, :, h], kd[0, :, h], vd[0, :, h], D ** -0.5, False)
+            assert_out(out8[0, :, h], ro, f"decode e4m3 Sq={sq} head {h}")
+            assert_lse(lse8[0, h], rl, f"decode e4m3 Sq={sq} head {h}")
