@@ -81,3 +81,28 @@ def test_the_librarys_choice_and_what_is_refused():
     torch.cuda.synchronize()
     with pytest.raises(ValueError):
         ops.flash_fwd(q, k, k, layout="bhsd", split_kv=8, workspace=ws)                # a workspace for four chunks
+
+
+def test_key_split_replays_from_a_captured_graph():
+    """Two launches and a caller's workspace, nothing allocated, no synchronisation: the call can be captured; every replay
+    (with eager work in between and new values in the captured buffers) equals the eager result."""
+    B, H, Sq, Sk, D, n = 1, 8, 4, 4096, 128, 6
+    q, k, v = (rand((B, s_, H, D), 1030 + i, torch.bfloat16).to(DEV) for i, s_ in enumerate((Sq, Sk, Sk)))
+    ws = ops.flash_fwd_splitkv_workspace(q, n)
+    out, lse = torch.empty_like(q), torch.empty((B, H, Sq), dtype=torch.float32, device=DEV)
+    call = lambda: ops.flash_fwd(q, k, v, None, False, out=out, lse=lse, split_kv=n, workspace=ws)
+    eager_out, eager_lse = (t.clone() for t in call())
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for rep in range(3):
+        out.fill_(7)
+        lse.fill_(7)
+        ws.fill_(0xFF)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager_out) and torch.equal(lse, eager_lse), f"replay {rep} differs"
+        k.mul_(-1)
+        torch.cuda.synchronize()
+        k.mul_(-1)
