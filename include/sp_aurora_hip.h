@@ -470,8 +470,10 @@ int spa_flash_bwd_varlen_out(const void* q, const void* k, const void* v, const 
  *   SPA_TUNE_BWD_DKDV_FORM 1       compiler-scheduled MFMAs in the D = 128 dk/dv kernel
  *   SPA_TUNE_FWD32_SPLIT  1 | 2    never / whenever D <= 64: the fp32 forward with 32-row workgroups whose waves share
  *                                  the key tiles (the library takes it when 128-row workgroups would leave half the CUs idle)
+ *   SPA_TUNE_FEW_ROWS     1        a key-split forward of up to 4 query rows runs on the MFMA kernels instead of the
+ *                                  kernel that streams K and V past those rows
  */
-enum { SPA_TUNE_FWD_GROUPS = 0, SPA_TUNE_FWD_SHARE = 1, SPA_TUNE_BWD_DQ_WAVES = 2, SPA_TUNE_BWD_DKDV_FORM = 3, SPA_TUNE_FWD32_SPLIT = 4 };
+enum { SPA_TUNE_FWD_GROUPS = 0, SPA_TUNE_FWD_SHARE = 1, SPA_TUNE_BWD_DQ_WAVES = 2, SPA_TUNE_BWD_DKDV_FORM = 3, SPA_TUNE_FWD32_SPLIT = 4, SPA_TUNE_FEW_ROWS = 5 };
 int spa_tune(int knob, int value);
 
 #ifdef __cplusplus

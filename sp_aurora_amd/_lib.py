@@ -168,7 +168,7 @@ def check(code):
         raise SpaError(code, load().spa_last_error().decode("utf-8", "replace"))
 
 
-TUNE_KNOBS = {"fwd_groups": 0, "fwd_share": 1, "bwd_dq_waves": 2, "bwd_dkdv_form": 3, "fwd32_split": 4}
+TUNE_KNOBS = {"fwd_groups": 0, "fwd_share": 1, "bwd_dq_waves": 2, "bwd_dkdv_form": 3, "fwd32_split": 4, "few_rows": 5}
 
 
 def tune(knob, value):

@@ -25,6 +25,7 @@ UNITS = [
     ("flash_bwd.hip", "flash_bwd_big.o", ["-DSPA_BWD_BIG_UNIT"]),
     ("spa_abi.hip", "spa_abi.o", []),
     ("merge.hip", "merge.o", []),
+    ("decode_fwd.hip", "decode_fwd.o", []),
     ("relayout.hip", "relayout.o", []),
 ]
 FLAGS = [

@@ -18,6 +18,7 @@ static __device__ __align__(256) unsigned char scratch[SPA_STATIC_SCRATCH_BYTES]
 
 hipError_t spa_launch_flash_fwd(FwdParams p, int D, int dtype, hipStream_t stream);
 hipError_t spa_launch_fwd16_splitkv(FwdParams p, int D, int dtype, hipStream_t stream);
+hipError_t spa_launch_fwd_fewrows(FwdParams p, int D, int dtype, hipStream_t stream);
 hipError_t spa_launch_splitkv_combine(void* out, float* lse, const void* part, const float* part_lse, int n, int B, int H, int Sq,
                                       int D, Strides3 os, int64_t lse_bh, int dtype, hipStream_t stream);
 hipError_t spa_launch_flash_bwd(BwdParams p, int D, int dtype, hipStream_t stream);
@@ -128,6 +129,7 @@ bool aligned8(const void* p, const int64_t* s, int n) {
 
 // The key-split forward: how the keys are cut for a wanted number of chunks (chunks of a multiple of 128 keys, the
 // last one what is left), and the scratch the chunks' results need.
+constexpr int kFewRows = 3;   // query rows the K/V-streaming kernel takes (spa_launch_fwd_fewrows)
 struct KeySplit {
   int n, chunk, last;
   KeySplit(int Sk, int nsplit) {
@@ -139,11 +141,13 @@ struct KeySplit {
 int64_t splitkv_out_bytes(int B, int H, int Sq, int D, int n, int esz) { return ((int64_t)B * n * Sq * H * D * esz + 255) / 256 * 256; }
 
 // k_scale / v_scale non-null: K and V are e4m3 bytes (strides in bytes), q / out of type `dtype`.
-// nsplit > 1 (with a workspace): the keys are cut into chunks that run side by side on the same query rows.
+// nsplit >= 1 (the key-split entry points; a workspace when more than one chunk comes of it): the keys are cut into
+// chunks that run side by side on the same query rows.
 int flash_fwd(const char* what, const void* q, const void* k, const void* v, const float* k_scale, const float* v_scale,
               void* out, float* lse, int B, int H, int Sq, int Sk, int D, const int64_t q_strides[3],
               const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3], float scale,
-              int mask_mode, int dtype, void* stream, void* workspace = nullptr, int nsplit = 1) {
+              int mask_mode, int dtype, void* stream, void* workspace = nullptr, int nsplit = 0) {
+  const bool workspace_call = nsplit >= 1;   // one of the key-split entry points
   const bool kv8 = k_scale || v_scale;
   if (!q || !k || !v || !out || !lse) return fail(SPA_EINVAL, "%s: null pointer", what);
   if (kv8 && (!k_scale || !v_scale)) return fail(SPA_EINVAL, "%s: null scale pointer", what);
@@ -181,23 +185,33 @@ int flash_fwd(const char* what, const void* q, const void* k, const void* v, con
   p.P = 1; p.rank0 = 0; p.nranks = 1; p.t_begin = 0; p.t_count = -1;
   p.cu_q = nullptr; p.cu_k = nullptr;
   p.k_scale = k_scale; p.v_scale = v_scale;
-  if (nsplit > 1) {
+  {
     if (nsplit > 1024) return fail(SPA_EINVAL, "%s: nsplit %d above 1024", what, nsplit);
-    if (p.causal) return fail(SPA_EUNSUPPORTED, "%s: the keys are split for calls without a mask", what);
-    if (dtype == SPA_F32 || D == 32 || p.big) return fail(SPA_EUNSUPPORTED, "%s: built for bf16 / fp16, head dim 64 or 128, K/V below 2 GiB per (batch, head)", what);
-    if (!workspace || ((uintptr_t)workspace & 15) != 0) return fail(SPA_EINVAL, "%s: the key split needs a 16-byte aligned workspace", what);
-    const KeySplit ks(Sk, nsplit);
+    const KeySplit ks(Sk, workspace_call ? nsplit : 1);
+    const bool can = !p.causal && dtype != SPA_F32 && D != 32 && !p.big;
     if (ks.n > 1) {
-      char* part_out = (char*)workspace;
-      float* part_lse = (float*)(part_out + splitkv_out_bytes(B, H, Sq, D, nsplit, esz));
+      if (p.causal) return fail(SPA_EUNSUPPORTED, "%s: the keys are split for calls without a mask", what);
+      if (!can) return fail(SPA_EUNSUPPORTED, "%s: built for bf16 / fp16, head dim 64 or 128, K/V below 2 GiB per (batch, head)", what);
+      if (!workspace || ((uintptr_t)workspace & 15) != 0) return fail(SPA_EINVAL, "%s: the key split needs a 16-byte aligned workspace", what);
+    }
+    // Up to kFewRows query rows without a mask, split or not: the kernel that streams K and V past them (16 bytes a lane,
+    // so e4m3 rows must be 16-byte aligned as well); more rows, or spa_tune(SPA_TUNE_FEW_ROWS, 1): the MFMA kernels (for a
+    // split with the chunks as grid planes).
+    const bool few = can && Sq <= kFewRows && spa_knob(SPA_KNOB_FEW_ROWS) != 1 &&
+                     (!kv8 || (aligned16(k, k_strides, 1) && aligned16(v, v_strides, 1)));
+    if (ks.n > 1 || few) {
       p.Sk = ks.chunk; p.sk_last = ks.last;
       p.P = ks.n; p.rank0 = 0; p.nranks = ks.n; p.t_begin = 0; p.t_count = 1;
-      // plane z writes rows z * Sq .. of the scratch tensors [B, n * Sq, H, D] and [B, H, n * Sq]
-      p.out = part_out; p.lse = part_lse;
-      p.os.b = (int64_t)ks.n * Sq * H * D; p.os.s = (int64_t)H * D; p.os.h = D;
-      p.lse_bh = (int64_t)ks.n * Sq;
-      hipError_t e = spa_launch_fwd16_splitkv(p, D, dtype, (hipStream_t)stream);
-      if (e == hipSuccess)
+      char* part_out = (char*)workspace;
+      float* part_lse = ks.n > 1 ? (float*)(part_out + splitkv_out_bytes(B, H, Sq, D, nsplit, esz)) : nullptr;
+      if (ks.n > 1) {
+        // plane z writes rows z * Sq .. of the scratch tensors [B, n * Sq, H, D] and [B, H, n * Sq]
+        p.out = part_out; p.lse = part_lse;
+        p.os.b = (int64_t)ks.n * Sq * H * D; p.os.s = (int64_t)H * D; p.os.h = D;
+        p.lse_bh = (int64_t)ks.n * Sq;
+      }
+      hipError_t e = few ? spa_launch_fwd_fewrows(p, D, dtype, (hipStream_t)stream) : spa_launch_fwd16_splitkv(p, D, dtype, (hipStream_t)stream);
+      if (e == hipSuccess && ks.n > 1)
         e = spa_launch_splitkv_combine(out, lse, part_out, part_lse, ks.n, B, H, Sq, D, S3(o_strides), Sq, dtype, (hipStream_t)stream);
       return launch_result(e, what);
     }
@@ -234,11 +248,20 @@ int64_t spa_flash_fwd_splitkv_workspace_bytes(int B, int H, int Sq, int D, int n
 int spa_flash_fwd_splitkv_suggest(int B, int H, int Sq, int Sk, int D, int mask_mode, int dtype) {
   if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0 || mask_mode != SPA_MASK_NONE || (dtype != SPA_BF16 && dtype != SPA_F16) || (D != 64 && D != 128))
     return 1;
-  // Worth it when the 128-row workgroups of the plain launch leave at least half of the CUs idle and every chunk keeps at
-  // least 512 keys: as many chunks as give every CU one workgroup (measured on six decode shapes: more chunks only add
-  // the workgroups' fixed cost and rows for the merge).
-  const int64_t wgs = (int64_t)B * H * ((Sq + 127) / 128);
   const int cus = spa_device_cus();
+  // Up to kFewRows query rows run on the kernel that streams K and V: one workgroup per CU measured best on ten decode
+  // shapes (more chunks: 3 to 15 % slower), chunks of at least 512 keys.
+  if (Sq <= kFewRows && spa_knob(SPA_KNOB_FEW_ROWS) != 1) {
+    if (Sk < 1024) return 1;
+    int64_t n = ((int64_t)cus + (int64_t)B * H / 2) / ((int64_t)B * H);
+    if (n > Sk / 512) n = Sk / 512;
+    if (n > 64) n = 64;
+    return n < 2 ? 1 : KeySplit(Sk, (int)n).n;
+  }
+  // Otherwise worth it when the 128-row workgroups of the plain launch leave at least half of the CUs idle and every
+  // chunk keeps at least 512 keys: as many chunks as give every CU one workgroup (measured on six decode shapes: more
+  // chunks only add the workgroups' fixed cost and rows for the merge).
+  const int64_t wgs = (int64_t)B * H * ((Sq + 127) / 128);
   if (wgs * 2 > cus || Sk < 2048) return 1;
   int64_t n = ((int64_t)cus + wgs / 2) / wgs;
   if (n > Sk / 512) n = Sk / 512;

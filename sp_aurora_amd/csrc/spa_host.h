@@ -16,7 +16,8 @@ enum {
   SPA_KNOB_BWD_DQ_WAVES = 2,  // 4 | 8 waves per workgroup of the backward's dq kernel
   SPA_KNOB_BWD_DKDV_FORM = 3, // 1: compiler-scheduled MFMAs in the D = 128 dk/dv kernel (test twin)
   SPA_KNOB_FWD32_SPLIT = 4,   // 1: never the 32-row fp32 forward whose waves share the key tiles, 2: whenever D <= 64
-  SPA_KNOB_COUNT = 5
+  SPA_KNOB_FEW_ROWS = 5,     // 1: a key-split forward of up to 4 query rows stays on the MFMA kernels
+  SPA_KNOB_COUNT = 6
 };
 extern std::atomic<int> g_spa_knob[SPA_KNOB_COUNT];
 static inline int spa_knob(int k) { return g_spa_knob[k].load(std::memory_order_relaxed); }

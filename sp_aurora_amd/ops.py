@@ -134,7 +134,8 @@ def flash_fwd(q, k, v, softmax_scale=None, causal=False, layout="bshd", out=None
     cache) the keys are cut into chunks that run side by side (spa_flash_fwd_splitkv[_fp8kv]): "auto" = as many as
     the library suggests, an int = that many, None or 1 = never.  The chunks' results wait in `workspace` (a uint8 tensor
     of flash_fwd_splitkv_workspace(...) bytes; allocated here when not given, except while the stream is being captured,
-    where "auto" then does not split)."""
+    where "auto" then does not split).  With up to three query rows and no mask the library runs a kernel that streams K and V
+    past the rows instead of the matrix-instruction kernel, split or not."""
     lib = _lib.load()
     fp8 = k.dtype == FP8 or v.dtype == FP8
     if q.dtype == FP8:

@@ -54,6 +54,7 @@ def _case(rng):
     _lib.tune("fwd_share", share)
     _lib.tune("fwd_groups", groups)
     _lib.tune("fwd32_split", rng.choice([0, 0, 1, 2]))
+    _lib.tune("few_rows", rng.choice([0, 0, 1]))   # up to three unmasked query rows: the streaming kernel, or the MFMA kernels
     g = torch.Generator().manual_seed(rng.randrange(1 << 30))
     mk = lambda *shape, dt=None: torch.randn(shape, generator=g).to(dt or dtype)
     atol, rtol = OUT_TOL[dtype]
@@ -61,7 +62,7 @@ def _case(rng):
         return
     if kind == "fp8_qkv":  # e4m3 q as well: scores on the 8-bit matrix instruction, D = 128
         dt = rng.choice([torch.bfloat16, torch.float16])
-        Sq, Sk = rng.choice([1, 64, 100, 128, 256, 300, 513]), rng.choice([1, 64, 65, 128, 200, 513, 769])
+        Sq, Sk = rng.choice([1, 3, 64, 100, 128, 256, 300, 513]), rng.choice([1, 64, 65, 128, 200, 513, 769])
         info = (kind, dt, B, H, Sq, Sk, causal, share, groups)
         qf, kf, vf = (mk(B, H, n_, 128, dt=torch.float32) for n_ in (Sq, Sk, Sk))
         (q8, qs), (k8, ks), (v8, vs) = (ops.quantize_fp8_per_head(t, "bhsd") for t in (qf, kf, vf))
@@ -86,7 +87,7 @@ def _case(rng):
         assert not flags.failed(), info
         return
     if kind == "block":
-        Sq = rng.choice([1, 7, 64, 65, 127, 128, 129, 200, 256, 300, 513, 700])
+        Sq = rng.choice([1, 2, 3, 7, 64, 65, 127, 128, 129, 200, 256, 300, 513, 700])
         Sk = rng.choice([1, 3, 64, 65, 128, 130, 255, 256, 400, 769])
         split = rng.choice(["auto", "auto", 2, 3, 5])   # keys cut into chunks that run side by side (calls without a mask, 16-bit, D >= 64)
         info = (kind, dtype, B, H, Sq, Sk, D, causal, share, groups, split)
@@ -200,3 +201,4 @@ def test_fixed_seed_sweep_of_random_shapes_against_the_oracle():
         _lib.tune("fwd_share", 0)
         _lib.tune("fwd_groups", 0)
         _lib.tune("fwd32_split", 0)
+        _lib.tune("few_rows", 0)

@@ -19,6 +19,12 @@ CASES = [
     (1, 2, 130, 1025, 64, torch.bfloat16, 8),       # two query tiles; 1025 keys: eight chunks of 256 would not do, 128-key chunks: 9 -> fewer planes
     (3, 1, 5, 700, 128, torch.float16, 2),          # the second chunk 316 keys
     (1, 2, 64, 200, 64, torch.bfloat16, 4),         # 200 keys: chunks of 128 -> two planes
+    # up to four query rows: the kernel that streams K and V past them
+    (2, 3, 1, 3000, 128, torch.float16, 6),         # chunks of 512, the last one 440 keys
+    (1, 5, 2, 777, 64, torch.bfloat16, 3),          # chunks of 384: a wave's eight loads reach past the chunk's end
+    (2, 2, 3, 1300, 128, torch.bfloat16, 1),        # one chunk: no workspace, written in place
+    (1, 3, 4, 130, 64, torch.float16, 2),           # the second chunk two keys: three of its waves see none
+    (1, 2, 4, 5, 128, torch.bfloat16, 1),           # five keys
 ]
 
 
@@ -60,11 +66,34 @@ def test_key_split_with_e4m3_cache():
         check_lse(lse, want_l)
 
 
+@pytest.mark.parametrize("D,Sq", [(64, 1), (64, 4), (128, 2)])
+def test_few_rows_with_e4m3_cache_against_the_mfma_kernel(D, Sq):
+    """The streaming kernel and the MFMA kernel on the same chunks (spa_tune few_rows = 1 keeps the latter), e4m3 K/V."""
+    B, H, Sk = 2, 3, 2500
+    from test_gpu_fp8kv import quantised
+    q = rand((B, Sq, H, D), 1030, torch.float16)
+    k8, ksc, k_deq = quantised((B, Sk, H, D), 1031, "bshd", spread=1.2)
+    v8, vsc, v_deq = quantised((B, Sk, H, D), 1032, "bshd")
+    want_o, want_l = O.full_attention(q, k_deq, v_deq, 0.2, False)
+    got = {}
+    try:
+        for knob in (0, 1):
+            _lib.tune("few_rows", knob)
+            for nsplit in (1, 4):
+                out, lse = ops.flash_fwd(q.to(DEV), k8.to(DEV), v8.to(DEV), 0.2, False, k_scale=ksc, v_scale=vsc, split_kv=nsplit)
+                check_out(out, want_o, torch.float16, f"e4m3 few rows knob {knob} split {nsplit}")
+                check_lse(lse, want_l)
+                got[knob, nsplit] = (out, lse)
+    finally:
+        _lib.tune("few_rows", 0)
+    assert (got[0, 4][1] - got[1, 4][1]).abs().max().item() < 1e-4
+
+
 def test_the_librarys_choice_and_what_is_refused():
     lib = _lib.load()
     sug = lambda B, H, Sq, Sk, D, mask=0, dt=_lib.SPA_BF16: lib.spa_flash_fwd_splitkv_suggest(B, H, Sq, Sk, D, mask, dt)
     assert sug(1, 32, 1, 32768, 128) > 1               # 32 workgroups on 256 CUs
-    assert sug(1, 32, 1, 1024, 128) == 1               # too few keys to cut
+    assert sug(1, 32, 8, 1024, 128) == 1 and sug(1, 32, 1, 512, 128) == 1   # too few keys to cut
     assert sug(1, 32, 8192, 8192, 128) == 1            # enough workgroups as it is
     assert sug(1, 32, 1, 32768, 128, mask=1) == 1      # causal
     assert sug(1, 32, 1, 32768, 32) == 1 and sug(1, 32, 1, 32768, 128, dt=_lib.SPA_F32) == 1
