@@ -372,13 +372,15 @@ ROW_SPECS = {
 # Rows that `--workload` can print and the default line leaves out (the line is short of room).
 EXTRA_ROW_NOTES = {
     "decode_key_split": "a decode step against a long cache: bf16 q [1,1,32,128] (one new token) x K, V [1,32768,32,128], no mask; the keys "
-                        "are cut into chunks that run side by side (spa_flash_fwd_splitkv, as many as the library suggests); value = K and V "
-                        "bytes per call time; plain_gbps = the same call as one launch of 32 workgroups (spa_flash_fwd); e4m3_gbps = the "
-                        "split call on an e4m3 cache (half the bytes per key); q128_tflops = the split call with 128 query rows",
+                        "are cut into chunks that run side by side (spa_flash_fwd_splitkv, as many as the library suggests) on the kernel "
+                        "that streams K and V past up to three query rows; value = K and V bytes per call time; plain_gbps = the same call "
+                        "as one launch of 32 workgroups (spa_flash_fwd); mfma_gbps = the split call on the matrix-instruction kernels "
+                        "(spa_tune few_rows = 1); e4m3_gbps / e4m3_mfma_gbps = the two on an e4m3 cache (half the bytes per key); "
+                        "q128_tflops = the split call with 128 query rows",
 }
 EXTRA_ROW_SPECS = {
-    "decode_key_split": ("decode: q [1,1,32,128] x K/V [1,32768,32,128] bf16, keys split", "GB/s", "hbm", "flash_fwd16<bf16,128,split keys>",
-                         HBM_PEAK_GBPS, ("plain_gbps", "e4m3_gbps", "q128_tflops", "chunks")),
+    "decode_key_split": ("decode: q [1,1,32,128] x K/V [1,32768,32,128] bf16, keys split", "GB/s", "hbm", "fewrows_fwd<bf16,128,1 row>",
+                         HBM_PEAK_GBPS, ("plain_gbps", "mfma_gbps", "e4m3_gbps", "e4m3_mfma_gbps", "q128_tflops", "chunks")),
 }
 
 
@@ -576,10 +578,17 @@ def gpu_rows(torch, spa, ops, which, steps, warmup):
             f_split = lambda: ops.flash_fwd(q, k, v, None, False, out=out, lse=lse, split_kv=n, workspace=ws)
             f_plain = lambda: ops.flash_fwd(q, k, v, None, False, out=out, lse=lse, split_kv=None)
             f_e4m3 = lambda: ops.flash_fwd(q, k8, v8, None, False, out=out, lse=lse, k_scale=ksc, v_scale=vsc, split_kv=n, workspace=ws)
-            res[sq] = (n, measure(torch, f_split, 20, 5, **light), measure(torch, f_plain, 20, 5, **light), measure(torch, f_e4m3, 20, 5, **light))
-        n1, m_split, m_plain, m_e4 = res[1]
+            res[sq] = [n, measure(torch, f_split, 20, 5, **light), measure(torch, f_plain, 20, 5, **light), measure(torch, f_e4m3, 20, 5, **light)]
+            if sq == 1:
+                _lib_mod().tune("few_rows", 1)
+                try:
+                    res[sq] += [measure(torch, f_split, 20, 5, **light), measure(torch, f_e4m3, 20, 5, **light)]
+                finally:
+                    _lib_mod().tune("few_rows", 0)
+        n1, m_split, m_plain, m_e4, m_mfma, m_e4_mfma = res[1]
         gbps = lambda nbytes, m: nbytes / (m["ms_per_step"] * 1e-3) / 1e9
-        finish("decode_key_split", m_split, gbps(kv_bytes, m_split), plain_gbps=gbps(kv_bytes, m_plain), e4m3_gbps=gbps(kv_bytes / 2, m_e4),
+        finish("decode_key_split", m_split, gbps(kv_bytes, m_split), plain_gbps=gbps(kv_bytes, m_plain), mfma_gbps=gbps(kv_bytes, m_mfma),
+               e4m3_gbps=gbps(kv_bytes / 2, m_e4), e4m3_mfma_gbps=gbps(kv_bytes / 2, m_e4_mfma),
                q128_tflops=tfl(4.0 * Bn * Hn * 128 * Skn * Dn, res[128][1]), chunks=n1)
         del k, v, k8, v8
     if "config5" in which:

@@ -111,6 +111,9 @@ int spa_flash_fwd_fp8kv(const void* q, const void* k8, const void* v8,
  * nsplit = 1 is spa_flash_fwd.  Chunks hold a multiple of 128 keys, so fewer than nsplit may run.  bf16 / fp16, D in
  * {64, 128}, mask none, K/V below 2 GiB per (batch, head).  workspace: spa_flash_fwd_splitkv_workspace_bytes() bytes, 16-byte
  * aligned, the caller's.  _fp8kv: K / V as e4m3 bytes with scales, as for spa_flash_fwd_fp8kv.
+ * With up to three query rows (and no mask, the same types and sizes; e4m3 K/V rows 16-byte aligned) these entry points and
+ * spa_flash_fwd / spa_flash_fwd_fp8kv run a kernel without matrix instructions that streams K and V past the rows at the
+ * rate of HBM (a 128-row tile would hold one to three live rows); spa_tune(SPA_TUNE_FEW_ROWS, 1) keeps the other kernels.
  */
 int64_t spa_flash_fwd_splitkv_workspace_bytes(int B, int H, int Sq, int D, int nsplit, int dtype);
 int spa_flash_fwd_splitkv_suggest(int B, int H, int Sq, int Sk, int D, int mask_mode, int dtype);
