@@ -764,7 +764,8 @@ def pmc_summary_rows(fetch_dir, write_dir):
     WRITE_SIZE per dispatch, each scaled by the calibration copy of the same run."""
     kernels = {"config4_relayout_s2h": ("relayout_kernel<16, true>", 268435456),
                "config4_relayout_h2s": ("relayout_kernel<16, false>", 268435456),
-               "merge_update_out_and_lse": ("merge_kernelIDF16bLb0E", 42336256)}  # (the profiler leaves bf16 names mangled)
+               "merge_update_out_and_lse": ("merge_kernelIDF16bLb0E", 42336256),  # (the profiler leaves bf16 names mangled)
+               "decode_key_split": ("fewrows_fwd_kernelIDF16bLi128ELb0ELi1E", 2 * 32768 * 32 * 128 * 2)}  # K and V once
 
     def read(d, counter):
         files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
@@ -800,7 +801,7 @@ def pmc_summary_rows(fetch_dir, write_dir):
 
 # ------------------------------------------------------------------------------------ main
 ROW_SETS = {"fp8kv": {"fp8kv"}, "relayout": {"config4"}, "ulysses": {"config4"}, "merge": {"merge"}, "backward": {"config5"},
-            "config1": {"config1"}, "config2": {"config2"}, "zigzag": {"zigzag"}, "hbm": {"config4", "merge"}, "decode": {"decode"}}
+            "config1": {"config1"}, "config2": {"config2"}, "zigzag": {"zigzag"}, "hbm": {"config4", "merge", "decode"}, "decode": {"decode"}}
 ALL_ROWS = {"config1", "config2", "zigzag", "config4", "fp8kv", "merge", "config5"}
 LINE_LIMIT = 7500  # bytes of the printed line: readers that keep only the end of the output keep 8 KB
 
