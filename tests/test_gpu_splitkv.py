@@ -112,10 +112,11 @@ def test_the_librarys_choice_and_what_is_refused():
         ops.flash_fwd(q, k, k, layout="bhsd", split_kv=8, workspace=ws)                # a workspace for four chunks
 
 
-def test_key_split_replays_from_a_captured_graph():
+@pytest.mark.parametrize("Sq", [2, 4])   # the kernel that streams K and V; the matrix-instruction kernel
+def test_key_split_replays_from_a_captured_graph(Sq):
     """Two launches and a caller's workspace, nothing allocated, no synchronisation: the call can be captured; every replay
     (with eager work in between and new values in the captured buffers) equals the eager result."""
-    B, H, Sq, Sk, D, n = 1, 8, 4, 4096, 128, 6
+    B, H, Sk, D, n = 1, 8, 4096, 128, 6
     q, k, v = (rand((B, s_, H, D), 1030 + i, torch.bfloat16).to(DEV) for i, s_ in enumerate((Sq, Sk, Sk)))
     ws = ops.flash_fwd_splitkv_workspace(q, n)
     out, lse = torch.empty_like(q), torch.empty((B, H, Sq), dtype=torch.float32, device=DEV)
