@@ -765,7 +765,7 @@ def pmc_summary_rows(fetch_dir, write_dir):
     kernels = {"config4_relayout_s2h": ("relayout_kernel<16, true>", 268435456),
                "config4_relayout_h2s": ("relayout_kernel<16, false>", 268435456),
                "merge_update_out_and_lse": ("merge_kernelIDF16bLb0E", 42336256),  # (the profiler leaves bf16 names mangled)
-               "decode_key_split": ("fewrows_fwd_kernelIDF16bLi128ELb0ELi1E", 2 * 32768 * 32 * 128 * 2)}  # K and V once
+               "decode_key_split": ("fewrows_fwd_kernelIDF16bLi128ELb0ELi1ELi4ELb1E", 2 * 32768 * 32 * 128 * 2)}  # K and V once
 
     def read(d, counter):
         files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)

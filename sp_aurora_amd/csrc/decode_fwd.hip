@@ -17,7 +17,6 @@
 namespace {
 
 constexpr int kWaves = 4;    // waves per workgroup
-constexpr int kUnroll = 8;   // loads of K (and of V) a wave keeps in flight
 
 template <int CTRL>
 static __device__ __forceinline__ float dpp_add(float x) {
@@ -58,8 +57,11 @@ struct Piece<T, true> {
   }
 };
 
-template <typename T, int D, bool KV8, int NQ>
+// kUnroll: loads of K (and of V) a wave keeps in flight.  NT: the loads carry the non-temporal hint (K and V are read
+// once and should not displace anything in the caches).
+template <typename T, int D, bool KV8, int NQ, int kUnroll, bool NT>
 __global__ void __launch_bounds__(kWaves * 64) fewrows_fwd_kernel(const FwdParams p) {
+  constexpr int AUX = NT ? 2 : 0;
   typedef Piece<T, KV8> Pc;
   constexpr int E = Pc::E;
   constexpr int LPR = D / E;        // lanes per key row
@@ -120,12 +122,12 @@ __global__ void __launch_bounds__(kWaves * 64) fewrows_fwd_kernel(const FwdParam
   auto load_k = [&](int row0) {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
-      kx[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(krs, (unsigned)((row0 + u * R) * krow_b) + kcol, 0, 0));
+      kx[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(krs, (unsigned)((row0 + u * R) * krow_b) + kcol, 0, AUX));
   };
   auto load_v = [&](int row0) {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
-      vx[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(vrs, (unsigned)((row0 + u * R) * vrow_b) + vcol, 0, 0));
+      vx[u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(vrs, (unsigned)((row0 + u * R) * vrow_b) + vcol, 0, AUX));
   };
   constexpr int kPass = kWaves * kUnroll * R;   // key rows the workgroup takes per pass
   const int first = k0 + wave * (kUnroll * R);
@@ -228,16 +230,43 @@ __global__ void __launch_bounds__(kWaves * 64) fewrows_fwd_kernel(const FwdParam
   }
 }
 
-template <typename T, int D, bool KV8>
-hipError_t launch_nq(const FwdParams& p, hipStream_t stream) {
+// Measured on twelve decode shapes: four loads in flight beat eight (6-10 %) except with three rows and with 64-byte
+// rows; the non-temporal hint gains 5-15 % on 16-bit K/V and on e4m3 rows of a whole line when the keys are not split,
+// and loses where neighbouring workgroups share lines (64-byte rows) and on split e4m3 calls.
+template <typename T, int D, bool KV8, int NQ, int U>
+hipError_t launch_variant(const FwdParams& p, hipStream_t stream) {
   const dim3 grid((unsigned)(p.B * p.H), (unsigned)p.P), block(kWaves * 64);
-  switch (p.Sq) {
-    case 1: hipLaunchKernelGGL((fewrows_fwd_kernel<T, D, KV8, 1>), grid, block, 0, stream, p); break;
-    case 2: hipLaunchKernelGGL((fewrows_fwd_kernel<T, D, KV8, 2>), grid, block, 0, stream, p); break;
-    case 3: hipLaunchKernelGGL((fewrows_fwd_kernel<T, D, KV8, 3>), grid, block, 0, stream, p); break;
-    default: return hipErrorInvalidValue;
+  if constexpr (!KV8) {
+    hipLaunchKernelGGL((fewrows_fwd_kernel<T, D, KV8, NQ, U, true>), grid, block, 0, stream, p);
+  } else if constexpr (D == 64) {
+    hipLaunchKernelGGL((fewrows_fwd_kernel<T, D, KV8, NQ, U, false>), grid, block, 0, stream, p);
+  } else if (p.P == 1) {
+    hipLaunchKernelGGL((fewrows_fwd_kernel<T, D, KV8, NQ, U, true>), grid, block, 0, stream, p);
+  } else {
+    hipLaunchKernelGGL((fewrows_fwd_kernel<T, D, KV8, NQ, U, false>), grid, block, 0, stream, p);
   }
   return hipGetLastError();
+}
+
+// A launch that leaves half of the CUs without a workgroup (a caller who did not split the keys) is bound by what its
+// few waves keep in flight: eight loads there too.
+template <typename T, int D, bool KV8, int NQ>
+hipError_t launch_unroll(const FwdParams& p, hipStream_t stream) {
+  constexpr int U = NQ == 3 || (KV8 && D == 64) ? 8 : 4;
+  if constexpr (U != 8) {
+    if ((int64_t)p.B * p.H * p.P * 2 <= spa_device_cus()) return launch_variant<T, D, KV8, NQ, 8>(p, stream);
+  }
+  return launch_variant<T, D, KV8, NQ, U>(p, stream);
+}
+
+template <typename T, int D, bool KV8>
+hipError_t launch_nq(const FwdParams& p, hipStream_t stream) {
+  switch (p.Sq) {
+    case 1: return launch_unroll<T, D, KV8, 1>(p, stream);
+    case 2: return launch_unroll<T, D, KV8, 2>(p, stream);
+    case 3: return launch_unroll<T, D, KV8, 3>(p, stream);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 template <typename T>
