@@ -392,6 +392,8 @@ int spa_flash_bwd_out(const void* q, const void* k, const void* v, const void* d
  * max_seqlen, ...) in test/flash_attention/test_intel_ring_flash_attn_varlen.py:23-26,66-74
  * (the function itself is missing from the reference), and the packed lse
  * layout of flatten_varlen_lse (sp_aurora/utils.py:150-157).
+ * With max_sq <= 3 and no mask (a decode step of a batch whose caches differ in length; bf16 / fp16, D in {64, 128}) the call
+ * runs on the kernel that streams each sequence's K and V past its rows, as spa_flash_fwd does (also _fp8kv).
  */
 int spa_flash_fwd_varlen(const void* q, const void* k, const void* v, void* out, float* lse,
                          const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,

@@ -77,17 +77,43 @@ __global__ void __launch_bounds__(kWaves * 64) fewrows_fwd_kernel(const FwdParam
   int bh = blockIdx.x;
   if (D * KESZ < 128 && (gridDim.x & 7) == 0) bh = (bh & 7) * (int)(gridDim.x >> 3) + (bh >> 3);
   const int z = blockIdx.y;
-  const int b = bh / p.H, h = bh - b * p.H;
+  int b = bh / p.H;
+  const int h = bh - b * p.H;
   const int c = lane % LPR, g = lane / LPR;
-  const int k0 = z * p.Sk;
-  const int k1 = k0 + (z == p.P - 1 ? p.sk_last : p.Sk);
+  int k0 = z * p.Sk;
+  int k1 = k0 + (z == p.P - 1 ? p.sk_last : p.Sk);
+  int nq = NQ;                                   // rows of this (batch or sequence, head) that exist
+  int64_t q_row0 = 0, k_row0 = 0;                // first row of the sequence in the packed tensors
+  int64_t lse_base = (int64_t)bh * p.lse_bh;     // lse is [B, H, rows], or [H, packed rows] for a packed batch
+  if (p.cu_q) {
+    // a packed variable-length batch: sequence b owns rows cu_q[b] .. of q / out / lse and cu_k[b] .. of K / V
+    // (one chunk: the keys of such a batch are not split)
+    q_row0 = p.cu_q[b];
+    k_row0 = p.cu_k[b];
+    nq = p.cu_q[b + 1] - (int)q_row0;
+    nq = nq < NQ ? nq : NQ;
+    k0 = 0;
+    k1 = p.cu_k[b + 1] - (int)k_row0;
+    lse_base = (int64_t)h * p.lse_bh + q_row0;
+    b = 0;
+    if (nq <= 0) return;
+    if (k1 <= 0) {
+      // no keys: the empty sum, out = 0 and lse = -inf
+      for (int t = threadIdx.x; t < nq * D; t += kWaves * 64) {
+        const int i = t / D, d = t - i * D;
+        ((T*)p.out)[h * p.os.h + (q_row0 + i) * p.os.s + d] = (T)0.f;
+        if (d == 0) p.lse[lse_base + i] = -INFINITY;
+      }
+      return;
+    }
+  }
 
   // the rows' queries, this lane's elements, scaled into the exponent's base-2 domain
   const float qmul = (p.negq ? -p.scale_log2 : p.scale_log2) * (KV8 ? p.k_scale[bh] : 1.f);
   float qf[NQ][E];
 #pragma unroll
   for (int i = 0; i < NQ; ++i) {
-    const T* qp = (const T*)p.q + b * p.qs.b + h * p.qs.h + (int64_t)i * p.qs.s + c * E;
+    const T* qp = (const T*)p.q + b * p.qs.b + h * p.qs.h + (q_row0 + (i < nq ? i : nq - 1)) * p.qs.s + c * E;
 #pragma unroll
     for (int e0 = 0; e0 < E; e0 += 8) {
       float t[8];
@@ -99,8 +125,8 @@ __global__ void __launch_bounds__(kWaves * 64) fewrows_fwd_kernel(const FwdParam
 
   // descriptors that end with this chunk's last row: rows past it read as zero and are masked below
   const int64_t krow_b = p.ks.s * KESZ, vrow_b = p.vs.s * KESZ;
-  const char* kp = (const char*)p.k + (b * p.ks.b + h * p.ks.h) * KESZ;
-  const char* vp = (const char*)p.v + (b * p.vs.b + h * p.vs.h) * KESZ;
+  const char* kp = (const char*)p.k + (b * p.ks.b + h * p.ks.h + k_row0 * p.ks.s) * KESZ;
+  const char* vp = (const char*)p.v + (b * p.vs.b + h * p.vs.h + k_row0 * p.vs.s) * KESZ;
   const __amdgpu_buffer_rsrc_t krs =
       __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, (int)((unsigned)((int64_t)(k1 - 1) * krow_b) + D * KESZ), 0x00020000);
   const __amdgpu_buffer_rsrc_t vrs =
@@ -223,10 +249,11 @@ __global__ void __launch_bounds__(kWaves * 64) fewrows_fwd_kernel(const FwdParam
       ls += sm_l[i][w] * f;
       a += sm_acc[i][w][d] * f;
     }
+    if (i >= nq) break;
     const int64_t orow = (int64_t)z * p.Sq + i;
-    T* op = (T*)p.out + b * p.os.b + h * p.os.h + orow * p.os.s;
+    T* op = (T*)p.out + b * p.os.b + h * p.os.h + (q_row0 + orow) * p.os.s;
     op[d] = (T)(a * vmul / ls);
-    if (d == 0) p.lse[(int64_t)bh * p.lse_bh + orow] = (mx + __builtin_amdgcn_logf(ls)) * 0.6931471805599453f;
+    if (d == 0) p.lse[lse_base + orow] = (mx + __builtin_amdgcn_logf(ls)) * 0.6931471805599453f;
   }
 }
 
@@ -281,9 +308,10 @@ hipError_t launch_t(const FwdParams& p, int D, hipStream_t stream) {
 
 // The caller's FwdParams as for the key-split launch: Sk = keys per chunk, sk_last = keys of the last chunk, P = number of
 // chunks; out / lse take rows z * Sq + i of chunk z.  No mask, 1 <= Sq <= 3, 16-bit q / out, K/V of one
-// (batch, head) below 2 GiB, 16-byte aligned K/V rows.
+// (batch, head) below 2 GiB, 16-byte aligned K/V rows.  A packed variable-length batch (cu_q, cu_k; Sq = the longest
+// sequence's rows, B = sequences) runs as one chunk.
 hipError_t spa_launch_fwd_fewrows(FwdParams p, int D, int dtype, hipStream_t stream) {
-  if (p.causal || p.cu_q || p.q_scale || p.big || p.Sq < 1 || p.Sq > 3 || p.P < 1 || p.P > 65535) return hipErrorInvalidValue;
+  if (p.causal || (p.cu_q && p.P != 1) || p.q_scale || p.big || p.Sq < 1 || p.Sq > 3 || p.P < 1 || p.P > 65535) return hipErrorInvalidValue;
   if (dtype == 1) return launch_t<__bf16>(p, D, stream);
   if (dtype == 2) return launch_t<_Float16>(p, D, stream);
   return hipErrorInvalidValue;

@@ -856,6 +856,13 @@ int flash_fwd_varlen(const char* what, const void* q, const void* k, const void*
   p.P = 1; p.rank0 = 0; p.nranks = 1; p.t_begin = 0; p.t_count = -1;
   p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k;
   p.k_scale = k_scale; p.v_scale = v_scale;
+  // Sequences of up to kFewRows query rows without a mask (a decode step of a batch with ragged caches): the kernel that
+  // streams each sequence's K and V past its rows, as in flash_fwd above.
+  if (P == 1 && !p.causal && dtype != SPA_F32 && D != 32 && !p.big && max_sq <= kFewRows && spa_knob(SPA_KNOB_FEW_ROWS) != 1 &&
+      (!kv8 || (aligned16v(k, k_strides, 1) && aligned16v(v, v_strides, 1)))) {
+    p.sk_last = max_sk;
+    return launch_result(spa_launch_fwd_fewrows(p, D, dtype, (hipStream_t)stream), what);
+  }
   if (P > 1) {
     p.P = P; p.chunk_rows = total_k; p.rank_rows = total_q;
     const int r_lo = rank < 0 ? 0 : rank, r_hi = rank < 0 ? P : rank + 1;

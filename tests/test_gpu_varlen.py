@@ -145,6 +145,57 @@ def test_varlen_backward_written_in_the_inputs_type_equals_accumulate_then_cast(
                                  dk=torch.empty_like(k[:1]))
 
 
+DECODE_CASES = [
+    # query rows per sequence, keys per sequence, H, D, dtype
+    ([1, 1, 1, 1, 1], [700, 1, 33, 1300, 64], 4, 128, torch.bfloat16),     # one new token per sequence, ragged caches
+    ([1, 3, 0, 2, 1], [100, 515, 40, 0, 257], 3, 64, torch.float16),       # a sequence without queries, one without keys
+    ([2, 2, 2], [4096, 5, 130], 2, 128, torch.float16),
+    ([3, 1], [70, 900], 5, 64, torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("lens_q,lens_k,H,D,dtype", DECODE_CASES)
+def test_varlen_few_query_rows_against_ragged_caches(lens_q, lens_k, H, D, dtype):
+    """Sequences of up to three query rows without a mask run on the kernel that streams K and V (spa_tune few_rows = 1:
+    the matrix-instruction kernels); both against the oracle's attention of each sequence alone, bf16 / fp16 and e4m3 K/V."""
+    from sp_aurora_amd import _lib
+    Tq, Tk = sum(lens_q), sum(lens_k)
+    q, k, v = rand((Tq, H, D), 470, dtype), rand((Tk, H, D), 471, dtype), rand((Tk, H, D), 472, dtype)
+    want_out, want_lse = per_sequence(q, k, v, lens_q, lens_k, False)
+    cq, ck = cu_of(lens_q).to(DEV), cu_of(lens_k).to(DEV)
+    k8, ksc = ops.quantize_fp8_per_head(k[None].float())
+    v8, vsc = ops.quantize_fp8_per_head(v[None].float())
+    nseq = len(lens_q)
+    ksc, vsc = ksc.expand(nseq, H).contiguous(), vsc.expand(nseq, H).contiguous()   # one scale per head for every sequence
+    k_deq = (k8[0].float() * ksc[0][None, :, None]).to(dtype)
+    v_deq = (v8[0].float() * vsc[0][None, :, None]).to(dtype)
+    want8_out, want8_lse = per_sequence(q, k_deq, v_deq, lens_q, lens_k, False)
+
+    def lse_ok(got_lse, want):   # (a sequence without keys: lse = -inf)
+        got_lse, fin = got_lse.cpu().double(), torch.isfinite(want)
+        assert torch.equal(torch.isneginf(got_lse), torch.isneginf(want))
+        assert (got_lse[fin] - want[fin]).abs().max() <= 1e-3
+
+    got = {}
+    try:
+        for knob in (0, 1):
+            _lib.tune("few_rows", knob)
+            out = torch.full((Tq, H, D), 7.0, dtype=dtype, device=DEV)
+            lse = torch.full((H, Tq), 7.0, dtype=torch.float32, device=DEV)
+            ops.flash_fwd_varlen(q.to(DEV), k.to(DEV), v.to(DEV), cq, ck, max(lens_q), max(lens_k), None, False, out=out, lse=lse)
+            check_out(out, want_out, dtype, f"knob {knob}")
+            lse_ok(lse, want_lse)
+            got[knob] = lse
+            o8, l8 = ops.flash_fwd_varlen(q.to(DEV), k8[0].to(DEV), v8[0].to(DEV), cq, ck, max(lens_q), max(lens_k), None, False,
+                                          k_scale=ksc.to(DEV), v_scale=vsc.to(DEV))
+            check_out(o8, want8_out, dtype, f"e4m3 knob {knob}")
+            lse_ok(l8, want8_lse)
+    finally:
+        _lib.tune("few_rows", 0)
+    both = torch.isfinite(got[0]) & torch.isfinite(got[1])
+    assert torch.equal(torch.isfinite(got[0]), torch.isfinite(got[1])) and (got[0][both] - got[1][both]).abs().max().item() < 1e-4
+
+
 def test_varlen_large_batch_matches_the_fixed_length_kernels():
     """Enough workgroups for the shared-buffer forward variant; equal lengths make the padded
     batch call a second opinion, the ragged tail a check that short sequences leave their
