@@ -343,3 +343,41 @@ def test_decode_step_against_a_long_cache_with_the_keys_split():
             ro, rl = ref_head(q[0, :, h], kd[0, :, h], vd[0, :, h], D ** -0.5, False)
             assert_out(out8[0, :, h], ro, f"decode e4m3 Sq={sq} head {h}")
             assert_lse(lse8[0, h], rl, f"decode e4m3 Sq={sq} head {h}")
+
+
+def test_decode_step_of_a_batch_with_ragged_caches():
+    """64 sequences with 1024 to 4096 cached keys each, one new token per sequence, 32 heads (a packed batch through
+    flash_fwd_varlen: the kernel that streams K and V): every head of eight sequences against the fp32 reference on the
+    GPU, the rows of two (sequence, head) pairs against the fp64 oracle, bf16 and e4m3 caches."""
+    import random
+    rng = random.Random(11)
+    nseq, H, D = 64, 32, 128
+    lens_k = [rng.randrange(1024, 4097) for _ in range(nseq)]
+    Tk = sum(lens_k)
+    (q,) = config_qkv((1, nseq, H, D), 9, n=1)
+    k, v = config_qkv((1, Tk, H, D), 10, n=2)
+    cu_q = torch.arange(nseq + 1, dtype=torch.int32, device=DEV)
+    starts = [0]
+    for n in lens_k:
+        starts.append(starts[-1] + n)
+    cu_k = torch.tensor(starts, dtype=torch.int32, device=DEV)
+    out, lse = ops.flash_fwd_varlen(q[0], k[0], v[0], cu_q, cu_k, 1, max(lens_k), None, False)
+    k8, ksc = ops.quantize_fp8_per_head(k.float())
+    v8, vsc = ops.quantize_fp8_per_head(v.float())
+    out8, lse8 = ops.flash_fwd_varlen(q[0], k8[0], v8[0], cu_q, cu_k, 1, max(lens_k), None, False,
+                                      k_scale=ksc.expand(nseq, H).contiguous(), v_scale=vsc.expand(nseq, H).contiguous())
+    kd, vd = k8.float() * ksc[:, None, :, None], v8.float() * vsc[:, None, :, None]
+    for b in list(range(0, nseq, 9)) + [nseq - 1]:
+        ks = slice(starts[b], starts[b + 1])
+        for h in range(H):
+            ro, rl = ref_head(q[0, b:b + 1, h], k[0, ks, h], v[0, ks, h], D ** -0.5, False)
+            assert_out(out[b:b + 1, h], ro, f"sequence {b} head {h}")
+            assert_lse(lse[h, b:b + 1], rl, f"sequence {b} head {h}")
+            ro, rl = ref_head(q[0, b:b + 1, h], kd[0, ks, h], vd[0, ks, h], D ** -0.5, False)
+            assert_out(out8[b:b + 1, h], ro, f"e4m3 sequence {b} head {h}")
+            assert_lse(lse8[h, b:b + 1], rl, f"e4m3 sequence {b} head {h}")
+    for b, h in ((0, 0), (nseq - 1, H - 1)):
+        ks = slice(starts[b], starts[b + 1])
+        spot_check_rows(out[b:b + 1, h], lse[h, b:b + 1], q[0, b:b + 1, h], k[0, ks, h], v[0, ks, h], D ** -0.5, False,
+                        f"sequence {b} head {h}", n_rows=1)
+
