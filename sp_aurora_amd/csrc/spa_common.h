@@ -227,6 +227,13 @@ static __device__ __forceinline__ void load_to_lds_b128(u32x4 rsrc, unsigned vof
                : "s"(lds_addr), "v"(voffset), "s"(rsrc)
                : "memory");
 }
+// The same with the non-temporal hint: for tiles that no other workgroup reads.
+static __device__ __forceinline__ void load_to_lds_b128_nt(u32x4 rsrc, unsigned voffset, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen nt lds"
+               :
+               : "s"(lds_addr), "v"(voffset), "s"(rsrc)
+               : "memory");
+}
 // The same for 4 bytes per lane: LDS at lds_addr + 4 * lane.
 static __device__ __forceinline__ void load_to_lds_b32(u32x4 rsrc, unsigned voffset, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds"
